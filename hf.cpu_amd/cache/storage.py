@@ -1,0 +1,57 @@
+"""The device memory behind the cache manager's books."""
+from dataclasses import dataclass
+
+import torch
+
+
+@dataclass
+class PagedView:
+    """What a mixer sees of its cache: row ``page * page_tokens + offset`` of ``k`` and
+    ``v`` belongs to one token; ``group`` names the block table to use."""
+    group: int
+    k: torch.Tensor            # [n_pages * page_tokens, k_width]
+    v: torch.Tensor            # [n_pages * page_tokens, v_width]
+    page_tokens: int
+    window: int
+
+
+@dataclass
+class StateView:
+    """Per-request state of fixed size: row ``slot`` of ``state`` ([n_slots, n_floats], fp32)."""
+    state: torch.Tensor
+
+
+class CacheStorage:
+    """Key/value rows for every schedule entry that stores, a block table per group
+    ([n_slots, max_blocks] int32, row = the request's slot), and the state rows."""
+
+    def __init__(self, manager, dtype, device):
+        self.manager = manager
+        self.views = [None] * len(manager.entry_group)
+        rows = None
+        for g, pool in zip(manager.groups, manager.pools):
+            rows = pool.n_pages * manager.page_tokens
+            for e in g.entries:
+                self.views[e] = PagedView(g.index,
+                                          torch.empty((rows, g.k_width), dtype=dtype, device=device),
+                                          torch.empty((rows, g.v_width), dtype=dtype, device=device),
+                                          manager.page_tokens, g.window)
+        for e, n_floats in manager.state_entries.items():
+            self.views[e] = StateView(torch.zeros((manager.n_slots, n_floats), dtype=torch.float32, device=device))
+        self.block_tables = [torch.zeros((manager.n_slots, manager.max_blocks), dtype=torch.int32, device=device)
+                             for _ in manager.groups]
+
+    def clear_slot(self, slot):
+        """State starts from zero for a newly admitted request."""
+        for v in self.views:
+            if isinstance(v, StateView):
+                v.state[slot].zero_()
+
+    def nbytes(self):
+        n = 0
+        for v in self.views:
+            if isinstance(v, PagedView):
+                n += v.k.numel() * v.k.element_size() + v.v.numel() * v.v.element_size()
+            elif isinstance(v, StateView):
+                n += v.state.numel() * 4
+        return n

@@ -1,0 +1,62 @@
+// The C interface of the kernel library. Pointers are device pointers unless named
+// host; sizes are in elements; `dtype` is HFA_F32 (0) or HFA_BF16 (1). Every function
+// returns 0 on success; otherwise hfa_last_error() describes what was refused.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+const char* hfa_last_error(void);
+int hfa_version(void);
+
+// x[t, :] = table[tokens[t], :] as fp32.  (reference: src/model.c:566-571)
+int hfa_embed(const void* table, int table_dtype, const int* tokens, float* x, int n_tokens, int width,
+              int vocab, hipStream_t stream);
+
+// out[r, :] = x[rows ? rows[r] : r, :] * rsqrt(mean(x^2) + eps) * w.  (src/mathx.c:65-75)
+int hfa_rmsnorm(const float* x, const float* w, void* out, int out_dtype, const int* rows, int n_rows,
+                int width, float eps, hipStream_t stream);
+
+// out[m, n] (+)= sum_k a[m, k] * w[n, k] + bias[n].  a: [M, K] row stride lda; w: [N, K] row
+// stride ldw; out row stride ldo. `accumulate` adds into fp32 `out` (the residual sum).
+// (src/model.c:408-424)
+int hfa_gemm(const void* a, int a_dtype, int lda, const void* w, int w_dtype, int ldw, const float* bias,
+             void* out, int out_dtype, int ldo, int accumulate, int M, int N, int K, hipStream_t stream);
+
+// Rotary position encoding on the q (and k) heads inside qkv rows [q | k | v], split-half
+// pairing, and the store of k (rotated) and v into cache rows slot_map[t] (src/model.c:468-493,
+// 587-600). rot_dim 0: no rotation. n_kv_heads 0: the rows hold q only, nothing is stored.
+int hfa_rope_store(void* qkv, int dtype, int ld, const int* positions, const float* inv_freq, int rot_dim,
+                   int n_heads, int n_kv_heads, int head_dim, void* k_cache, void* v_cache,
+                   const int* slot_map, int n_tokens, hipStream_t stream);
+
+// Softmax attention of each token's query heads over its request's cached keys and values
+// (src/model.c:499-528). Key j of the request in slot s lies in cache row
+// block_table[s, j / page_tokens] * page_tokens + j % page_tokens. A key is visible to the
+// query at position p iff j <= p and (window == 0 or p - j < window).
+int hfa_paged_attention(const void* q, int dtype, int ldq, const void* k_cache, const void* v_cache,
+                        int kv_width, const int* block_table, int max_blocks, const int* token_slot,
+                        const int* positions, void* out, int ldo, int n_tokens, int n_heads,
+                        int n_kv_heads, int head_dim, int page_tokens, int window, float scale,
+                        hipStream_t stream);
+
+// out[t, i] = silu(gate_up[t, i]) * gate_up[t, width + i].  (src/model.c:532-538)
+int hfa_swiglu(const void* gate_up, void* out, int dtype, int n_tokens, int width, hipStream_t stream);
+
+// dst[idx[i]] = val[i]
+int hfa_scatter_i32(int* dst, const int* idx, const int* val, int n, hipStream_t stream);
+
+// out[r] = first index of the maximum of logits[r, :].  (src/sample.c:72-77)
+int hfa_argmax(const float* logits, int ld, int* out, int n_rows, int vocab, hipStream_t stream);
+
+// The k best of each row in the order (logit descending, id ascending) (src/sample.c:59-64),
+// and stats[r] = {max, log(sum(exp(l - max)))} (src/sample.c:25-33). k <= 1024.
+int hfa_topk(const float* logits, int ld, int* ids, float* vals, float* stats, int n_rows, int vocab, int k,
+             hipStream_t stream);
+
+#ifdef __cplusplus
+}
+#endif

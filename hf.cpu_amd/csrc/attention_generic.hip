@@ -1,0 +1,145 @@
+// Paged softmax attention, plain form: one wave per (token, query head), for any mix of
+// prompt portions and decoded tokens, any head count and grouping, head_dim up to 256,
+// with or without a window, fp32 or bf16 cache. Scores, softmax and the weighted sum are
+// fp32; keys are visited in tiles of 64 aligned to absolute positions, in ascending order,
+// so a token's result depends on its request's cache alone, never on the rest of the batch.
+#include "api.h"
+#include "common.h"
+
+#define ATT_MAX_D 256
+
+template <typename T> struct Vec8;
+template <> struct Vec8<bf16> { uint4 v; };
+
+__device__ __forceinline__ float dot_row(const float* __restrict__ q_s, const bf16* __restrict__ kp, int D) {
+    float dot = 0.f;
+    if ((D & 7) == 0) {
+        for (int d = 0; d < D; d += 8) {
+            const uint4 u = *reinterpret_cast<const uint4*>(kp + d);
+            const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                dot = fmaf(q_s[d + 2 * i], __uint_as_float(w[i] << 16), dot);
+                dot = fmaf(q_s[d + 2 * i + 1], __uint_as_float(w[i] & 0xffff0000u), dot);
+            }
+        }
+    } else {
+        for (int d = 0; d < D; d++) dot = fmaf(q_s[d], to_f32(kp[d]), dot);
+    }
+    return dot;
+}
+__device__ __forceinline__ float dot_row(const float* __restrict__ q_s, const float* __restrict__ kp, int D) {
+    float dot = 0.f;
+    if ((D & 3) == 0) {
+        for (int d = 0; d < D; d += 4) {
+            const float4 u = *reinterpret_cast<const float4*>(kp + d);
+            dot = fmaf(q_s[d], u.x, dot);
+            dot = fmaf(q_s[d + 1], u.y, dot);
+            dot = fmaf(q_s[d + 2], u.z, dot);
+            dot = fmaf(q_s[d + 3], u.w, dot);
+        }
+    } else {
+        for (int d = 0; d < D; d++) dot = fmaf(q_s[d], kp[d], dot);
+    }
+    return dot;
+}
+
+template <typename T>
+__global__ __launch_bounds__(WAVE) void attn_generic_kernel(
+    const T* __restrict__ q, int ldq, const T* __restrict__ kc, const T* __restrict__ vc, int kvw,
+    const int* __restrict__ block_table, int max_blocks, const int* __restrict__ token_slot,
+    const int* __restrict__ positions, T* __restrict__ out, int ldo, int H, int G, int D, int page_tokens,
+    int window, float scale) {
+    __shared__ float q_s[ATT_MAX_D];
+    __shared__ float p_s[WAVE];
+    __shared__ int row_s[WAVE];
+    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    const int kvh = h / (H / G);
+    const int pos = positions[t];
+    const int* bt = block_table + (size_t)token_slot[t] * max_blocks;
+    for (int d = lane; d < D; d += WAVE) q_s[d] = to_f32(q[(size_t)t * ldq + h * D + d]);
+    __syncthreads();
+    const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+    float m = -INFINITY, l = 0.f;
+    float acc[ATT_MAX_D / WAVE];
+#pragma unroll
+    for (int i = 0; i < ATT_MAX_D / WAVE; i++) acc[i] = 0.f;
+
+    for (int j0 = (lo / WAVE) * WAVE; j0 <= pos; j0 += WAVE) {
+        const int j = j0 + lane;
+        const bool valid = j >= lo && j <= pos;
+        float s = -INFINITY;
+        int row = 0;
+        if (valid) {
+            row = bt[j / page_tokens] * page_tokens + j % page_tokens;
+            s = dot_row(q_s, kc + (size_t)row * kvw + kvh * D, D) * scale;
+        }
+        // every tile holds at least one visible key, so the maximum is finite
+        const float mn = fmaxf(m, wave_max(s));
+        const float corr = expf(m - mn);
+        const float p = valid ? expf(s - mn) : 0.f;
+        l = l * corr + wave_sum(p);
+        m = mn;
+        p_s[lane] = p;
+        row_s[lane] = row;
+        __syncthreads();
+        const int first = lo > j0 ? lo - j0 : 0;
+        const int last = pos - j0 < WAVE - 1 ? pos - j0 : WAVE - 1;
+#pragma unroll
+        for (int i = 0; i < ATT_MAX_D / WAVE; i++) acc[i] *= corr;
+        for (int jj = first; jj <= last; jj++) {
+            const float pj = p_s[jj];
+            const T* vp = vc + (size_t)row_s[jj] * kvw + kvh * D;
+#pragma unroll
+            for (int i = 0; i < ATT_MAX_D / WAVE; i++) {
+                const int d = lane + WAVE * i;
+                if (d < D) acc[i] = fmaf(pj, to_f32(vp[d]), acc[i]);
+            }
+        }
+        __syncthreads();
+    }
+    const float inv = 1.0f / l;
+#pragma unroll
+    for (int i = 0; i < ATT_MAX_D / WAVE; i++) {
+        const int d = lane + WAVE * i;
+        if (d < D) out[(size_t)t * ldo + h * D + d] = from_f32<T>(acc[i] * inv);
+    }
+}
+
+int attn_generic_launch(const void* q, int dtype, int ldq, const void* k_cache, const void* v_cache, int kv_width,
+                        const int* block_table, int max_blocks, const int* token_slot, const int* positions,
+                        void* out, int ldo, int n_tokens, int n_heads, int n_kv_heads, int head_dim,
+                        int page_tokens, int window, float scale, hipStream_t stream) {
+    HFA_REQUIRE(head_dim <= ATT_MAX_D, "paged_attention: head_dim %d exceeds the kernel's limit %d", head_dim,
+                ATT_MAX_D);
+    HFA_REQUIRE(n_heads <= 65535, "paged_attention: %d heads exceed the grid", n_heads);
+    dim3 grid(n_tokens, n_heads);
+    if (dtype == HFA_F32)
+        attn_generic_kernel<float><<<grid, WAVE, 0, stream>>>(
+            (const float*)q, ldq, (const float*)k_cache, (const float*)v_cache, kv_width, block_table, max_blocks,
+            token_slot, positions, (float*)out, ldo, n_heads, n_kv_heads, head_dim, page_tokens, window, scale);
+    else
+        attn_generic_kernel<bf16><<<grid, WAVE, 0, stream>>>(
+            (const bf16*)q, ldq, (const bf16*)k_cache, (const bf16*)v_cache, kv_width, block_table, max_blocks,
+            token_slot, positions, (bf16*)out, ldo, n_heads, n_kv_heads, head_dim, page_tokens, window, scale);
+    HFA_LAUNCH_CHECK("paged_attention");
+    return 0;
+}
+
+extern "C" int hfa_paged_attention(const void* q, int dtype, int ldq, const void* k_cache, const void* v_cache,
+                                   int kv_width, const int* block_table, int max_blocks, const int* token_slot,
+                                   const int* positions, void* out, int ldo, int n_tokens, int n_heads,
+                                   int n_kv_heads, int head_dim, int page_tokens, int window, float scale,
+                                   hipStream_t stream) {
+    HFA_REQUIRE(n_tokens > 0 && n_heads > 0 && n_kv_heads > 0 && head_dim > 0 && page_tokens > 0 && max_blocks > 0,
+                "paged_attention: bad sizes");
+    HFA_REQUIRE(n_heads % n_kv_heads == 0, "paged_attention: %d heads are not a multiple of %d key/value heads",
+                n_heads, n_kv_heads);
+    HFA_REQUIRE(kv_width >= n_kv_heads * head_dim && ldq >= n_heads * head_dim && ldo >= n_heads * head_dim,
+                "paged_attention: a row stride is smaller than its row");
+    HFA_REQUIRE(window >= 0, "paged_attention: negative window");
+    HFA_REQUIRE(dtype == HFA_F32 || dtype == HFA_BF16, "paged_attention: unknown dtype %d", dtype);
+    return attn_generic_launch(q, dtype, ldq, k_cache, v_cache, kv_width, block_table, max_blocks, token_slot,
+                               positions, out, ldo, n_tokens, n_heads, n_kv_heads, head_dim, page_tokens, window,
+                               scale, stream);
+}

@@ -1,0 +1,17 @@
+// The matrix-product variants behind hfa_gemm. Each takes the same arguments and returns
+// 0, or non-zero after hfa_set_error(). The dispatcher in gemm.hip picks one by dtype and shape.
+#pragma once
+#include <hip/hip_runtime.h>
+
+struct GemmArgs {
+    const void* a; int a_dtype; int lda;
+    const void* w; int w_dtype; int ldw;
+    const float* bias;
+    void* out; int out_dtype; int ldo;
+    int accumulate;
+    int M, N, K;
+    hipStream_t stream;
+};
+
+// Any dtype mix, any size: fp32 multiply-add over K in ascending order for every output.
+int gemm_generic_launch(const GemmArgs& g);

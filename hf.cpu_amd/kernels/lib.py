@@ -1,0 +1,51 @@
+"""Loading the kernel library and declaring its C interface (csrc/api.h) to ctypes.
+
+There is no fallback: if the library is missing it is built, and if it cannot be
+built or loaded the error is raised to the caller.
+"""
+import ctypes
+import threading
+from ctypes import c_char_p, c_float, c_int, c_void_p
+
+from . import build as _build
+
+_lock = threading.Lock()
+_lib = None
+
+P, I, F = c_void_p, c_int, c_float
+_SIGNATURES = {
+    "hfa_embed": [P, I, P, P, I, I, I, P],
+    "hfa_rmsnorm": [P, P, P, I, P, I, I, F, P],
+    "hfa_gemm": [P, I, I, P, I, I, P, P, I, I, I, I, I, I, P],
+    "hfa_rope_store": [P, I, I, P, P, I, I, I, I, P, P, P, I, P],
+    "hfa_paged_attention": [P, I, I, P, P, I, P, I, P, P, P, I, I, I, I, I, I, I, F, P],
+    "hfa_swiglu": [P, P, I, I, I, P],
+    "hfa_scatter_i32": [P, P, P, I, P],
+    "hfa_argmax": [P, I, P, I, I, P],
+    "hfa_topk": [P, I, P, P, P, I, I, I, P],
+}
+
+
+def library():
+    """The loaded library (built first if there is none, or if its sources changed)."""
+    global _lib
+    with _lock:
+        if _lib is None:
+            path, current = _build.find_library()
+            if path is None or not current:
+                path = _build.build()
+            lib = ctypes.CDLL(path)
+            lib.hfa_last_error.restype = c_char_p
+            lib.hfa_last_error.argtypes = []
+            lib.hfa_version.restype = c_int
+            for name, args in _SIGNATURES.items():
+                fn = getattr(lib, name)
+                fn.argtypes = args
+                fn.restype = c_int
+            lib.path = path
+            _lib = lib
+        return _lib
+
+
+def last_error():
+    return library().hfa_last_error().decode("utf-8", "replace")

@@ -1,0 +1,172 @@
+"""The kernels as methods on tensors.
+
+``Ops`` belongs to one device and one compute dtype. Every method checks shapes,
+dtypes and layout on the host, hands raw pointers to the library on the current
+stream, and raises EngineError if the library refuses the call. Nothing here
+computes with a library routine or on the CPU.
+"""
+import torch
+
+from ..status import EINVAL, ENOTSUP, EngineError, fail
+from .lib import last_error, library
+
+F32, BF16 = 0, 1
+_CODE = {torch.float32: F32, torch.bfloat16: BF16}
+
+
+def _code(t):
+    if t.dtype not in _CODE:
+        fail(EINVAL, f"tensor dtype {t.dtype} is neither float32 nor bfloat16")
+    return _CODE[t.dtype]
+
+
+def _rows(t, what):
+    """A 2-D tensor whose rows are contiguous; returns its row stride."""
+    if t.dim() != 2 or t.stride(1) != 1:
+        fail(EINVAL, f"{what}: expected a matrix with contiguous rows, got shape {tuple(t.shape)} "
+                     f"strides {t.stride()}")
+    return t.stride(0) if t.shape[0] > 1 else max(t.stride(0), t.shape[1])
+
+
+def _ints(t, what, n=None):
+    if t.dtype != torch.int32 or not t.is_contiguous() or (n is not None and t.numel() < n):
+        fail(EINVAL, f"{what}: expected a contiguous int32 tensor of at least {n} elements")
+    return t.data_ptr()
+
+
+class Ops:
+    def __init__(self, act_dtype=torch.bfloat16, device="cuda:0"):
+        if not torch.cuda.is_available():
+            fail(ENOTSUP, "no GPU is visible: the engine runs on gfx950 only and has no CPU path")
+        if act_dtype not in _CODE:
+            fail(EINVAL, f"compute dtype {act_dtype} is neither float32 nor bfloat16")
+        self.device = torch.device(device)
+        self.act_dtype = act_dtype
+        self.lib = library()
+        self._scratch = {}
+
+    # ---- plumbing ----------------------------------------------------------
+    def _stream(self):
+        return torch.cuda.current_stream(self.device).cuda_stream
+
+    def _check(self, rc):
+        if rc != 0:
+            raise EngineError(EINVAL if rc == 1 else ENOTSUP, last_error())
+
+    def scratch(self, name, shape, dtype):
+        """A named work buffer that is reused from step to step; its contents are
+        undefined on return. The same name always aliases the same memory."""
+        n = 1
+        for s in shape:
+            n *= int(s)
+        nbytes = max(n, 1) * torch.empty((), dtype=dtype).element_size()
+        buf = self._scratch.get(name)
+        if buf is None or buf.numel() < nbytes:
+            buf = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=self.device)
+            self._scratch[name] = buf
+        return buf[:nbytes].view(dtype).view(*shape)
+
+    # ---- kernels -----------------------------------------------------------
+    def embed(self, table, tokens, out_x):
+        T = out_x.shape[0]
+        if out_x.dtype != torch.float32 or not out_x.is_contiguous() or not table.is_contiguous() \
+                or table.shape[1] != out_x.shape[1]:
+            fail(EINVAL, "embed: the output must be contiguous fp32 with the table's width")
+        self._check(self.lib.hfa_embed(table.data_ptr(), _code(table), _ints(tokens, "embed tokens", T),
+                                       out_x.data_ptr(), T, table.shape[1], table.shape[0], self._stream()))
+
+    def rmsnorm(self, x, weight, eps, out, rows=None):
+        R = out.shape[0]
+        E = x.shape[1]
+        if x.dtype != torch.float32 or weight.dtype != torch.float32 or not x.is_contiguous() \
+                or not out.is_contiguous() or out.shape[1] != E or weight.numel() != E:
+            fail(EINVAL, "rmsnorm: x and weight must be fp32, contiguous, and of one width with out")
+        if rows is None and R != x.shape[0]:
+            fail(EINVAL, "rmsnorm: without row indices the output must have x's rows")
+        self._check(self.lib.hfa_rmsnorm(x.data_ptr(), weight.data_ptr(), out.data_ptr(), _code(out),
+                                         None if rows is None else _ints(rows, "rmsnorm rows", R),
+                                         R, E, float(eps), self._stream()))
+
+    def gemm(self, a, w, out, bias=None, accumulate=False):
+        """out (+)= a @ w.T + bias, fp32 accumulation."""
+        lda, ldw, ldo = _rows(a, "gemm a"), _rows(w, "gemm w"), _rows(out, "gemm out")
+        M, K = a.shape
+        N = w.shape[0]
+        if w.shape[1] != K or tuple(out.shape) != (M, N):
+            fail(EINVAL, f"gemm: shapes a{tuple(a.shape)} w{tuple(w.shape)} out{tuple(out.shape)} do not fit")
+        if bias is not None and (bias.dtype != torch.float32 or bias.numel() != N or not bias.is_contiguous()):
+            fail(EINVAL, "gemm: the bias must be contiguous fp32 with one value per output column")
+        self._check(self.lib.hfa_gemm(a.data_ptr(), _code(a), lda, w.data_ptr(), _code(w), ldw,
+                                      None if bias is None else bias.data_ptr(), out.data_ptr(), _code(out), ldo,
+                                      1 if accumulate else 0, M, N, K, self._stream()))
+
+    def rope_store(self, qkv, positions, inv_freq, rot_dim, n_heads, n_kv_heads, head_dim, cache, slot_map):
+        """Rotates q (and k) inside ``qkv`` and, if ``slot_map`` is given, stores k and v
+        rows into ``cache.k`` / ``cache.v`` at the rows it names."""
+        ld = _rows(qkv, "rope_store qkv")
+        T = qkv.shape[0]
+        if qkv.shape[1] < (n_heads + 2 * n_kv_heads) * head_dim:
+            fail(EINVAL, "rope_store: the rows are narrower than the heads they should hold")
+        k_ptr = v_ptr = None
+        if n_kv_heads and slot_map is not None:
+            width = n_kv_heads * head_dim
+            for c in (cache.k, cache.v):
+                if c.dtype != qkv.dtype or c.dim() != 2 or c.shape[1] != width or not c.is_contiguous():
+                    fail(EINVAL, "rope_store: the cache must have the activations' dtype and one row of "
+                                 f"{width} values per token")
+            k_ptr, v_ptr = cache.k.data_ptr(), cache.v.data_ptr()
+        self._check(self.lib.hfa_rope_store(
+            qkv.data_ptr(), _code(qkv), ld, None if positions is None else _ints(positions, "positions", T),
+            None if inv_freq is None else inv_freq.data_ptr(), rot_dim, n_heads, n_kv_heads, head_dim,
+            k_ptr, v_ptr, None if slot_map is None else _ints(slot_map, "slot_map", T), T, self._stream()))
+
+    def paged_attention(self, q, n_heads, n_kv_heads, head_dim, cache, step, window, scale, out):
+        """Attention of the first ``n_heads * head_dim`` columns of ``q`` over ``cache``."""
+        T = q.shape[0]
+        ldq, ldo = _rows(q, "attention q"), _rows(out, "attention out")
+        g = step.group(cache.group)
+        if cache.k.dtype != q.dtype or out.dtype != q.dtype:
+            fail(EINVAL, "paged_attention: queries, cache and output must share a dtype")
+        if cache.k.shape[1] != n_kv_heads * head_dim:
+            fail(EINVAL, "paged_attention: the cache rows do not hold n_kv_heads * head_dim values")
+        self._check(self.lib.hfa_paged_attention(
+            q.data_ptr(), _code(q), ldq, cache.k.data_ptr(), cache.v.data_ptr(), cache.k.shape[1],
+            g.block_table.data_ptr(), g.block_table.shape[1], _ints(step.token_slot, "token_slot", T),
+            _ints(step.positions, "positions", T), out.data_ptr(), ldo, T, n_heads, n_kv_heads, head_dim,
+            cache.page_tokens, int(window), float(scale), self._stream()))
+
+    def swiglu(self, gate_up, out):
+        T, F2 = gate_up.shape
+        if not gate_up.is_contiguous() or not out.is_contiguous() or tuple(out.shape) != (T, F2 // 2) \
+                or out.dtype != gate_up.dtype or F2 % 2:
+            fail(EINVAL, "swiglu: expected contiguous [T, 2F] in and [T, F] out of one dtype")
+        self._check(self.lib.hfa_swiglu(gate_up.data_ptr(), out.data_ptr(), _code(out), T, F2 // 2, self._stream()))
+
+    def scatter_i32(self, dst, idx, val):
+        n = idx.numel()
+        if n:
+            self._check(self.lib.hfa_scatter_i32(_ints(dst, "scatter dst"), _ints(idx, "scatter idx"),
+                                                 _ints(val, "scatter val", n), n, self._stream()))
+
+    def argmax(self, logits, out=None):
+        R, V = logits.shape
+        if logits.dtype != torch.float32:
+            fail(EINVAL, "argmax: logits must be fp32")
+        if out is None:
+            out = torch.empty(R, dtype=torch.int32, device=logits.device)
+        self._check(self.lib.hfa_argmax(logits.data_ptr(), _rows(logits, "argmax logits"), _ints(out, "argmax out", R),
+                                        R, V, self._stream()))
+        return out
+
+    def topk(self, logits, k, want_stats=True):
+        """(ids [R, k] int32, values [R, k] fp32, stats [R, 2] fp32 = max and log-sum-exp
+        above the max), candidates in the order (logit descending, id ascending)."""
+        R, V = logits.shape
+        if logits.dtype != torch.float32:
+            fail(EINVAL, "topk: logits must be fp32")
+        ids = torch.empty((R, max(k, 1)), dtype=torch.int32, device=logits.device)
+        vals = torch.empty((R, max(k, 1)), dtype=torch.float32, device=logits.device)
+        stats = torch.empty((R, 2), dtype=torch.float32, device=logits.device) if want_stats else None
+        self._check(self.lib.hfa_topk(logits.data_ptr(), _rows(logits, "topk logits"), ids.data_ptr(), vals.data_ptr(),
+                                      None if stats is None else stats.data_ptr(), R, V, k, self._stream()))
+        return ids[:, :k], vals[:, :k], stats

@@ -1,0 +1,135 @@
+"""A model: the parts a plan names, built, with their tensors bound.
+
+``Model.from_dir`` is the one way in for a model folder: config.json names the
+architecture, the registry gives its configuration class and plan function, the
+plan gives the parts, the parts declare the tensors the loader must find.
+"""
+from dataclasses import dataclass
+
+import torch
+
+from .config import config_from_dict, read_config
+from .parts.base import FixedState, PagedKV
+from .registry import architecture, make_part
+from .status import EINVAL, fail
+from .weights.loader import load_tensors
+from .weights.random_init import random_device_tensors
+
+COMPUTE_DTYPES = {"float32": torch.float32, "fp32": torch.float32,
+                  "bfloat16": torch.bfloat16, "bf16": torch.bfloat16}
+
+
+def compute_dtype(name):
+    if isinstance(name, torch.dtype):
+        return name
+    if name not in COMPUTE_DTYPES:
+        fail(EINVAL, f"dtype '{name}' is not one of {', '.join(sorted(COMPUTE_DTYPES))}")
+    return COMPUTE_DTYPES[name]
+
+
+@dataclass
+class Layer:
+    label: str
+    block: object
+    norm1: object
+    mixer: object
+    norm2: object
+    feed_forward: object
+
+    def parts(self):
+        return [self.block, self.norm1, self.mixer, self.norm2, self.feed_forward]
+
+
+class Model:
+    def __init__(self, plan, config=None):
+        plan.check()
+        self.plan = plan
+        self.config = config
+        self.embedding = make_part("embedding", plan.embedding)
+        self.layers = [Layer(lp.label, make_part("block", lp.block), make_part("norm", lp.norm1),
+                             make_part("mixer", lp.mixer), make_part("norm", lp.norm2),
+                             make_part("feed_forward", lp.feed_forward)) for lp in plan.layers]
+        self.final_norm = make_part("norm", plan.final_norm)
+        self.head = make_part("head", plan.head)
+        self.schedule = plan.schedule
+        self.hidden_size = plan.hidden_size
+        self.vocab_size = plan.vocab_size
+        self.dtype = None
+        self.device = None
+
+    # ---- construction --------------------------------------------------
+    @classmethod
+    def from_config(cls, config):
+        """Parts without tensors (enough to list them or to plan a cache)."""
+        _, plan_fn = architecture(config.architecture)
+        return cls(plan_fn(config), config)
+
+    @classmethod
+    def from_dir(cls, model_dir, dtype, ops):
+        model = cls.from_config(read_config(model_dir))
+        dt = compute_dtype(dtype)
+        model._bind(load_tensors(model_dir, model.param_specs(), dt, ops.device), dt, ops)
+        return model
+
+    @classmethod
+    def from_random(cls, config, seed, dtype, ops):
+        """Random weights made on the device, without a file."""
+        if isinstance(config, dict):
+            config = config_from_dict(config)
+        model = cls.from_config(config)
+        dt = compute_dtype(dtype)
+        model._bind(random_device_tensors(model.param_specs(), seed, dt, ops.device), dt, ops)
+        return model
+
+    def _all_parts(self):
+        parts = [self.embedding]
+        for layer in self.layers:
+            parts.extend(layer.parts())
+        return parts + [self.final_norm, self.head]
+
+    def param_specs(self):
+        specs, seen = [], set()
+        for p in self._all_parts():
+            for s in p.all_param_specs():
+                if s.name in seen:
+                    raise ValueError(f"two parts declare the tensor '{s.name}'")
+                seen.add(s.name)
+                specs.append(s)
+        return specs
+
+    def _bind(self, params, dtype, ops):
+        self.dtype, self.device = dtype, ops.device
+        for p in self._all_parts():
+            p.bind_all(params, ops)
+
+    # ---- what the cache manager needs to know -----------------------------
+    def cache_needs(self):
+        """For each schedule entry: PagedKV, FixedState, or None (no cache of its own)."""
+        needs = []
+        for e in self.schedule:
+            mixer = self.layers[e.layer].mixer
+            need = mixer.cache_need() if e.cache_of is None and hasattr(mixer, "cache_need") else None
+            if need is not None and not isinstance(need, (PagedKV, FixedState)):
+                raise TypeError(f"{type(mixer).__name__}.cache_need() returned {need!r}")
+            needs.append(need)
+        return needs
+
+    # ---- the forward pass of one step ----------------------------------------
+    def forward(self, ops, step, caches, logits_out):
+        """Runs ``step``'s tokens through the schedule. ``caches[i]`` is the cache view
+        of schedule entry ``i`` (None if it needs none). Writes fp32 logits for
+        ``step.logit_rows`` into ``logits_out`` ([R, V]; R may be 0)."""
+        T = step.n_tokens
+        x = ops.scratch("residual", (T, self.hidden_size), torch.float32)
+        self.embedding.forward(ops, step, x)
+        for i, e in enumerate(self.schedule):
+            layer = self.layers[e.layer]
+            own = e.cache_of is None
+            cache = caches[i if own else e.cache_of]
+            layer.block.forward(ops, step, x, layer.norm1, layer.mixer, layer.norm2, layer.feed_forward,
+                                cache, write_cache=own)
+        R = step.n_logit_rows
+        if R:
+            h = ops.scratch("head_in", (R, self.hidden_size), ops.act_dtype)
+            self.final_norm.forward(ops, x, h, rows=step.logit_rows)      # src/model.c:629-636
+            self.head.forward(ops, h, logits_out)

@@ -1,0 +1,77 @@
+"""Softmax attention over a paged key/value cache, with grouped heads and an
+optional window."""
+import math
+
+import torch
+
+from ..registry import make_part, register_part
+from ..status import EINVAL, fail
+from .base import PagedKV, ParamSpec, Part
+
+
+@register_part("mixer", "attention")
+class Attention(Part):
+    """``q = Wq h + bq`` etc. (src/model.c:581-585); position encoding on q and k;
+    for query head ``h`` the key/value head is ``h / (heads / kv_heads)``; scores
+    ``dot(q, k) * scale`` over the visible keys, softmax in fp32, weighted sum of
+    values (src/model.c:499-528); ``x += Wo att`` (src/model.c:606-609).
+
+    A key at ``pk`` is visible to a query at ``pq`` iff ``0 <= pq - pk`` and, when
+    ``window > 0``, ``pq - pk < window``.
+    """
+
+    def __init__(self, hidden_size, n_heads, n_kv_heads, head_dim, qkv_bias, window, position,
+                 scale=None, out_bias=False, prefix=""):
+        super().__init__(prefix)
+        if n_heads % n_kv_heads:
+            fail(EINVAL, f"attention: {n_heads} heads are not a multiple of {n_kv_heads} key/value heads")
+        self.E, self.H, self.G, self.D = hidden_size, n_heads, n_kv_heads, head_dim
+        self.QD, self.KD = n_heads * head_dim, n_kv_heads * head_dim
+        self.qkv_bias = bool(qkv_bias)
+        self.out_bias = bool(out_bias)
+        self.window = int(window)
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_dim)   # src/model.c:507
+        self.position = make_part("position", position)
+        self.w_qkv = self.b_qkv = self.w_o = self.b_o = None
+
+    def sub_parts(self):
+        return [self.position]
+
+    def param_specs(self):
+        p = self.prefix
+        specs = [ParamSpec(p + "q_proj.weight", (self.QD, self.E)),
+                 ParamSpec(p + "k_proj.weight", (self.KD, self.E)),
+                 ParamSpec(p + "v_proj.weight", (self.KD, self.E)),
+                 ParamSpec(p + "o_proj.weight", (self.E, self.QD))]
+        if self.qkv_bias:
+            specs += [ParamSpec(p + "q_proj.bias", (self.QD,), "vector"),
+                      ParamSpec(p + "k_proj.bias", (self.KD,), "vector"),
+                      ParamSpec(p + "v_proj.bias", (self.KD,), "vector")]
+        if self.out_bias:
+            specs.append(ParamSpec(p + "o_proj.bias", (self.E,), "vector"))
+        return specs
+
+    def cache_need(self):
+        return PagedKV(self.KD, self.KD, self.window)
+
+    def bind(self, params, ops):
+        p = self.prefix
+        # One matrix for the three projections that share an input: rows of q, then k, then v.
+        mats = [params[p + n + "_proj.weight"] for n in "qkv"]
+        dt = torch.float32 if any(m.dtype == torch.float32 for m in mats) else mats[0].dtype
+        self.w_qkv = torch.cat([m.to(dt) for m in mats], dim=0).contiguous()
+        if self.qkv_bias:
+            self.b_qkv = torch.cat([params[p + n + "_proj.bias"] for n in "qkv"]).contiguous()
+        self.w_o = params[p + "o_proj.weight"]
+        if self.out_bias:
+            self.b_o = params[p + "o_proj.bias"]
+
+    def forward(self, ops, step, h, cache, x, write_cache=True):
+        T = h.shape[0]
+        width = self.QD + 2 * self.KD if write_cache else self.QD
+        qkv = ops.scratch("qkv", (T, width), ops.act_dtype)
+        ops.gemm(h, self.w_qkv[:width], qkv, bias=None if self.b_qkv is None else self.b_qkv[:width])
+        self.position.store(ops, step, qkv, self.H, self.G if write_cache else 0, cache, write_cache)
+        att = ops.scratch("att", (T, self.QD), ops.act_dtype)
+        ops.paged_attention(qkv, self.H, self.G, self.D, cache, step, self.window, self.scale, att)
+        ops.gemm(att, self.w_o, x, bias=self.b_o, accumulate=True)

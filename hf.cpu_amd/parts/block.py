@@ -1,0 +1,20 @@
+"""Arrangements of a layer's parts around the residual stream."""
+from ..registry import register_part
+from .base import Part
+
+
+@register_part("block", "prenorm")
+class PreNormBlock(Part):
+    """``x += mixer(norm1(x)); x += feed_forward(norm2(x))`` (src/model.c:580-623):
+    norms in front of each part, nothing after, the residual stream in fp32."""
+
+    def __init__(self, hidden_size, prefix=""):
+        super().__init__(prefix)
+        self.E = hidden_size
+
+    def forward(self, ops, step, x, norm1, mixer, norm2, feed_forward, cache, write_cache=True):
+        h = ops.scratch("normed", (x.shape[0], self.E), ops.act_dtype)
+        norm1.forward(ops, x, h)
+        mixer.forward(ops, step, h, cache, x, write_cache)
+        norm2.forward(ops, x, h)
+        feed_forward.forward(ops, step, h, x)

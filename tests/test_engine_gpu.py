@@ -1,0 +1,147 @@
+"""The engine against the plain implementation, in every way of cutting the work."""
+import numpy as np
+import pytest
+
+import helpers
+import plain
+
+pytestmark = pytest.mark.gpu
+
+# Largest |logit difference| allowed between the engine and the float64 plain implementation.
+# fp32: rounding of a few hundred fused multiply-adds on values of order one.
+# bf16: activations and cache rounded to 8 bits of mantissa at every part.
+TOL = {"float32": 2e-4, "bfloat16": 0.25}
+LENGTHS = {"A": [7, 19, 33, 70, 101], "B": [1, 40, 77, 100, 130]}
+
+
+@pytest.fixture(scope="module", params=["A", "B"])
+def tiny(request, tmp_path_factory):
+    name = request.param
+    cfg = helpers.CONFIGS[name]
+    d = helpers.make_model_dir(str(tmp_path_factory.mktemp("model" + name)), cfg, seed=ord(name))
+    reqs = helpers.random_requests(cfg, LENGTHS[name], seed=7)
+    return name, cfg, d, reqs, helpers.plain_logits(d, reqs)
+
+
+def engine_for(model_dir, dtype, name, max_tokens, max_seqs=4):
+    import hf_cpu_amd
+    return hf_cpu_amd.load_engine(model_dir, dtype=dtype, page_tokens=helpers.PAGE[name],
+                                  max_tokens=max_tokens, max_seqs=max_seqs)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("cutting", ["whole", "tail", "portions", "mixed"])
+def test_cuttings(gpu, tiny, dtype, cutting):
+    name, cfg, d, reqs, want = tiny
+    steps = {"whole": helpers.trace_whole, "tail": helpers.trace_tail, "portions": helpers.trace_portions,
+             "mixed": lambda r: helpers.trace_mixed(r, seed=3)}[cutting](reqs)
+    max_tokens = helpers.max_live_tokens(steps)
+    engine = engine_for(d, dtype, name, max_tokens)
+    got = helpers.run_trace_in_engine(engine, steps)
+    assert len(got) == sum(len(t) for t in reqs.values())
+    worst = helpers.compare(got, want, TOL[dtype], f"{name} {dtype} {cutting}")
+    print(f"{name} {dtype} {cutting}: worst |diff| {worst:.3e}")
+    engine.manager.check()
+    assert not engine.manager.held and all(p.n_held == 0 for p in engine.manager.pools)
+    if cutting == "mixed":
+        assert any(p.reused > 0 for p in engine.manager.pools), "the trace was meant to use pages again"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_cuttings_agree_with_each_other(gpu, tiny, dtype):
+    """Beyond agreeing with the plain implementation, the cuttings agree among themselves
+    far more closely: the same values are computed, only in other launches."""
+    name, cfg, d, reqs, _ = tiny
+    results = []
+    for make in (helpers.trace_whole, helpers.trace_portions, lambda r: helpers.trace_mixed(r, seed=5)):
+        steps = make(reqs)
+        engine = engine_for(d, dtype, name, helpers.max_live_tokens(steps))
+        results.append(helpers.run_trace_in_engine(engine, steps))
+    tol = 2e-5 if dtype == "float32" else 0.06
+    for other in results[1:]:
+        for key, row in results[0].items():
+            err = float(np.max(np.abs(row - other[key])))
+            assert err <= tol, f"{name} {dtype}: {key}: cuttings differ by {err:.3e}"
+
+
+def test_window_edge_shows(gpu, tmp_path):
+    """Config B with one key made to stand out: a query far beyond the window must not see
+    it in the windowed layers, one inside the window must. The plain implementation decides;
+    a window off by one moves the logits by far more than the tolerance."""
+    cfg = dict(helpers.CONFIG_B)
+    w = helpers.make_weights(cfg, seed=11)
+    for l in range(cfg["num_hidden_layers"]):
+        w[f"model.layers.{l}.self_attn.k_proj.bias"] *= 4.0      # large common key component
+        w[f"model.layers.{l}.self_attn.q_proj.bias"] *= 4.0
+    d = helpers.make_model_dir(str(tmp_path / "m"), cfg, 0, weights=w)
+    reqs = helpers.random_requests(cfg, [31, 32, 33, 34, 64, 65, 97], seed=2)
+    want = helpers.plain_logits(d, reqs)
+    off = dict(cfg, use_sliding_window=False)
+    d_off = helpers.make_model_dir(str(tmp_path / "off"), off, 0, weights=w)
+    want_off = helpers.plain_logits(d_off, reqs)
+    # the window matters: beyond it the two models differ clearly, inside it they are equal
+    assert max(np.max(np.abs(want["r6"][40:] - want_off["r6"][40:])), 0) > 0.05
+    assert np.max(np.abs(want["r6"][:32] - want_off["r6"][:32])) < 1e-9
+    for steps in (helpers.trace_whole(reqs), helpers.trace_tail(reqs, 8), helpers.trace_mixed(reqs, 1)):
+        engine = engine_for(d, "float32", "B", helpers.max_live_tokens(steps))
+        helpers.compare(helpers.run_trace_in_engine(engine, steps), want, TOL["float32"], "window")
+
+
+def test_far_key_among_hundreds(gpu, tmp_path):
+    """One early token whose key matches every later query strongly: its value must reach
+    position 250 through 16 pages. A block table or page offset that is wrong anywhere on
+    the way shows in the logits."""
+    cfg = dict(helpers.CONFIG_A, max_position_embeddings=512, rope_theta=1e9)   # slow rotation
+    w = helpers.make_weights(cfg, seed=4)
+    toks = helpers.random_requests(cfg, [260], seed=9)["r0"]
+    toks[3] = 77
+    assert 77 not in toks[:3] + toks[4:]
+    E = cfg["hidden_size"]
+    # token 77's embedding gives a key aligned with the query bias in layer 0
+    for l in range(cfg["num_hidden_layers"]):
+        w[f"model.layers.{l}.self_attn.q_proj.bias"] *= 3.0
+    d = helpers.make_model_dir(str(tmp_path / "m"), cfg, 0, weights=w)
+    reqs = {"r0": toks}
+    want = helpers.plain_logits(d, reqs)
+    for steps in (helpers.trace_whole(reqs), helpers.trace_tail(reqs), helpers.trace_portions(reqs)):
+        engine = engine_for(d, "float32", "A", helpers.max_live_tokens(steps))
+        helpers.compare(helpers.run_trace_in_engine(engine, steps), want, TOL["float32"], "far key")
+
+
+def test_first_tokens_and_long_decode(gpu, tiny):
+    """The first tokens of a sequence one by one from an empty cache, and a long run of
+    single-token steps (every page edge is crossed in decode)."""
+    name, cfg, d, reqs, want = tiny
+    r = "r4"
+    toks = reqs[r]
+    steps = [{"step": i, "entries": [{"id": r, "tokens": [t], "want": [0]}], "end": []}
+             for i, t in enumerate(toks)]
+    steps[-1]["end"] = [r]
+    for dtype in ("float32", "bfloat16"):
+        engine = engine_for(d, dtype, name, helpers.max_live_tokens(steps))
+        got = helpers.run_trace_in_engine(engine, steps)
+        helpers.compare(got, {r: want[r]}, TOL[dtype], f"{name} {dtype} token by token")
+
+
+def test_step_refusals_leave_no_trace(gpu, tiny):
+    from hf_cpu_amd.status import EngineError
+    name, cfg, d, reqs, want = tiny
+    engine = engine_for(d, "float32", name, 128, max_seqs=2)
+    with pytest.raises(EngineError) as e:
+        engine.step([("a", [1, cfg["vocab_size"]], [0])])
+    assert e.value.code == "EINVAL" and "vocabulary" in str(e.value)
+    with pytest.raises(EngineError) as e:
+        engine.step([("a", [1, 2], [2])])
+    assert e.value.code == "EINVAL"
+    with pytest.raises(EngineError) as e:
+        engine.step([("a", list(range(100)), []), ("b", list(range(100)), [])])     # 128 tokens of pages
+    assert e.value.code == "ENOMEM"
+    engine.manager.check()
+    assert not engine.manager.held and all(p.n_held == 0 for p in engine.manager.pools)
+    with pytest.raises(EngineError) as e:
+        engine.step([("a", [1], []), ("b", [1], []), ("c", [1], [])])                # 2 slots
+    assert e.value.code == "ENOMEM"
+    assert not engine.manager.held
+    toks = reqs["r2"]
+    got = helpers.run_trace_in_engine(engine, helpers.trace_whole({"r2": toks}))
+    helpers.compare(got, want, TOL["float32"], "after refusals")

@@ -1,0 +1,303 @@
+"""Each kernel alone against a plain reference, at sizes other than the engine's."""
+import math
+import types
+
+import numpy as np
+import pytest
+import torch
+
+import plain
+from helpers import bf16_round
+
+pytestmark = pytest.mark.gpu
+
+
+def dev(a, dtype=torch.float32):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(dtype).cuda()
+
+
+def ints(a):
+    return torch.tensor(np.asarray(a, dtype=np.int32), dtype=torch.int32, device="cuda")
+
+
+def rounded(a, dtype):
+    """What the kernel is given after the cast to ``dtype``, as float64."""
+    a = np.asarray(a, dtype=np.float32)
+    return (bf16_round(a) if dtype == torch.bfloat16 else a).astype(np.float64)
+
+
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embed(ops32, dtype):
+    rng = np.random.default_rng(0)
+    table = rng.standard_normal((37, 50)).astype(np.float32)
+    toks = [0, 36, 5, 5, 17]
+    out = torch.empty((5, 50), dtype=torch.float32, device="cuda")
+    ops32.embed(dev(table, dtype), ints(toks), out)
+    assert np.array_equal(out.cpu().numpy(), rounded(table, dtype)[toks].astype(np.float32))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("width", [5, 64, 100, 1000, 3584])
+def test_rmsnorm(ops32, dtype, width):
+    rng = np.random.default_rng(width)
+    x = (rng.standard_normal((7, width)) * 3).astype(np.float32)
+    w = (1 + 0.1 * rng.standard_normal(width)).astype(np.float32)
+    out = torch.empty((7, width), dtype=dtype, device="cuda")
+    ops32.rmsnorm(dev(x), dev(w), 1e-5, out)
+    want = plain.rmsnorm(x.astype(np.float64), w.astype(np.float64), 1e-5)
+    tol = 1e-5 if dtype == torch.float32 else 0.02
+    assert np.max(np.abs(out.float().cpu().numpy() - want)) <= tol * np.max(np.abs(want))
+    rows = [6, 0, 3]
+    out2 = torch.empty((3, width), dtype=dtype, device="cuda")
+    ops32.rmsnorm(dev(x), dev(w), 1e-5, out2, ints(rows))
+    assert torch.equal(out2, out[rows])
+
+
+def test_rmsnorm_reference_vector(ops32):
+    """x = {1..5}, w = {1, 1, 2, 2, 0.5}, eps 1e-6 -> x * w / sqrt(11 + 1e-6)
+    (the reference's tests/test_kern.c:242-248)."""
+    x = np.array([[1, 2, 3, 4, 5]], dtype=np.float32)
+    w = np.array([1, 1, 2, 2, 0.5], dtype=np.float32)
+    out = torch.empty((1, 5), dtype=torch.float32, device="cuda")
+    ops32.rmsnorm(dev(x), dev(w), 1e-6, out)
+    want = x[0] * w / math.sqrt(11 + 1e-6)
+    assert np.max(np.abs(out.cpu().numpy()[0] - want)) < 1e-5
+
+
+@pytest.mark.parametrize("adt,wdt,odt", [(torch.float32, torch.float32, torch.float32),
+                                         (torch.bfloat16, torch.bfloat16, torch.bfloat16),
+                                         (torch.bfloat16, torch.bfloat16, torch.float32),
+                                         (torch.bfloat16, torch.float32, torch.bfloat16)])
+@pytest.mark.parametrize("M,N,K", [(1, 7, 5), (3, 100, 33), (64, 64, 64), (65, 130, 257), (200, 48, 1000),
+                                   (8, 512, 3584), (257, 1000, 96)])
+def test_gemm(ops32, adt, wdt, odt, M, N, K):
+    rng = np.random.default_rng(M * 1000 + N + K)
+    a = rng.standard_normal((M, K)).astype(np.float32)
+    w = (rng.standard_normal((N, K)) / math.sqrt(K)).astype(np.float32)
+    b = rng.standard_normal(N).astype(np.float32)
+    want = rounded(a, adt) @ rounded(w, wdt).T + b
+    out = torch.empty((M, N), dtype=odt, device="cuda")
+    ops32.gemm(dev(a, adt), dev(w, wdt), out, bias=dev(b))
+    tol = 2e-5 if odt == torch.float32 else 0.02
+    got = out.float().cpu().numpy()
+    assert np.max(np.abs(got - want)) <= tol * max(1.0, np.max(np.abs(want)))
+    if odt == torch.float32:       # accumulate into the residual sum, through a strided view
+        wide = torch.zeros((M, N + 3), dtype=torch.float32, device="cuda")
+        res = rng.standard_normal((M, N)).astype(np.float32)
+        wide[:, :N] = dev(res)
+        ops32.gemm(dev(a, adt), dev(w, wdt), wide[:, :N], accumulate=True)
+        got = wide[:, :N].cpu().numpy()
+        assert np.max(np.abs(got - (want - b + res))) <= tol * max(1.0, np.max(np.abs(want)))
+        assert float(wide[:, N:].abs().max()) == 0.0
+
+
+def test_gemm_matches_library_product(ops32):
+    """The kernel against the library's fp32 matrix product on the same operands."""
+    torch.manual_seed(0)
+    a = torch.randn(70, 300, device="cuda")
+    w = torch.randn(90, 300, device="cuda")
+    out = torch.empty(70, 90, device="cuda")
+    ops32.gemm(a, w, out)
+    ref = (a.double() @ w.double().T).float()
+    assert float((out - ref).abs().max()) < 1e-3
+
+
+class FakeCache(types.SimpleNamespace):
+    pass
+
+
+class FakeStep:
+    def __init__(self, positions, token_slot, block_table, slot_map):
+        self.positions, self.token_slot = positions, token_slot
+        self._g = types.SimpleNamespace(block_table=block_table, slot_map=slot_map)
+
+    def group(self, i):
+        return self._g
+
+
+def paged_setup(rng, lengths, G, D, page, dtype, n_pages=None, shuffle=True):
+    """Random keys and values for requests of the given lengths, scattered over pages in a
+    random order. Returns (k [list of [n, G, D]], v, cache, block_table)."""
+    blocks = [-(-n // page) for n in lengths]
+    n_pages = n_pages or sum(blocks) + 3
+    perm = rng.permutation(n_pages) if shuffle else np.arange(n_pages)
+    max_blocks = max(blocks) + 2
+    table = np.zeros((len(lengths), max_blocks), np.int32)
+    kc = np.full((n_pages * page, G * D), 1e4, np.float32)     # stale rows hold large values
+    vc = np.full((n_pages * page, G * D), -1e4, np.float32)
+    ks, vs, at = [], [], 0
+    for s, n in enumerate(lengths):
+        k = rng.standard_normal((n, G, D)).astype(np.float32)
+        v = rng.standard_normal((n, G, D)).astype(np.float32)
+        for b in range(blocks[s]):
+            pg = perm[at]
+            at += 1
+            table[s, b] = pg
+            rows = slice(b * page, min((b + 1) * page, n))
+            cnt = rows.stop - rows.start
+            kc[pg * page:pg * page + cnt] = k[rows].reshape(cnt, G * D)
+            vc[pg * page:pg * page + cnt] = v[rows].reshape(cnt, G * D)
+        ks.append(k)
+        vs.append(v)
+    cache = FakeCache(group=0, k=dev(kc, dtype), v=dev(vc, dtype), page_tokens=page, window=0)
+    return ks, vs, cache, ints(table)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,G,D,page,window", [(4, 2, 16, 16, 0), (3, 1, 32, 8, 20), (8, 8, 64, 16, 0),
+                                               (14, 2, 64, 32, 0), (6, 2, 128, 16, 70), (5, 5, 48, 4, 0),
+                                               (2, 1, 256, 64, 0)])
+def test_paged_attention(ops32, dtype, H, G, D, page, window):
+    """Queries at the last positions of each request (a prompt portion of several tokens for
+    some, a single token for others) against attention over whole sequences."""
+    rng = np.random.default_rng(H * 100 + D + page)
+    lengths = [1, 5, 64, 130, 203]
+    q_lens = [1, 3, 64, 1, 17]
+    ks, vs, cache, table = paged_setup(rng, lengths, G, D, page, dtype)
+    qs, positions, slots, wants = [], [], [], []
+    for s, (n, ql) in enumerate(zip(lengths, q_lens)):
+        q_full = rng.standard_normal((n, H, D)).astype(np.float32)
+        full = plain.attention(rounded(q_full, dtype), rounded(ks[s], dtype), rounded(vs[s], dtype), window)
+        qs.append(q_full[n - ql:])
+        wants.append(full[n - ql:])
+        positions += list(range(n - ql, n))
+        slots += [s] * ql
+    q = np.concatenate(qs).reshape(-1, H * D)
+    want = np.concatenate(wants).reshape(-1, H * D)
+    T = q.shape[0]
+    qpad = torch.zeros((T, H * D + 2 * G * D), dtype=dtype, device="cuda")    # q inside wider rows
+    qpad[:, :H * D] = dev(q, dtype)
+    out = torch.empty((T, H * D), dtype=dtype, device="cuda")
+    step = FakeStep(ints(positions), ints(slots), table, None)
+    ops32.paged_attention(qpad[:, :H * D], H, G, D, cache, step, window, 1.0 / math.sqrt(D), out)
+    tol = 2e-5 if dtype == torch.float32 else 0.02
+    err = np.max(np.abs(out.float().cpu().numpy() - want))
+    assert err <= tol, f"max |diff| {err:.3e}"
+
+
+def test_attention_special_cases(ops32):
+    """A single query at position 0 returns value row 0 exactly; equal scores (zero query)
+    return the mean of the visible value rows (softmax of equal numbers)."""
+    rng = np.random.default_rng(1)
+    H, G, D, page = 2, 1, 32, 8
+    ks, vs, cache, table = paged_setup(rng, [1, 40], G, D, page, torch.float32)
+    q = np.zeros((2, H * D), np.float32)
+    q[0] = rng.standard_normal(H * D)
+    out = torch.empty((2, H * D), dtype=torch.float32, device="cuda")
+    step = FakeStep(ints([0, 39]), ints([0, 1]), table, None)
+    ops32.paged_attention(dev(q), H, G, D, cache, step, 0, 1.0, out)
+    got = out.cpu().numpy()
+    assert np.array_equal(got[0].reshape(H, D), np.repeat(vs[0][0], H, axis=0))
+    assert np.max(np.abs(got[1].reshape(H, D) - vs[1].mean(axis=0))) < 1e-6
+    ops32.paged_attention(dev(q), H, G, D, cache, step, 10, 1.0, out)     # window of 10: mean of the last 10
+    assert np.max(np.abs(out.cpu().numpy()[1].reshape(H, D) - vs[1][30:].mean(axis=0))) < 1e-6
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,G,D,rot", [(4, 2, 16, 16), (3, 1, 32, 32), (5, 5, 48, 32), (2, 1, 128, 128)])
+def test_rope_store(ops32, dtype, H, G, D, rot):
+    rng = np.random.default_rng(D + rot)
+    T, base = 9, 1e4 if D < 100 else 1e6
+    positions = [0, 1, 2, 77, 500, 4095, 3, 30000, 17]
+    qkv = rng.standard_normal((T, (H + 2 * G) * D)).astype(np.float32)
+    slot_map = [4, 0, 11, 7, 2, 9, 1, 3, 10]
+    t_qkv = dev(qkv, dtype)
+    cache = FakeCache(group=0, k=torch.zeros((12, G * D), dtype=dtype, device="cuda"),
+                      v=torch.zeros((12, G * D), dtype=dtype, device="cuda"))
+    i = np.arange(rot // 2, dtype=np.float64)
+    inv_freq = dev((base ** (-2.0 * i / rot)).astype(np.float32))
+    ops32.rope_store(t_qkv, ints(positions), inv_freq, rot, H, G, D, cache, ints(slot_map))
+    src = rounded(qkv, dtype)
+    q_want = plain.rope(src[:, :H * D].reshape(T, H, D), positions, rot, base).reshape(T, H * D)
+    k_want = plain.rope(src[:, H * D:(H + G) * D].reshape(T, G, D), positions, rot, base).reshape(T, G * D)
+    v_want = src[:, (H + G) * D:]
+    # the angle is an fp32 product: at position 30000 it is off by up to 30000 * 2^-24 rad
+    tol = 4e-3 if dtype == torch.float32 else 0.03
+    got = t_qkv.float().cpu().numpy()
+    assert np.max(np.abs(got[:, :H * D] - q_want)) <= tol
+    small = [t for t, p in enumerate(positions) if p < 100]
+    assert np.max(np.abs(got[small, :H * D] - q_want[small])) <= (1e-5 if dtype == torch.float32 else 0.03)
+    kc, vc = cache.k.float().cpu().numpy(), cache.v.float().cpu().numpy()
+    assert np.max(np.abs(kc[slot_map] - k_want)) <= tol
+    assert np.array_equal(vc[slot_map], v_want.astype(np.float32))
+    assert np.array_equal(got[0, :H * D], src[0, :H * D].astype(np.float32)), "position 0 is the identity"
+    unused = [r for r in range(12) if r not in slot_map]
+    assert float(cache.k[unused].abs().max()) == 0.0
+
+
+def test_rope_relative_position(ops32):
+    """<rope(q, p + s), rope(k, p' + s)> does not depend on the shift s: only distances count.
+    A wrong sign or a wrong pairing breaks this."""
+    rng = np.random.default_rng(5)
+    H, G, D = 1, 1, 64
+    qkv = rng.standard_normal((1, 3 * D)).astype(np.float32)
+    i = np.arange(D // 2, dtype=np.float64)
+    inv_freq = dev((1e4 ** (-2.0 * i / D)).astype(np.float32))
+    dots = []
+    for shift in (0, 5, 100):
+        rows = torch.cat([dev(qkv), dev(qkv)])
+        cache = FakeCache(group=0, k=torch.zeros((2, D), device="cuda"), v=torch.zeros((2, D), device="cuda"))
+        ops32.rope_store(rows, ints([9 + shift, 2 + shift]), inv_freq, D, H, G, D, cache, ints([0, 1]))
+        dots.append(float((rows[0, :D].double() * cache.k[1].double()).sum()))
+    assert abs(dots[0] - dots[1]) < 1e-4 and abs(dots[0] - dots[2]) < 1e-4
+    want = float((plain.rope(qkv[:, :D].reshape(1, 1, D).astype(np.float64), [9], D, 1e4) *
+                  plain.rope(qkv[:, D:2 * D].reshape(1, 1, D).astype(np.float64), [2], D, 1e4)).sum())
+    assert abs(dots[0] - want) < 1e-4
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_swiglu(ops32, dtype):
+    rng = np.random.default_rng(3)
+    gu = (rng.standard_normal((5, 2 * 177)) * 3).astype(np.float32)
+    out = torch.empty((5, 177), dtype=dtype, device="cuda")
+    ops32.swiglu(dev(gu, dtype), out)
+    src = rounded(gu, dtype)
+    want = plain.silu(src[:, :177]) * src[:, 177:]
+    tol = 1e-5 if dtype == torch.float32 else 0.02
+    assert np.max(np.abs(out.float().cpu().numpy() - want)) <= tol * np.max(np.abs(want))
+    one = torch.empty((1, 2), dtype=torch.float32, device="cuda")
+    ops32.swiglu(dev(np.array([[0.0, 1.0, 5.0, 1.0]], np.float32)), one)     # silu(0) = 0, silu(1) = 0.7310585786
+    assert float(one[0, 0]) == 0.0 and abs(float(one[0, 1]) - 0.7310585786) < 1e-6
+
+
+def test_argmax_and_topk(ops32):
+    rng = np.random.default_rng(8)
+    logits = rng.standard_normal((6, 1000)).astype(np.float32)
+    logits[1, 17] = logits[1, 900] = 9.0        # a tie: the lower id wins
+    logits[2, :] = 0.5                          # all equal
+    logits[3, 999] = 50.0
+    t = dev(logits)
+    assert ops32.argmax(t).cpu().tolist() == [int(np.argmax(r)) for r in logits]
+    assert ops32.argmax(t).cpu().tolist()[1:4] == [17, 0, 999]
+    ids, vals, stats = ops32.topk(t, 40)
+    for r in range(6):
+        order = sorted(range(1000), key=lambda i: (-logits[r, i], i))[:40]
+        assert ids[r].cpu().tolist() == order
+        assert np.array_equal(vals[r].cpu().numpy(), logits[r, order])
+        mx = logits[r].max()
+        lse = np.log(np.sum(np.exp(logits[r].astype(np.float64) - mx)))
+        assert float(stats[r, 0]) == mx and abs(float(stats[r, 1]) - lse) < 1e-5
+    big = dev(rng.standard_normal((2, 152064)).astype(np.float32))
+    assert ops32.argmax(big).cpu().tolist() == big.argmax(dim=1).cpu().tolist()
+
+
+def test_kernels_refuse_what_they_cannot_do(ops32):
+    from hf_cpu_amd.status import EngineError
+    with pytest.raises(EngineError, match="head_dim"):
+        cache = FakeCache(group=0, k=torch.zeros((16, 512), device="cuda"), v=torch.zeros((16, 512), device="cuda"),
+                          page_tokens=16, window=0)
+        step = FakeStep(ints([0]), ints([0]), ints(np.zeros((1, 4))), None)
+        ops32.paged_attention(torch.zeros((1, 512), device="cuda"), 1, 1, 512, cache, step, 0, 1.0,
+                              torch.zeros((1, 512), device="cuda"))
+    with pytest.raises(EngineError, match="shapes"):
+        ops32.gemm(torch.zeros((2, 3), device="cuda"), torch.zeros((4, 5), device="cuda"),
+                   torch.zeros((2, 4), device="cuda"))
+    with pytest.raises(EngineError, match="multiple"):
+        cache = FakeCache(group=0, k=torch.zeros((16, 32), device="cuda"), v=torch.zeros((16, 32), device="cuda"),
+                          page_tokens=16, window=0)
+        step = FakeStep(ints([0]), ints([0]), ints(np.zeros((1, 4))), None)
+        ops32.paged_attention(torch.zeros((1, 48), device="cuda"), 3, 2, 16, cache, step, 0, 1.0,
+                              torch.zeros((1, 48), device="cuda"))

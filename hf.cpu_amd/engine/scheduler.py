@@ -1,0 +1,265 @@
+"""The scheduler: admits requests, cuts prompts into portions under a token budget,
+decodes, finishes and frees.
+
+The reference serves one request at a time: prefill in chunks of ``--batch`` tokens with
+logits only for the last chunk (src/ops.c:788-795), then sample -> check -> feed per step
+(src/ops.c:827-893). Here many requests share every step. Per request the order of events
+is the reference's: the first token is sampled from the prefill's logits; an end-of-sequence
+token is neither reported nor fed (src/ops.c:849); a token sampled at the last allowed step
+is reported but not fed (src/ops.c:881); the cap on new tokens is
+``min(max_tokens, ctx_max - prompt)`` with stop reason ``length`` or ``ctx`` (src/ops.c:757-758).
+
+Each step:
+ 1. every running request whose next token is a single decoded token brings it;
+ 2. what is left of the token budget goes to prompt portions, oldest request first:
+    first those already running, then waiting ones, admitted while a state slot is free
+    and fewer than ``max_seqs`` are live;
+ 3. pages for the whole step are checked before it runs. If they do not suffice, prompt
+    portions are shrunk or dropped, newest first. If the decoded tokens alone do not fit,
+    the most recently admitted running request is preempted: its pages and slot are given
+    back, its tokens (prompt and what it generated) are kept, and it waits at the head of
+    the queue to be recomputed as a prompt, which starts once pages for all its tokens are
+    free again (so it is not thrown out again at once). A request that does not fit even
+    alone fails with ERANGE.
+"""
+import time
+from collections import deque
+from dataclasses import dataclass, field
+
+from ..cache import OutOfPages
+from ..sampling import Rng, SamplerParams
+from ..status import ECANCEL, EINVAL, ERANGE, EngineError, fail
+
+WAITING, RUNNING, FINISHED = "waiting", "running", "finished"
+
+
+@dataclass
+class Request:
+    req_id: object
+    prompt: list
+    params: SamplerParams = field(default_factory=SamplerParams)
+    max_tokens: int = 512                    # src/opts.c:107
+    seed: int = 0
+    logprobs: int = 0
+    eos_ids: tuple = ()
+    timeout: float = 0.0                     # seconds, 0 = none
+    # ---- state ----
+    status: str = WAITING
+    tokens: list = None                      # prompt + generated tokens (the next input stream)
+    n_fed: int = 0                           # how many of `tokens` are in the cache
+    generated: list = field(default_factory=list)
+    choices: list = field(default_factory=list)
+    stop: str = None                         # eos | length | ctx | cancel | timeout
+    error: EngineError = None
+    cancel: bool = False
+    n_cap: int = 0
+    rng: Rng = None
+    preemptions: int = 0
+    t_submit: float = 0.0
+    t_first: float = None                    # when the prompt was done (first logits)
+    t_done: float = None
+    admitted_at: int = -1                    # admission order, for the preemption choice
+
+    @property
+    def unfed(self):
+        return len(self.tokens) - self.n_fed
+
+
+@dataclass
+class StepPlan:
+    entries: list            # (request, n_tokens, wants_logits)
+    preempted: list
+    failed: list
+
+
+class Scheduler:
+    def __init__(self, engine, sampler, token_budget=64, max_seqs=None, ctx_max=None, clock=time.monotonic):
+        self.engine, self.sampler = engine, sampler
+        self.manager = engine.manager
+        self.token_budget = int(token_budget)                          # --batch, src/opts.c:44
+        self.max_seqs = min(max_seqs or self.manager.n_slots, self.manager.n_slots)
+        self.ctx_max = min(ctx_max or self.manager.max_context, self.manager.max_context)
+        if self.token_budget < 1 or self.max_seqs < 1:
+            fail(EINVAL, "scheduler: the token budget and max_seqs must be at least 1")
+        self.clock = clock
+        self.waiting = deque()
+        self.running = []
+        self.finished = []
+        self._admissions = 0
+        self.steps = 0
+        self.on_token = None          # callback(request, choice)
+        self.on_finish = None         # callback(request)
+        self.on_prefill = None        # callback(request)
+
+    # ---- submission --------------------------------------------------------
+    def submit(self, req):
+        if len(req.prompt) == 0:
+            fail(EINVAL, "the prompt is empty")                                     # src/ops.c:752
+        if len(req.prompt) >= self.ctx_max:
+            fail(ERANGE, f"the prompt has {len(req.prompt)} tokens, --ctx-max is {self.ctx_max}")   # src/ops.c:753-756
+        vocab = self.engine.vocab_size
+        for t in req.prompt:
+            if not 0 <= int(t) < vocab:
+                fail(EINVAL, f"token id {t} is outside the vocabulary of {vocab}")  # src/ops.c:582
+        if req.max_tokens < 1:
+            fail(EINVAL, "--max-tokens must be at least 1")
+        req.params.check()
+        req.tokens = [int(t) for t in req.prompt]
+        req.n_cap = min(req.max_tokens, self.ctx_max - len(req.prompt))             # src/ops.c:757
+        req.rng = Rng(req.seed)
+        req.status = WAITING
+        req.t_submit = self.clock()
+        self.waiting.append(req)
+        return req
+
+    @property
+    def idle(self):
+        return not self.waiting and not self.running
+
+    # ---- planning ------------------------------------------------------------
+    def plan(self):
+        """Decides what the next step holds. Changes the books only by preempting or failing
+        requests that cannot go on; every pass of the loop either returns or removes a
+        request from the running set, so it ends."""
+        preempted, failed = [], []
+        while True:
+            entries = self._fill(preempted)
+            if entries is not None and (entries or not self.running):
+                break
+            # The decoded tokens do not fit, or nobody can move: the newest running request yields.
+            victim = max(self.running, key=lambda r: r.admitted_at)
+            if len(self.running) == 1:
+                self._finish(victim, error=EngineError(ERANGE, f"request {victim.req_id!r} does not fit the "
+                                                                "cache even alone"))
+                failed.append(victim)
+            else:
+                self._preempt(victim)
+                preempted.append(victim)
+        if not entries and self.waiting:
+            head = self.waiting.popleft()         # nothing runs and the head of the queue cannot start
+            self._finish(head, error=EngineError(ERANGE, f"request {head.req_id!r} does not fit the cache "
+                                                         "even alone"))
+            failed.append(head)
+        return StepPlan(entries, preempted, failed)
+
+    def _fill(self, preempted):
+        """The entries of a step under the budget and the pages at hand, or None if not even
+        the decoded tokens fit."""
+        mgr = self.manager
+        decode = [r for r in self.running if r.unfed == 1 and r.n_fed > 0]
+        if not mgr.can_reserve([(r.req_id, 1) for r in decode]):
+            return None
+        budget = self.token_budget
+        entries = [(r, 1, True) for r in decode[:budget]]
+        budget -= len(entries)
+        wanted = [(r.req_id, 1) for r, _, _ in entries]
+        prefilling = [r for r in self.running if not (r.unfed == 1 and r.n_fed > 0)]
+        live = len(self.running)
+        free_slots = mgr.n_slots - len(mgr.held)
+        candidates = [(r, False) for r in prefilling] + [(r, True) for r in self.waiting]
+        for r, is_new in candidates:
+            if budget <= 0:
+                break
+            if is_new and (live >= self.max_seqs or free_slots <= 0 or r in preempted):
+                break
+            if is_new and r.preemptions and not mgr.can_reserve(wanted + [(r.req_id, r.unfed)]):
+                break                          # a preempted request returns when all it lost fits again
+            n = min(r.unfed, budget)
+            # shrink the portion to what the pages allow; skip the request if not even one token fits
+            while n > 0 and not mgr.can_reserve(wanted + [(r.req_id, n)]):
+                n = self._shrink(r, n)
+            if n <= 0:
+                if is_new:
+                    break                      # keep the queue's order: nobody overtakes
+                continue
+            entries.append((r, n, n == r.unfed))
+            wanted.append((r.req_id, n))
+            budget -= n
+            if is_new:
+                live += 1
+                free_slots -= 1
+        return entries
+
+    def _shrink(self, r, n):
+        """The next smaller portion worth trying: one page less."""
+        P = self.manager.page_tokens
+        held = self.manager.held.get(r.req_id)
+        start = held.length if held else 0
+        return ((start + n - 1) // P) * P - start        # tokens that end just before the last page touched
+
+    def _preempt(self, r):
+        self.engine.release(r.req_id)
+        self.running.remove(r)
+        r.n_fed = 0
+        r.status = WAITING
+        r.preemptions += 1
+        self.waiting.appendleft(r)
+
+    def _finish(self, r, stop=None, error=None):
+        if r.status == RUNNING:
+            self.running.remove(r)
+            if self.engine.has(r.req_id):
+                self.engine.release(r.req_id)
+        r.status, r.stop, r.error, r.t_done = FINISHED, stop, error, self.clock()
+        self.finished.append(r)
+        if self.on_finish:
+            self.on_finish(r)
+
+    # ---- one step ------------------------------------------------------------
+    def step(self):
+        """Plans, runs and books one step. Returns the plan (None if there was nothing to do)."""
+        now = self.clock()
+        for r in list(self.running) + list(self.waiting):                       # src/ops.c:790, 829
+            expired = r.timeout > 0 and now - r.t_submit > r.timeout
+            if r.cancel or expired:
+                if r.status == WAITING:
+                    self.waiting.remove(r)
+                if r.t_first is None:       # still in its prompt: an error, as in the reference
+                    self._finish(r, error=EngineError(ECANCEL, "cancelled" if r.cancel else "timeout during prefill"))
+                else:
+                    self._finish(r, stop="cancel" if r.cancel else "timeout")
+        if self.idle:
+            return None
+        plan = self.plan()
+        if not plan.entries:
+            return plan
+        for r, _, _ in plan.entries:
+            if r.status == WAITING:
+                self.waiting.remove(r)
+                r.status = RUNNING
+                r.admitted_at = self._admissions
+                self._admissions += 1
+                self.running.append(r)
+        step_entries = [(r.req_id, r.tokens[r.n_fed:r.n_fed + n], [n - 1] if want else [])
+                        for r, n, want in plan.entries]
+        logits = self.engine.step(step_entries)
+        self.steps += 1
+        sampled = [r for r, n, want in plan.entries if want]
+        for r, n, _ in plan.entries:
+            r.n_fed += n
+        if sampled:
+            choices = self.sampler.sample(logits, [(r.params, r.rng, r.logprobs) for r in sampled])
+            for r, ch in zip(sampled, choices):
+                self._accept(r, ch)
+        return plan
+
+    def _accept(self, r, ch):
+        if r.t_first is None:
+            r.t_first = self.clock()
+            if self.on_prefill:
+                self.on_prefill(r)
+        if ch.token in r.eos_ids:                                              # src/ops.c:849
+            return self._finish(r, stop="eos")
+        r.generated.append(ch.token)
+        r.choices.append(ch)
+        if self.on_token:
+            self.on_token(r, ch)
+        if len(r.generated) >= r.n_cap:                                        # src/ops.c:881, 758
+            return self._finish(r, stop="length" if r.n_cap == r.max_tokens else "ctx")
+        r.tokens.append(ch.token)
+
+    def run(self):
+        """Steps until every submitted request is finished; returns them in finishing order."""
+        while not self.idle:
+            self.step()
+        return self.finished

@@ -1,0 +1,134 @@
+"""Sampling the next token from a row of logits.
+
+The pipeline and its order are the reference's ``hfc_sample`` (src/sample.c:66-117):
+greedy when the temperature is not positive (first index of the maximum); otherwise
+candidates ordered by (logit descending, id ascending), cut to ``top_k``, turned into
+probabilities ``exp((l - max) / temp)`` normalised in fp32, cut by ``min_p`` (leading run
+with ``p >= min_p * p_max``), cut by ``top_p`` (shortest prefix whose sum reaches it), and
+one draw ``r = uniform * sum`` picks the first candidate whose running sum exceeds ``r``.
+
+The GPU does the part that touches the whole vocabulary (argmax; the ordered best-k and
+the row's log-sum-exp, kernels in csrc/sampling.hip); the few candidates left are finished
+on the host in fp32 in exactly the order above. With ``top_k`` off (0) or beyond the
+kernel's 1024 the row is copied and ordered on the host.
+"""
+from dataclasses import dataclass
+
+import numpy as np
+
+from ..status import EINVAL, fail
+
+TOPK_KERNEL_MAX = 1024
+f32 = np.float32
+
+
+@dataclass(frozen=True)
+class SamplerParams:
+    """Defaults are the reference's (src/opts.c:102-106)."""
+    temp: float = 0.8
+    top_k: int = 40
+    top_p: float = 0.95
+    min_p: float = 0.05
+
+    def check(self):
+        if not 0 <= self.temp <= 5:
+            fail(EINVAL, f"--temp {self.temp} is outside 0..5")                 # src/opts.c:55
+        if not 0 <= self.top_k <= 1000000:
+            fail(EINVAL, f"--top-k {self.top_k} is outside 0..1000000")
+        if not 0 <= self.top_p <= 1 or not 0 <= self.min_p <= 1:
+            fail(EINVAL, "--top-p and --min-p must lie in 0..1")
+        return self
+
+    @property
+    def greedy(self):
+        return self.temp <= 0
+
+
+def pick(ids, logits, params, rng):
+    """The draw among candidates already ordered (logit descending, id ascending) and cut
+    to top_k: steps 3 to 6 of the pipeline, in fp32 (src/sample.c:99-114)."""
+    logits = np.asarray(logits, dtype=f32)
+    p = np.exp((logits - logits[0]) / f32(params.temp), dtype=f32)
+    total = f32(0)
+    for v in p:
+        total = f32(total + v)
+    p = (p / total).astype(f32)
+    kept = len(p)
+    if params.min_p > 0:
+        kept = 0
+        while kept < len(p) and p[kept] >= f32(params.min_p) * p[0]:
+            kept += 1
+        kept = max(kept, 1)
+    if 0 < params.top_p < 1:
+        cum = f32(0)
+        for i in range(kept):
+            cum = f32(cum + p[i])
+            if cum >= f32(params.top_p):
+                kept = i + 1
+                break
+    total = f32(0)
+    for i in range(kept):
+        total = f32(total + p[i])
+    r = f32(rng.uniform() * total)
+    cum = f32(0)
+    for i in range(kept):
+        cum = f32(cum + p[i])
+        if r < cum:
+            return int(ids[i])
+    return int(ids[kept - 1])
+
+
+def order_on_host(row, top_k):
+    """All candidates of a row in order, cut to top_k if it is on (src/sample.c:59-64, 81-98)."""
+    row = np.asarray(row, dtype=f32)
+    order = np.lexsort((np.arange(len(row)), -row))
+    if 0 < top_k < len(order):
+        order = order[:top_k]
+    return order.astype(np.int64), row[order]
+
+
+@dataclass
+class Choice:
+    token: int
+    logprob: float = None          # of the chosen token, if asked for
+    top: list = None               # [(id, logprob), ...] best first, if asked for
+
+
+class Sampler:
+    """Samples one token per row of a step's logits. ``wants[i]`` = (params, rng, n_logprobs)."""
+
+    def __init__(self, ops):
+        self.ops = ops
+
+    def sample(self, logits, wants):
+        R = logits.shape[0]
+        if R != len(wants):
+            fail(EINVAL, f"sampler: {R} rows of logits for {len(wants)} requests")
+        out = [None] * R
+        need_k = 0
+        for params, _, n_lp in wants:
+            if n_lp or (not params.greedy and 0 < params.top_k <= TOPK_KERNEL_MAX):
+                need_k = max(need_k, n_lp, 0 if params.greedy else min(params.top_k, TOPK_KERNEL_MAX))
+        need_k = min(need_k, logits.shape[1])
+        greedy = [i for i, (p, _, _) in enumerate(wants) if p.greedy]
+        arg = self.ops.argmax(logits).cpu().numpy() if greedy else None
+        ids = vals = stats = None
+        if need_k or any(n for _, _, n in wants):
+            ids, vals, stats = self.ops.topk(logits, need_k)
+            ids, vals, stats = ids.cpu().numpy(), vals.cpu().numpy(), stats.cpu().numpy()
+        for i, (params, rng, n_lp) in enumerate(wants):
+            if params.greedy:
+                tok = int(arg[i])
+            elif 0 < params.top_k <= TOPK_KERNEL_MAX and params.top_k < logits.shape[1]:
+                tok = pick(ids[i, :params.top_k], vals[i, :params.top_k], params, rng)
+            else:
+                cand, cl = order_on_host(logits[i].cpu().numpy(), params.top_k)
+                tok = pick(cand, cl, params, rng)
+            ch = Choice(tok)
+            if n_lp:
+                mx, lse = float(stats[i, 0]), float(stats[i, 1])
+                ch.top = [(int(t), float(v) - mx - lse) for t, v in zip(ids[i, :n_lp], vals[i, :n_lp])]
+                hit = [lp for t, lp in ch.top if t == tok]
+                ch.logprob = hit[0] if hit else float(logits[i, tok].item()) - mx - lse     # src/sample.c:25-33
+            out[i] = ch
+        return out

@@ -227,11 +227,14 @@ def plain_logits(model_dir, reqs, round_weights_bf16=False):
 
 
 def compare(got, want, tol, what=""):
-    """Every wanted row within ``tol`` (max abs difference) of the plain implementation;
-    reports the first wrong place in position order."""
+    """Every wanted row within ``tol`` times the request's largest |logit| of the plain
+    implementation (max abs difference); reports the first wrong place in position order.
+    Returns the worst relative difference."""
     worst = 0.0
+    scale = {r: float(np.max(np.abs(v))) for r, v in want.items()}
     for (r, pos) in sorted(got, key=lambda k: (k[0], k[1])):
-        err = float(np.max(np.abs(got[(r, pos)].astype(np.float64) - want[r][pos])))
+        err = float(np.max(np.abs(got[(r, pos)].astype(np.float64) - want[r][pos]))) / scale[r]
         worst = max(worst, err)
-        assert err <= tol, f"{what}: request {r} position {pos}: max |diff| {err:.3e} > {tol:.1e}"
+        assert err <= tol, (f"{what}: request {r} position {pos}: max |diff| / max |logit| = {err:.3e} "
+                            f"> {tol:.1e}")
     return worst

@@ -1,0 +1,221 @@
+"""The scheduler's decisions (no GPU): a stand-in engine with the real cache manager, and a
+stand-in sampler that follows a script."""
+import pytest
+
+from hf_cpu_amd.cache import CacheManager
+from hf_cpu_amd.engine.scheduler import Request, Scheduler
+from hf_cpu_amd.parts import PagedKV
+from hf_cpu_amd.sampling import Choice, SamplerParams
+from hf_cpu_amd.status import EngineError
+
+
+class FakeEngine:
+    """Books pages like the real engine; 'logits' are the list of (request, position) wanted."""
+
+    def __init__(self, n_pages=8, page=4, slots=4, ctx=64, window=0, vocab=100):
+        self.manager = CacheManager([PagedKV(4, 4, 0), PagedKV(4, 4, window)], page, n_pages, slots, ctx)
+        self.vocab_size = vocab
+        self.log = []
+
+    def has(self, r):
+        return r in self.manager.held
+
+    def release(self, r):
+        self.manager.release(r)
+
+    def step(self, entries):
+        m = self.manager
+        for r, toks, want in entries:
+            if r not in m.held:
+                m.admit(r)
+            m.reserve(r, len(toks))
+        rows = []
+        for r, toks, want in entries:
+            rows += [(r, m.held[r].length + w) for w in want]
+            m.commit(r, len(toks))
+        self.log.append([(r, len(t), list(w)) for r, t, w in entries])
+        m.check()
+        return rows
+
+    @property
+    def shape(self):
+        return None
+
+
+class Rows(list):
+    @property
+    def shape(self):
+        return (len(self), 0)
+
+
+class ScriptSampler:
+    """Token = 10 + number of tokens generated so far, or what ``script[req]`` says."""
+
+    def __init__(self, script=None):
+        self.script = script or {}
+        self.count = {}
+
+    def sample(self, logits, wants):
+        assert len(logits) == len(wants)
+        out = []
+        for (req, pos), _ in zip(logits, wants):
+            i = self.count.get(req, 0)
+            self.count[req] = i + 1
+            seq = self.script.get(req)
+            out.append(Choice(seq[i] if seq and i < len(seq) else 10 + i))
+        return out
+
+
+def greedy():
+    return SamplerParams(temp=0.0)
+
+
+def make(budget=8, **kw):
+    eng = FakeEngine(**kw)
+    return eng, Scheduler(eng, ScriptSampler(), token_budget=budget)
+
+
+def test_prompt_is_cut_into_portions_under_the_budget():
+    eng, s = make(budget=8, n_pages=16)
+    r = s.submit(Request("a", list(range(19)), greedy(), max_tokens=3))
+    s.run()
+    assert eng.log[:3] == [[("a", 8, [])], [("a", 8, [])], [("a", 3, [2])]]       # logits only for the last portion
+    assert eng.log[3:] == [[("a", 1, [0])], [("a", 1, [0])]]
+    assert r.generated == [10, 11, 12] and r.stop == "length"
+    # the token sampled at the last allowed step is reported but never fed (src/ops.c:881)
+    assert sum(n for step in eng.log for _, n, _ in step) == 19 + 2
+    assert not eng.manager.held and all(p.n_held == 0 for p in eng.manager.pools)
+
+
+def test_decode_tokens_go_first_and_share_steps_with_prompt_portions():
+    eng, s = make(budget=8, n_pages=32)
+    a = s.submit(Request("a", [1, 2, 3], greedy(), max_tokens=4))
+    s.step()
+    b = s.submit(Request("b", list(range(20)), greedy(), max_tokens=2))
+    s.step()
+    assert eng.log[1] == [("a", 1, [0]), ("b", 7, [])]       # one decoded token, the rest of the budget to b
+    s.step()
+    assert eng.log[2] == [("a", 1, [0]), ("b", 7, [])]
+    s.run()
+    assert a.generated == [10, 11, 12, 13] and b.generated == [10, 11]
+    assert a.stop == b.stop == "length"
+
+
+def test_admission_is_fifo_and_bounded_by_slots():
+    eng, s = make(budget=64, n_pages=32, slots=2)
+    rs = [s.submit(Request(i, [1, 2, 3, 4], greedy(), max_tokens=2 + i)) for i in range(4)]
+    s.step()
+    assert [r for r, _, _ in eng.log[0]] == [0, 1]             # two slots
+    s.run()
+    order = [r.req_id for r in s.finished]
+    assert order == [0, 1, 2, 3]
+    first_seen = {}
+    for i, step in enumerate(eng.log):
+        for r, _, _ in step:
+            first_seen.setdefault(r, i)
+    assert first_seen[2] < first_seen[3] or first_seen[2] == first_seen[3]
+    assert first_seen[2] > first_seen[1]
+
+
+def test_eos_is_neither_reported_nor_fed():
+    eng = FakeEngine()
+    s = Scheduler(eng, ScriptSampler({"a": [5, 6, 99, 7]}), token_budget=8)
+    seen = []
+    s.on_token = lambda r, ch: seen.append(ch.token)
+    r = s.submit(Request("a", [1, 2], greedy(), max_tokens=10, eos_ids=(99,)))
+    s.run()
+    assert r.generated == [5, 6] and seen == [5, 6] and r.stop == "eos"        # src/ops.c:849
+    assert sum(n for step in eng.log for _, n, _ in step) == 2 + 2
+
+
+def test_context_cap_gives_stop_ctx():
+    eng, s = make(budget=8, ctx=8, n_pages=8)
+    r = s.submit(Request("a", [1, 2, 3, 4, 5], greedy(), max_tokens=10))
+    s.run()
+    assert len(r.generated) == 3 and r.stop == "ctx"           # min(max_tokens, ctx_max - prompt), src/ops.c:757-758
+    with pytest.raises(EngineError) as e:
+        s.submit(Request("b", list(range(8)), greedy()))
+    assert e.value.code == "ERANGE" and "ctx-max" in str(e.value)
+    with pytest.raises(EngineError) as e:
+        s.submit(Request("c", [], greedy()))
+    assert e.value.code == "EINVAL"
+    with pytest.raises(EngineError) as e:
+        s.submit(Request("d", [1, 100], greedy()))
+    assert e.value.code == "EINVAL" and "vocabulary" in str(e.value)
+
+
+def test_prompt_portion_shrinks_to_the_pages_left():
+    eng, s = make(budget=64, n_pages=6, page=4)                # 24 tokens of pages
+    a = s.submit(Request("a", list(range(13)), greedy(), max_tokens=8))
+    s.step()                                                   # a holds 4 pages
+    b = s.submit(Request("b", list(range(30)), greedy(), max_tokens=1))
+    s.step()
+    # a decodes (position 13 fits its 4th page); b gets the two pages left: 8 tokens
+    assert eng.log[1] == [("a", 1, [0]), ("b", 8, [])]
+    s.step()
+    assert eng.log[2] == [("a", 1, [0])]                       # nothing left for b, a goes on
+
+
+def test_preemption_when_decode_runs_out_of_pages():
+    eng, s = make(budget=64, n_pages=4, page=4)                # 16 tokens of pages
+    a = s.submit(Request("a", list(range(7)), greedy(), max_tokens=6))
+    b = s.submit(Request("b", list(range(7)), greedy(), max_tokens=6))
+    s.step()                                                   # both prompts: 2 pages each, pool full
+    assert eng.manager.pools[0].n_free == 0
+    s.step()                                                   # both decode inside their pages (positions 7)
+    assert [r for r, _, _ in eng.log[1]] == ["a", "b"]
+    plan = s.step()                                            # position 8 needs a page each: none free
+    assert [r.req_id for r in plan.preempted] == ["b"]         # the most recently admitted goes
+    assert b.status == "waiting" and b.n_fed == 0 and b.preemptions == 1 and b.generated == [10, 11]
+    assert eng.log[2] == [("a", 1, [0])]
+    s.run()
+    assert a.generated == [10, 11, 12, 13, 14, 15] and a.stop == "length"
+    # b was recomputed as a prompt of 7 + 2 tokens and went on where it was
+    assert b.generated == [10, 11, 12, 13, 14, 15] and b.stop == "length"
+    recompute = [e for step in eng.log for e in step if e[0] == "b" and e[1] == 9]
+    assert recompute == [("b", 9, [8])]
+    assert not eng.manager.held and all(p.n_held == 0 for p in eng.manager.pools)
+
+
+def test_request_that_fits_not_even_alone_fails_with_erange():
+    eng, s = make(budget=64, n_pages=2, page=4, ctx=64)        # 8 tokens of pages
+    r = s.submit(Request("a", list(range(5)), greedy(), max_tokens=20))
+    s.run()
+    assert r.error is not None and r.error.code == "ERANGE" and len(r.generated) == 4
+    assert not eng.manager.held
+    big = s.submit(Request("b", list(range(20)), greedy(), max_tokens=2))
+    s.run()
+    # its prompt is fed in what the pool allows, then it cannot go on
+    assert big.error is not None and big.error.code == "ERANGE"
+    assert not eng.manager.held and all(p.n_held == 0 for p in eng.manager.pools)
+
+
+def test_cancel_and_timeout():
+    now = [0.0]
+    eng = FakeEngine(n_pages=32)
+    s = Scheduler(eng, ScriptSampler(), token_budget=4, clock=lambda: now[0])
+    b = s.submit(Request("b", [1, 2], greedy(), max_tokens=50, timeout=5.0))
+    a = s.submit(Request("a", list(range(10)), greedy(), max_tokens=50, timeout=5.0))
+    s.step()
+    s.step()
+    assert eng.log == [[("b", 2, [1]), ("a", 2, [])], [("b", 1, [0]), ("a", 3, [])]]
+    assert b.t_first is not None and a.t_first is None
+    now[0] = 6.0
+    s.step()
+    assert a.error.code == "ECANCEL" and a.stop is None       # expiry during the prompt is an error
+    assert b.stop == "timeout" and b.error is None and len(b.generated) >= 1
+    c = s.submit(Request("c", [1], greedy(), max_tokens=50))
+    s.step()
+    s.step()
+    c.cancel = True
+    s.step()
+    assert c.stop == "cancel" and not eng.manager.held
+
+
+def test_windowed_group_frees_pages_for_others():
+    eng, s = make(budget=4, n_pages=5, page=4, window=4, ctx=64)
+    r = s.submit(Request("a", list(range(3)), greedy(), max_tokens=30))
+    s.run()
+    # 33 tokens need 9 pages in the full group: it fails there, but the windowed group never held more than 3
+    assert eng.manager.pools[1].high_water <= 3
+    assert r.error is not None and r.error.code == "ERANGE"

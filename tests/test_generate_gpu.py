@@ -1,0 +1,176 @@
+"""Generation through the entry points: the Python session, the command line, the replay tool."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+import helpers
+import plain
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def plain_greedy(model_dir, prompt, n):
+    """Greedy continuation by the plain implementation: the whole sequence again for every token.
+    Returns the tokens and, for each, the margin between the best and the second logit."""
+    cfg, w = plain.read_model(model_dir)
+    toks, margins = list(prompt), []
+    for _ in range(n):
+        row = plain.forward(cfg, w, toks)[-1]
+        order = np.argsort(-row, kind="stable")
+        margins.append(float(row[order[0]] - row[order[1]]))
+        toks.append(int(order[0]))
+    return toks[len(prompt):], margins
+
+
+@pytest.fixture(scope="module")
+def models(tmp_path_factory):
+    out = {}
+    for name in "AB":
+        out[name] = helpers.make_model_dir(str(tmp_path_factory.mktemp("gen" + name)), helpers.CONFIGS[name],
+                                           seed=21 + ord(name))
+    return out
+
+
+@pytest.mark.parametrize("name,dtype", [("A", "float32"), ("B", "float32"), ("A", "bfloat16"), ("B", "bfloat16")])
+def test_greedy_generation_matches_plain(gpu, models, name, dtype):
+    """Prompts of the baseline's workloads decoded together, greedy, through Session.generate.
+    In fp32 the tokens are the plain implementation's; in bf16 they may part only where the
+    plain implementation's two best logits are closer than the bf16 tolerance."""
+    import hf_cpu_amd.session as S
+    cfg = helpers.CONFIGS[name]
+    lengths = [7, 19, 33] if name == "A" else [1, 40, 77]
+    n_new = 16
+    prompts = list(helpers.random_requests(cfg, lengths, seed=5).values())
+    s = S.Session(models[name], dtype=dtype, ctx_max=cfg["max_position_embeddings"], batch=24,
+                  page_size=helpers.PAGE[name], max_seqs=4)
+    gens = s.generate(prompts, temp=0.0, max_tokens=n_new)
+    assert [g.stop for g in gens] == ["length"] * 3 and not s.engine.manager.held
+    for g, p in zip(gens, prompts):
+        want, margins = plain_greedy(models[name], p, n_new)
+        if dtype == "float32":
+            assert g.tokens == want
+        else:
+            for i, (a, b) in enumerate(zip(g.tokens, want)):
+                if a != b:
+                    assert margins[i] < 0.3, f"token {i}: {a} != {b} with margin {margins[i]:.3f}"
+                    break
+    # the same prompts one at a time give the same tokens as together
+    alone = [s.generate(p, temp=0.0, max_tokens=n_new)[0].tokens for p in prompts]
+    assert alone == [g.tokens for g in gens]
+
+
+def test_sampling_is_reproducible_and_follows_the_plain_sampler(gpu, models):
+    """Temperature 0.8 with a fixed seed (the second baseline workload): the same seed gives the
+    same tokens; continuation i of --n uses seed + i; each token is what the plain sampler
+    picks from the plain logits of the sequence so far, unless bf16-free fp32 rounding moves a
+    probability across the draw (never seen at these sizes: asserted exactly)."""
+    import hf_cpu_amd.session as S
+    cfg = helpers.CONFIG_B
+    prompt = helpers.random_requests(cfg, [40], seed=8)["r0"]
+    s = S.Session(models["B"], dtype="float32", ctx_max=256, batch=16, page_size=8, max_seqs=4)
+    a = s.generate(prompt, n=3, temp=0.8, seed=11, max_tokens=24, logprobs=3)
+    b = s.generate(prompt, n=1, temp=0.8, seed=12, max_tokens=24)
+    assert a[1].tokens == b[0].tokens and a[0].tokens != a[1].tokens
+    assert s.generate(prompt, n=3, temp=0.8, seed=11, max_tokens=24)[2].tokens == a[2].tokens
+    pcfg, w = plain.read_model(models["B"])
+    rng, toks = plain.Rng(11), list(prompt)
+    for i, t in enumerate(a[0].tokens):
+        row = plain.forward(pcfg, w, toks)[-1]
+        assert plain.sample(row, 0.8, 40, 0.95, 0.05, rng) == t, f"token {i}"
+        assert abs(a[0].logprobs[i] - plain.logprob(row, t)) < 1e-4
+        top = sorted(range(len(row)), key=lambda j: (-row[j], j))[:3]
+        assert [j for j, _ in a[0].top[i]] == top
+        toks.append(t)
+
+
+def run_cli(args, stdin=""):
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "hfamd")] + args, input=stdin, text=True,
+                       capture_output=True, timeout=300)
+    return r.returncode, r.stdout, r.stderr
+
+
+def events(out):
+    evs = []
+    for line in out.replace("\x1e", "\n").splitlines():
+        if line.startswith("@"):
+            name, _, rest = line[1:].partition(" ")
+            evs.append((name, dict(p.split("=", 1) for p in rest.split(" ") if "=" in p)))
+    return evs
+
+
+def test_command_line_generate(gpu, models):
+    """``--op generate`` with ``--prompt-ids``: the events of the reference's e2e test
+    (tests/e2e.pl:155-179): @prefill tokens=5, six @token, @gen tokens=6 stop=length,
+    @done status=ok; two requests in one process give the same first token; clean errors."""
+    cfg = helpers.CONFIG_A
+    base = ["--dtype", "float32", "--ctx-max", "128", "--page-size", "16", "--max-seqs", "4", "--log-level", "error"]
+    rc, out, err = run_cli(base + ["--stdin-mode", "none", "--model", models["A"], "--prompt-ids", "1 2 3 4 5",
+                                   "--temp", "0", "--max-tokens", "6", "--logprobs", "2", "--id", "x1"])
+    assert rc == 0, err
+    ev = events(out)
+    names = [n for n, _ in ev]
+    assert names == ["begin", "prompt", "prefill"] + ["token"] * 6 + ["gen", "done"]
+    assert ev[0][1] == {"id": "x1", "op": "generate"} and ev[2][1]["tokens"] == "5"
+    assert [e[1]["pos"] for e in ev if e[0] == "token"] == [str(i) for i in range(6)]
+    assert ev[-2][1]["tokens"] == "6" and ev[-2][1]["stop"] == "length" and ev[-1][1]["status"] == "ok"
+    want, _ = plain_greedy(models["A"], [1, 2, 3, 4, 5], 6)
+    assert [int(e[1]["id"]) for e in ev if e[0] == "token"] == want
+    assert all("logprob" in e[1] and "top" in e[1] for e in ev if e[0] == "token")
+    # args mode: two requests, the model stays resident; then errors that do not end the process
+    lines = "\n".join([f"--model {models['A']} --prompt-ids 1,2,3,4,5 --temp 0 --max-tokens 2",
+                       f"--model {models['A']} --prompt-ids '1 2 3 4 5' --temp 0 --max-tokens 3 --n 2",
+                       f"--model {models['A']} --prompt-ids '1 2 999' --temp 0",
+                       f"--model {models['A']} --temp 0",
+                       f"--model {models['A']} --prompt-ids '{' '.join(['7'] * 128)}'",
+                       "--batch 8 --op echo", "!stats", "--op nothing"]) + "\n"
+    rc, out, err = run_cli(base + ["--stdin-mode", "args"], lines)
+    assert rc == 0, err
+    ev = events(out)
+    dones = [e[1] for e in ev if e[0] == "done"]
+    assert [d["status"] for d in dones] == ["ok", "ok", "error", "error", "error", "error", "error"]
+    assert [d.get("code") for d in dones[2:]] == ["EINVAL", "ENOTSUP", "ERANGE", "EINVAL", "EINVAL"]
+    toks = [e[1] for e in ev if e[0] == "token"]
+    assert toks[0]["id"] == str(want[0]) and toks[2]["id"] == str(want[0]) and toks[2]["seq"] == "0"
+    assert any(e[0] == "genall" and e[1]["sequences"] == "2" for e in ev)
+    assert any(e[0] == "stats" and e[1]["requests"] == "6" for e in ev)
+    rc, out, err = run_cli(["--stdin-mode", "none", "--temp", "77"])
+    assert rc == 2 and "outside" in err
+    rc, out, err = run_cli(base + ["--stdin-mode", "none", "--model", "/nonexistent"])
+    assert rc == 1 and "code=EIO" in out
+
+
+def test_trace_run_program(gpu, models, tmp_path):
+    """bin/trace_run as a user calls it: steps on stdin, ``done <step>`` lines, <step>.f32 files;
+    a mixed trace with few pages, in both dtypes, against the plain implementation."""
+    cfg = helpers.CONFIG_B
+    reqs = helpers.random_requests(cfg, [1, 40, 77, 100, 130], seed=4)
+    want = helpers.plain_logits(models["B"], reqs)
+    steps = helpers.trace_mixed(reqs, seed=9)
+    places = helpers.wanted_places(steps)
+    for dtype, tol in (("float32", 5e-6), ("bfloat16", 2e-2)):
+        out = tmp_path / dtype
+        r = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", models["B"],
+                            "--dtype", dtype, "--out", str(out), "--max-tokens", str(helpers.max_live_tokens(steps)),
+                            "--page-size", "8"],
+                           input="".join(json.dumps(s) + "\n" for s in steps), text=True, capture_output=True,
+                           timeout=300)
+        assert r.returncode == 0, r.stderr
+        assert r.stdout.split() == [w for s in steps for w in ("done", str(s["step"]))]
+        got = {}
+        for s in steps:
+            if s["step"] in places:
+                rows = np.fromfile(out / f"{s['step']}.f32", dtype="<f4").reshape(len(places[s["step"]]), -1)
+                for row, key in zip(rows, places[s["step"]]):
+                    got[key] = row
+        assert len(got) == sum(len(t) for t in reqs.values())
+        helpers.compare(got, want, tol, "trace_run " + dtype)
+    bad = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", models["B"], "--dtype",
+                          "float32", "--out", str(tmp_path / "x"), "--max-tokens", "64"],
+                         input=json.dumps({"step": 0, "entries": [{"id": "a", "tokens": list(range(100)), "want": []}],
+                                           "end": []}) + "\n", text=True, capture_output=True, timeout=300)
+    assert bad.returncode == 1 and "ERANGE" in bad.stderr

@@ -1,0 +1,257 @@
+"""Each part alone, a schedule that is more than a list of layers, and a toy mixer with
+state of its own that is registered, built and stepped without touching the package."""
+import dataclasses
+import json
+import math
+import os
+import types
+
+import numpy as np
+import pytest
+import torch
+
+import helpers
+import plain
+import hf_cpu_amd
+from hf_cpu_amd import PartSpec, ScheduleEntry, register_architecture, register_part
+from hf_cpu_amd.engine import Engine
+from hf_cpu_amd.parts import FixedState, PagedKV, ParamSpec, Part
+from hf_cpu_amd.registry import make_part
+
+pytestmark = pytest.mark.gpu
+
+
+def dev(a, dtype=torch.float32):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(dtype).cuda()
+
+
+class Harness:
+    """A cache and step inputs for parts that are run outside a model."""
+
+    def __init__(self, ops, needs, page=4, n_pages=64, slots=4):
+        dtype = ops.act_dtype
+        stub = types.SimpleNamespace(cache_needs=lambda: needs, dtype=dtype, vocab_size=1000)
+        self.engine = Engine(stub, ops, page_tokens=page, n_pages=n_pages, max_seqs=slots)
+
+    def inputs(self, entries):
+        m = self.engine.manager
+        entries = [hf_cpu_amd.engine.Entry(r, t, []) for r, t in entries]
+        for e in entries:
+            if e.req_id not in m.held:
+                m.admit(e.req_id)
+            m.reserve(e.req_id, len(e.tokens))
+        step = self.engine._inputs(entries)
+        for e in entries:
+            m.commit(e.req_id, len(e.tokens))
+        return step
+
+    @property
+    def views(self):
+        return self.engine.storage.views
+
+
+def bind(part, params, ops):
+    part.bind_all({k: dev(v) for k, v in params.items()}, ops)
+    return part
+
+
+def test_norm_part(ops32):
+    rng = np.random.default_rng(0)
+    part = make_part("norm", PartSpec("rmsnorm", dict(size=50, eps=1e-3, prefix="n.")))
+    assert [(s.name, s.shape, s.kind) for s in part.param_specs()] == [("n.weight", (50,), "vector")]
+    w = rng.standard_normal(50).astype(np.float32)
+    bind(part, {"n.weight": w}, ops32)
+    x = rng.standard_normal((6, 50)).astype(np.float32)
+    out = torch.empty((6, 50), device="cuda")
+    part.forward(ops32, dev(x), out)
+    assert np.max(np.abs(out.cpu().numpy() - plain.rmsnorm(x.astype(np.float64), w, 1e-3))) < 1e-5
+
+
+def test_feed_forward_part(ops32):
+    rng = np.random.default_rng(1)
+    E, F = 40, 72
+    part = make_part("feed_forward", PartSpec("gated_mlp", dict(hidden_size=E, intermediate_size=F, prefix="m.")))
+    p = {"m.gate_proj.weight": rng.standard_normal((F, E)) / 6, "m.up_proj.weight": rng.standard_normal((F, E)) / 6,
+         "m.down_proj.weight": rng.standard_normal((E, F)) / 8}
+    p = {k: v.astype(np.float32) for k, v in p.items()}
+    bind(part, p, ops32)
+    h = rng.standard_normal((5, E)).astype(np.float32)
+    x = rng.standard_normal((5, E)).astype(np.float32)
+    tx = dev(x)
+    part.forward(ops32, None, dev(h), tx)
+    want = x + plain.swiglu_mlp(h.astype(np.float64), *(p[k].astype(np.float64) for k in p))
+    assert np.max(np.abs(tx.cpu().numpy() - want)) < 2e-5
+
+
+def attention_reference(p, prefix, h, positions, H, G, D, theta, window, rot=None):
+    T = h.shape[0]
+    q = plain.linear(h, p[prefix + "q_proj.weight"], p[prefix + "q_proj.bias"]).reshape(T, H, D)
+    k = plain.linear(h, p[prefix + "k_proj.weight"], p[prefix + "k_proj.bias"]).reshape(T, G, D)
+    v = plain.linear(h, p[prefix + "v_proj.weight"], p[prefix + "v_proj.bias"]).reshape(T, G, D)
+    q, k = plain.rope(q, positions, rot or D, theta), plain.rope(k, positions, rot or D, theta)
+    return plain.linear(plain.attention(q, k, v, window).reshape(T, H * D), p[prefix + "o_proj.weight"])
+
+
+@pytest.mark.parametrize("H,G,D,window,rot", [(4, 2, 16, 0, 16), (6, 3, 32, 9, 32), (2, 2, 48, 0, 32)])
+def test_attention_part_alone(ops32, H, G, D, window, rot):
+    """One attention mixer with its cache: a prompt in two portions, then single tokens; two
+    requests side by side. The reference is attention over each whole sequence. The third
+    case rotates only part of each head and has a width that is no multiple of 64."""
+    rng = np.random.default_rng(H * D)
+    E, theta = 56, 5e4
+    spec = PartSpec("attention", dict(hidden_size=E, n_heads=H, n_kv_heads=G, head_dim=D, qkv_bias=True,
+                                      window=window, prefix="a.",
+                                      position=PartSpec("rotary", dict(head_dim=D, rot_dim=rot, theta=theta))))
+    part = make_part("mixer", spec)
+    assert part.cache_need() == PagedKV(G * D, G * D, window)
+    p = {s.name: (rng.standard_normal(s.shape) * (0.3 if s.kind == "vector" else 1.2 / math.sqrt(s.shape[1])))
+         .astype(np.float32) for s in part.all_param_specs()}
+    bind(part, p, ops32)
+    p64 = {k: v.astype(np.float64) for k, v in p.items()}
+    hs = {r: rng.standard_normal((n, E)).astype(np.float32) for r, n in (("a", 21), ("b", 13))}
+    want = {r: attention_reference(p64, "a.", h.astype(np.float64), range(len(h)), H, G, D, theta, window, rot)
+            for r, h in hs.items()}
+    har = Harness(ops32, [part.cache_need()])
+    cuts = [[("a", 0, 9)], [("a", 9, 19), ("b", 0, 12)], [("a", 19, 20), ("b", 12, 13)], [("a", 20, 21)]]
+    for cut in cuts:
+        step = har.inputs([(r, [0] * (e - s)) for r, s, e in cut])
+        h = np.concatenate([hs[r][s:e] for r, s, e in cut])
+        x = torch.zeros((h.shape[0], E), device="cuda")
+        part.forward(ops32, step, dev(h), har.views[0], x)
+        ref = np.concatenate([want[r][s:e] for r, s, e in cut])
+        err = np.max(np.abs(x.cpu().numpy() - ref))
+        assert err < 5e-5, f"cut {cut}: {err:.3e}"
+
+
+def toy_plan_factory():
+    """Registers a toy mixer that keeps a running average per request in a state slot, and an
+    architecture whose layers differ: attention + gated mlp, then the toy mixer + gated mlp,
+    with a schedule that runs layer 0 twice and lets the second run of it read the first
+    run's cache. Nothing in the package is edited for this."""
+
+    @register_part("mixer", "toy_ema")
+    class ToyEma(Part):
+        """s <- decay * s + (1 - decay) * h_t per request, in token order; x_t += W s."""
+
+        def __init__(self, hidden_size, decay, prefix=""):
+            super().__init__(prefix)
+            self.E, self.decay = hidden_size, decay
+
+        def param_specs(self):
+            return [ParamSpec(self.prefix + "mix.weight", (self.E, self.E), "matrix", ("normal", 0.2))]
+
+        def cache_need(self):
+            return FixedState(self.E)
+
+        def bind(self, params, ops):
+            self.w = params[self.prefix + "mix.weight"]
+
+        def forward(self, ops, step, h, cache, x, write_cache=True):
+            q_start = step.host["q_start"]
+            for s in range(step.n_seqs):
+                slot = int(step.host["seq_slot"][s])
+                state = cache.state[slot]
+                for t in range(int(q_start[s]), int(q_start[s + 1])):
+                    state.mul_(self.decay).add_(h[t].float(), alpha=1 - self.decay)
+                    x[t] += self.w.float() @ state
+
+    @dataclasses.dataclass(frozen=True)
+    class ToyConfig:
+        architecture: str
+        vocab_size: int
+        hidden_size: int
+        decay: float
+
+        @classmethod
+        def from_dict(cls, obj, origin="config.json"):
+            return cls(obj["architectures"][0], obj["vocab_size"], obj["hidden_size"], obj["decay"])
+
+    def toy_plan(cfg):
+        E = cfg.hidden_size
+
+        def layer(l, mixer):
+            pre = f"layers.{l}."
+            return hf_cpu_amd.LayerPlan(
+                label=pre, block=PartSpec("prenorm", dict(hidden_size=E)),
+                norm1=PartSpec("rmsnorm", dict(size=E, eps=1e-5, prefix=pre + "norm1.")), mixer=mixer,
+                norm2=PartSpec("rmsnorm", dict(size=E, eps=1e-5, prefix=pre + "norm2.")),
+                feed_forward=PartSpec("gated_mlp", dict(hidden_size=E, intermediate_size=2 * E, prefix=pre + "mlp.")))
+        att = PartSpec("attention", dict(hidden_size=E, n_heads=2, n_kv_heads=1, head_dim=16, qkv_bias=False,
+                                         window=0, prefix="layers.0.attn.",
+                                         position=PartSpec("rotary", dict(head_dim=16, rot_dim=16, theta=1e4))))
+        toy = PartSpec("toy_ema", dict(hidden_size=E, decay=cfg.decay, prefix="layers.1.ema."))
+        return hf_cpu_amd.ModelPlan(
+            hidden_size=E, vocab_size=cfg.vocab_size,
+            embedding=PartSpec("lookup", dict(vocab_size=cfg.vocab_size, hidden_size=E, prefix="embed.")),
+            layers=(layer(0, att), layer(1, toy)),
+            schedule=(ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(0, cache_of=0)),
+            final_norm=PartSpec("rmsnorm", dict(size=E, eps=1e-5, prefix="final.")),
+            head=PartSpec("linear", dict(vocab_size=cfg.vocab_size, hidden_size=E, tied=True,
+                                         tied_to="embed.weight", prefix="head.")))
+    register_architecture("ToyEmaForCausalLM", ToyConfig, toy_plan)
+    return ToyConfig
+
+
+def toy_reference(w, toks, decay):
+    """The toy model over a whole sequence, written out directly."""
+    E = w["embed.weight"].shape[1]
+    T = len(toks)
+    x = w["embed.weight"][toks]
+
+    def mlp(x, pre):
+        return plain.swiglu_mlp(plain.rmsnorm(x, w[pre + "norm2.weight"], 1e-5), w[pre + "mlp.gate_proj.weight"],
+                                w[pre + "mlp.up_proj.weight"], w[pre + "mlp.down_proj.weight"])
+
+    def attn(x, own_kv=None):
+        h = plain.rmsnorm(x, w["layers.0.norm1.weight"], 1e-5)
+        q = plain.rope(plain.linear(h, w["layers.0.attn.q_proj.weight"]).reshape(T, 2, 16), range(T), 16, 1e4)
+        if own_kv is None:
+            k = plain.rope(plain.linear(h, w["layers.0.attn.k_proj.weight"]).reshape(T, 1, 16), range(T), 16, 1e4)
+            v = plain.linear(h, w["layers.0.attn.v_proj.weight"]).reshape(T, 1, 16)
+        else:
+            k, v = own_kv
+        out = plain.linear(plain.attention(q, k, v).reshape(T, 32), w["layers.0.attn.o_proj.weight"])
+        return out, (k, v)
+    a, kv = attn(x)
+    x = x + a
+    x = x + mlp(x, "layers.0.")
+    h = plain.rmsnorm(x, w["layers.1.norm1.weight"], 1e-5)
+    s = np.zeros(E)
+    outs = []
+    for t in range(T):
+        s = decay * s + (1 - decay) * h[t]
+        outs.append(w["layers.1.ema.mix.weight"] @ s)
+    x = x + np.array(outs)
+    x = x + mlp(x, "layers.1.")
+    a, _ = attn(x, own_kv=kv)                     # layer 0 again, reading the cache of its first run
+    x = x + a
+    x = x + mlp(x, "layers.0.")
+    return plain.linear(plain.rmsnorm(x, w["final.weight"], 1e-5), w["embed.weight"])
+
+
+def test_toy_mixer_with_state_and_a_schedule_that_repeats(gpu, tmp_path):
+    toy_plan_factory()
+    cfg = {"architectures": ["ToyEmaForCausalLM"], "vocab_size": 90, "hidden_size": 24, "decay": 0.8}
+    d = str(tmp_path / "toy")
+    os.makedirs(d)
+    with open(os.path.join(d, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    model = hf_cpu_amd.Model.from_config(hf_cpu_amd.config_from_dict(cfg))
+    assert [type(n).__name__ for n in model.cache_needs()] == ["PagedKV", "FixedState", "NoneType"]
+    rng = np.random.default_rng(3)
+    w = {}
+    for s in model.param_specs():
+        if s.optional:
+            continue
+        std = {"embed.weight": 0.5}.get(s.name, 0.3 if s.kind == "matrix" else 0.1)
+        w[s.name] = ((1.0 if s.kind == "vector" else 0.0) + rng.standard_normal(s.shape) * std).astype(np.float32)
+    helpers.write_safetensors(os.path.join(d, "model.safetensors"), w)
+    reqs = {f"r{i}": [int(t) for t in rng.integers(0, 90, n)] for i, n in enumerate([5, 23, 40, 31])}
+    w64 = {k: v.astype(np.float64) for k, v in w.items()}
+    want = {r: toy_reference(w64, t, 0.8) for r, t in reqs.items()}
+    for steps in (helpers.trace_whole(reqs), helpers.trace_portions(reqs), helpers.trace_mixed(reqs, seed=2, max_live=3)):
+        engine = hf_cpu_amd.load_engine(d, dtype="float32", page_tokens=8, max_tokens=helpers.max_live_tokens(steps),
+                                        max_seqs=3)
+        got = helpers.run_trace_in_engine(engine, steps)
+        helpers.compare(got, want, 2e-5, "toy model")
+        assert not engine.manager.held

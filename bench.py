@@ -1,0 +1,173 @@
+#!/usr/bin/env python3
+"""Throughput of the engine on the Qwen2.5-7B shape with random weights, one GPU.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L] [--no-points]
+
+A step is one decode step of ``--batch`` sequences (default 8) whose prompts of 2,048
+random ids were prefilled before; W steps are run untimed, then exactly K steps are timed
+between device synchronisations. One JSON line is printed: ``value`` is decoded tokens per
+second; ``prefill`` is one 2,048-token prompt in one step; ``roofline`` prices the decode
+step against HBM bandwidth (every weight it uses once, plus the cache of the live
+requests); ``points`` holds decode at batch 1 and 64. Peaks: HBM 8 TB/s, dense bf16 MFMA
+2.5 PFLOP/s, fp32 157.3 TFLOP/s.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+
+SHAPE_7B = dict(architectures=["Qwen2ForCausalLM"], model_type="qwen2", num_hidden_layers=28, hidden_size=3584,
+                num_attention_heads=28, num_key_value_heads=4, head_dim=128, intermediate_size=18944,
+                vocab_size=152064, rope_theta=1000000.0, rms_norm_eps=1e-6, tie_word_embeddings=False,
+                use_sliding_window=False, max_position_embeddings=32768, hidden_act="silu")
+PROMPT, NEW, PAGE = 2048, 256, 16
+HBM_PEAK = 8.0e12
+FLOP_PEAK = {"bf16": 2.5e15, "fp32": 157.3e12}
+
+
+def matmul_params(c):
+    E, F, QD, KD = c["hidden_size"], c["intermediate_size"], c["num_attention_heads"] * c["head_dim"], \
+        c["num_key_value_heads"] * c["head_dim"]
+    per_layer = E * (QD + 2 * KD) + QD * E + 2 * F * E + F * E
+    return per_layer, c["vocab_size"] * E
+
+
+def decode_bytes(c, elem, batch, mean_ctx):
+    """Bytes one decode step has to read: every matrix, bias and norm once, and the keys and
+    values of every live request."""
+    per_layer, head = matmul_params(c)
+    L, E = c["num_hidden_layers"], c["hidden_size"]
+    KD = c["num_key_value_heads"] * c["head_dim"]
+    QD = c["num_attention_heads"] * c["head_dim"]
+    weights = (L * per_layer + head) * elem + (L * (2 * E + QD + 2 * KD) + E) * 4
+    cache = batch * mean_ctx * 2 * KD * L * elem
+    return weights + cache
+
+
+def prefill_flops(c, T):
+    per_layer, head = matmul_params(c)
+    L, H, D = c["num_hidden_layers"], c["num_attention_heads"], c["head_dim"]
+    return 2.0 * T * L * per_layer + L * 4.0 * D * H * T * (T + 1) / 2 + 2.0 * head
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=0, help="run fewer layers than the shape has (0 = all)")
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
+    ap.add_argument("--prefill-reps", type=int, default=3)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this engine runs on one GPU; --gpus must be 1")
+        return 2
+    if args.steps + args.warmup > NEW:
+        print(f"bench.py: --steps + --warmup must not exceed the {NEW} new tokens of the workload")
+        return 2
+
+    import numpy as np
+    import torch
+    import hf_cpu_amd
+    import hf_cpu_amd.session as S
+
+    shape = dict(SHAPE_7B)
+    layers_of_shape = shape["num_hidden_layers"]
+    if args.layers:
+        shape["num_hidden_layers"] = args.layers
+    cfg = hf_cpu_amd.config_from_dict(shape)
+    short = "bf16" if args.dtype == "bfloat16" else "fp32"
+    elem = 2 if short == "bf16" else 4
+    biggest = max(args.batch, 1 if args.no_points else 64)
+    t_load = time.perf_counter()
+    s = S.Session(cfg, dtype=args.dtype, ctx_max=PROMPT + NEW, batch=PROMPT, page_size=PAGE, max_seqs=biggest,
+                  kv_tokens=biggest * (PROMPT + NEW), seed=0)
+    eng, ops = s.engine, s.ops
+    torch.cuda.synchronize()
+    print(f"[bench] weights and cache ready in {time.perf_counter() - t_load:.1f} s", file=sys.stderr, flush=True)
+    rng = np.random.default_rng(0)
+
+    def prompt():
+        return [int(t) for t in rng.integers(0, cfg.vocab_size, PROMPT)]
+
+    # ---- prefill: one prompt of 2,048 tokens in one step, logits for its last token ----
+    times = []
+    for rep in range(args.prefill_reps + 1):
+        p = prompt()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        logits = eng.step([("prefill", p, [PROMPT - 1])])
+        ops.argmax(logits).cpu()
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t0)
+        eng.release("prefill")
+    pre_s = sorted(times[1:])[len(times[1:]) // 2]            # the first run warms up
+    print(f"[bench] prefill {PROMPT} tokens: {pre_s * 1e3:.1f} ms", file=sys.stderr, flush=True)
+
+    def decode(batch, steps, warmup):
+        ids = [("d", i) for i in range(batch)]
+        last = []
+        for r in ids:
+            logits = eng.step([(r, prompt(), [PROMPT - 1])])
+            last.append(int(ops.argmax(logits).cpu()[0]))
+
+        def one():
+            logits = eng.step([(r, [t], [0]) for r, t in zip(ids, last)])
+            last[:] = ops.argmax(logits).cpu().tolist()
+        for _ in range(warmup):
+            one()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            one()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        for r in ids:
+            eng.release(r)
+        return dt
+
+    dt = decode(args.batch, args.steps, args.warmup)
+    ms_step = dt / args.steps * 1e3
+    value = args.batch * args.steps / dt
+    print(f"[bench] decode batch {args.batch}: {ms_step:.3f} ms/step", file=sys.stderr, flush=True)
+    mean_ctx = PROMPT + args.warmup + (args.steps + 1) / 2.0
+    nbytes = decode_bytes(shape, elem, args.batch, mean_ctx)
+    achieved = nbytes / (dt / args.steps) / 1e9
+    points = {}
+    if not args.no_points:
+        for b in (1, 64):
+            k = min(args.steps, 32)
+            d = decode(b, k, min(args.warmup, 4))
+            points[f"decode_b{b}"] = round(b * k / d, 1)
+            print(f"[bench] decode batch {b}: {d / k * 1e3:.3f} ms/step", file=sys.stderr, flush=True)
+    flops = prefill_flops(shape, PROMPT)
+    line = {
+        "metric": "decode tok/s at batch 8 (Qwen2.5-7B shape, 2048-token prompts)" if args.batch == 8
+        else f"decode tok/s at batch {args.batch} (Qwen2.5-7B shape, 2048-token prompts)",
+        "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": short, "data": "synthetic",
+        "config": {"model": "Qwen2.5-7B shape, random weights", "num_hidden_layers": layers_of_shape,
+                   "layers_run": shape["num_hidden_layers"], "hidden_size": shape["hidden_size"],
+                   "num_attention_heads": shape["num_attention_heads"],
+                   "num_key_value_heads": shape["num_key_value_heads"], "head_dim": shape["head_dim"],
+                   "intermediate_size": shape["intermediate_size"], "vocab_size": shape["vocab_size"],
+                   "tie_word_embeddings": False, "global_batch": args.batch, "seq_len": PROMPT + NEW,
+                   "prompt_len": PROMPT, "new_tokens": NEW, "page_size": PAGE, "parallelism": "none"},
+        "prefill": {"value": round(PROMPT / pre_s, 1), "tokens": PROMPT, "ms": round(pre_s * 1e3, 3),
+                    "frac": round(flops / pre_s / FLOP_PEAK[short], 4)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                     "frac": round(achieved * 1e9 / HBM_PEAK, 4)},
+        "points": points,
+    }
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

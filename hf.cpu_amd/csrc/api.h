@@ -22,9 +22,12 @@ int hfa_rmsnorm(const float* x, const float* w, void* out, int out_dtype, const 
 
 // out[m, n] (+)= sum_k a[m, k] * w[n, k] + bias[n].  a: [M, K] row stride lda; w: [N, K] row
 // stride ldw; out row stride ldo. `accumulate` adds into fp32 `out` (the residual sum).
-// (src/model.c:408-424)
+// bf16 operands with K and the row strides multiples of 8 run on the matrix cores (K split over
+// `workspace` for small M); everything else, and everything when `force_plain`, runs the plain
+// fp32 multiply-add kernel. (src/model.c:408-424)
 int hfa_gemm(const void* a, int a_dtype, int lda, const void* w, int w_dtype, int ldw, const float* bias,
-             void* out, int out_dtype, int ldo, int accumulate, int M, int N, int K, hipStream_t stream);
+             void* out, int out_dtype, int ldo, int accumulate, int M, int N, int K, void* workspace,
+             size_t workspace_bytes, int force_plain, hipStream_t stream);
 
 // Rotary position encoding on the q (and k) heads inside qkv rows [q | k | v], split-half
 // pairing, and the store of k (rotated) and v into cache rows slot_map[t] (src/model.c:468-493,

@@ -4,8 +4,8 @@
 #include "gemm_internal.h"
 
 extern "C" int hfa_gemm(const void* a, int a_dtype, int lda, const void* w, int w_dtype, int ldw, const float* bias,
-                        void* out, int out_dtype, int ldo, int accumulate, int M, int N, int K,
-                        hipStream_t stream) {
+                        void* out, int out_dtype, int ldo, int accumulate, int M, int N, int K, void* workspace,
+                        size_t workspace_bytes, int force_plain, hipStream_t stream) {
     HFA_REQUIRE(M > 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
     HFA_REQUIRE(lda >= K && ldw >= K && ldo >= N, "gemm: a row stride is smaller than its row (lda=%d ldw=%d K=%d ldo=%d N=%d)",
                 lda, ldw, K, ldo, N);
@@ -14,5 +14,6 @@ extern "C" int hfa_gemm(const void* a, int a_dtype, int lda, const void* w, int 
                 "gemm: unknown dtype (a=%d w=%d out=%d)", a_dtype, w_dtype, out_dtype);
     HFA_REQUIRE(!accumulate || out_dtype == HFA_F32, "gemm: accumulation needs an fp32 output");
     GemmArgs g = {a, a_dtype, lda, w, w_dtype, ldw, bias, out, out_dtype, ldo, accumulate, M, N, K, stream};
+    if (!force_plain && gemm_mfma_supports(g)) return gemm_mfma_launch(g, workspace, workspace_bytes);
     return gemm_generic_launch(g);
 }

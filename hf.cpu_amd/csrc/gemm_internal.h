@@ -15,3 +15,8 @@ struct GemmArgs {
 
 // Any dtype mix, any size: fp32 multiply-add over K in ascending order for every output.
 int gemm_generic_launch(const GemmArgs& g);
+
+// bf16 x bf16 on the matrix cores (K and both row strides multiples of 8, 16-byte aligned bases).
+// `workspace` holds the partial sums when K is split for small M; without one K is not split.
+bool gemm_mfma_supports(const GemmArgs& g);
+int gemm_mfma_launch(const GemmArgs& g, void* workspace, size_t workspace_bytes);

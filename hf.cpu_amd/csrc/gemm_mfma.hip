@@ -1,0 +1,260 @@
+// bf16 matrix product on the matrix cores: out[m, n] = sum_k a[m, k] * w[n, k], fp32 accumulation.
+//
+// Both operands are K-contiguous, which is what v_mfma_f32_32x32x16_bf16 wants: a lane supplies
+// 8 consecutive k of one row of A (rows -> output rows) and of one row of W (rows -> output
+// columns), so every operand fragment is one 16-byte LDS read and output columns lie along
+// lanes (coalesced stores). A block of WM x WN waves owns a BM x BN output tile and walks K in
+// steps of BK through two LDS stages: the next tile travels global -> registers while the
+// current one is multiplied, then registers -> LDS, one barrier per step. LDS rows are padded
+// by 8 elements, which makes the 16-byte fragment reads conflict-free.
+//
+// Block ids are dealt round-robin to the 8 XCDs by the hardware; the kernel undoes that so
+// that each XCD works on a contiguous run of tiles, and walks tiles in groups of 8 rows of
+// tiles, so the tiles resident on an XCD at one time share operand panels in its L2.
+//
+// Small M (decode) is bandwidth-bound and has few output tiles: K is split over blockIdx.z,
+// partial sums go to a workspace and a second kernel adds them in a fixed order and applies
+// bias and the output mode. Nothing is accumulated with atomics: results are reproducible.
+#include "common.h"
+#include "gemm_internal.h"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+#define N_XCD 8
+#define GROUP_M 8
+#define OUT_BF16 0
+#define OUT_F32 1
+#define OUT_ACC 2
+#define OUT_PARTIAL 3
+
+template <int BM, int BN, int BK, int WM, int WN>
+struct MfmaCfg {
+    static constexpr int NT = WM * WN * WAVE;
+    static constexpr int STRIDE = BK + 8;                    // LDS row stride in elements
+    static constexpr int STAGE = (BM + BN) * STRIDE;         // elements per stage
+    static constexpr int SMEM = 2 * STAGE * 2;               // bytes
+    static constexpr int CPR = BK / 8;                       // 16-byte chunks per tile row
+    static constexpr int A_CH = BM * CPR / NT;
+    static constexpr int W_CH = BN * CPR / NT;
+    static constexpr int TM = BM / WM, TN = BN / WN;         // per wave
+    static constexpr int FM = TM / 32, FN = TN / 32;
+    static_assert(BM * CPR % NT == 0 && BN * CPR % NT == 0, "tile rows must spread evenly over the threads");
+    static_assert(TM % 32 == 0 && TN % 32 == 0 && BK % 16 == 0, "wave tiles are made of 32x32x16 products");
+};
+
+template <int BM, int BN, int BK, int WM, int WN, int MODE>
+__global__ __launch_bounds__(WM* WN* WAVE) void gemm_mfma_kernel(
+    const uint16_t* __restrict__ A, int lda, const uint16_t* __restrict__ W, int ldw,
+    const float* __restrict__ bias, void* __restrict__ out, int ldo, int M, int N, int K, int k_per_split,
+    int tiles_m, int tiles_n) {
+    using C = MfmaCfg<BM, BN, BK, WM, WN>;
+    extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
+    const int tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
+    const int wm = wave / WN, wn = wave % WN;
+
+    // ---- which tile: undo the round-robin over XCDs, then grouped order ----
+    const int n_tiles = tiles_m * tiles_n;
+    int pid = blockIdx.x;
+    {
+        const int per = n_tiles / N_XCD, rem = n_tiles % N_XCD, x = pid % N_XCD, q = pid / N_XCD;
+        pid = x * per + (x < rem ? x : rem) + q;             // XCD x owns a contiguous run of tiles
+    }
+    const int in_group = GROUP_M * tiles_n;
+    const int group = pid / in_group, first_m = group * GROUP_M;
+    const int gsize = tiles_m - first_m < GROUP_M ? tiles_m - first_m : GROUP_M;
+    const int tm = first_m + (pid % in_group) % gsize, tn = (pid % in_group) / gsize;
+    const int m0 = tm * BM, n0 = tn * BN;
+    const int kbeg = blockIdx.z * k_per_split;
+    const int kend = kbeg + k_per_split < K ? kbeg + k_per_split : K;
+
+    floatx16 acc[C::FM][C::FN];
+#pragma unroll
+    for (int i = 0; i < C::FM; i++)
+#pragma unroll
+        for (int j = 0; j < C::FN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+
+    uint4 ra[C::A_CH], rw[C::W_CH];
+    auto gload = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < C::A_CH; i++) {
+            const int c = tid + i * C::NT, row = c / C::CPR, kk = k0 + (c % C::CPR) * 8;
+            int gr = m0 + row;
+            gr = gr < M ? gr : M - 1;                        // rows past the edge repeat the last one
+            ra[i] = kk < kend ? *reinterpret_cast<const uint4*>(A + (size_t)gr * lda + kk) : make_uint4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < C::W_CH; i++) {
+            const int c = tid + i * C::NT, row = c / C::CPR, kk = k0 + (c % C::CPR) * 8;
+            int gr = n0 + row;
+            gr = gr < N ? gr : N - 1;
+            rw[i] = kk < kend ? *reinterpret_cast<const uint4*>(W + (size_t)gr * ldw + kk) : make_uint4(0, 0, 0, 0);
+        }
+    };
+    auto sstore = [&](int stage) {
+        uint16_t* sa = smem + stage * C::STAGE;
+        uint16_t* sw = sa + BM * C::STRIDE;
+#pragma unroll
+        for (int i = 0; i < C::A_CH; i++) {
+            const int c = tid + i * C::NT, row = c / C::CPR, kc = c % C::CPR;
+            *reinterpret_cast<uint4*>(sa + row * C::STRIDE + kc * 8) = ra[i];
+        }
+#pragma unroll
+        for (int i = 0; i < C::W_CH; i++) {
+            const int c = tid + i * C::NT, row = c / C::CPR, kc = c % C::CPR;
+            *reinterpret_cast<uint4*>(sw + row * C::STRIDE + kc * 8) = rw[i];
+        }
+    };
+
+    gload(kbeg);
+    sstore(0);
+    __syncthreads();
+    int cur = 0;
+    for (int k0 = kbeg; k0 < kend; k0 += BK) {
+        const bool more = k0 + BK < kend;
+        if (more) gload(k0 + BK);
+        const uint16_t* sa = smem + cur * C::STAGE + (wm * C::TM + (lane & 31)) * C::STRIDE + (lane >> 5) * 8;
+        const uint16_t* sw = smem + cur * C::STAGE + (BM + wn * C::TN + (lane & 31)) * C::STRIDE + (lane >> 5) * 8;
+#pragma unroll
+        for (int kk = 0; kk < BK; kk += 16) {
+            bf16x8 fa[C::FM], fw[C::FN];
+#pragma unroll
+            for (int i = 0; i < C::FM; i++) fa[i] = *reinterpret_cast<const bf16x8*>(sa + i * 32 * C::STRIDE + kk);
+#pragma unroll
+            for (int j = 0; j < C::FN; j++) fw[j] = *reinterpret_cast<const bf16x8*>(sw + j * 32 * C::STRIDE + kk);
+#pragma unroll
+            for (int i = 0; i < C::FM; i++)
+#pragma unroll
+                for (int j = 0; j < C::FN; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fw[j], acc[i][j], 0, 0, 0);
+        }
+        if (more) sstore(cur ^ 1);
+        __syncthreads();
+        cur ^= 1;
+    }
+
+    // ---- epilogue: element r of a lane is row 8 * (r / 4) + 4 * (lane / 32) + r % 4, column lane % 32 ----
+#pragma unroll
+    for (int i = 0; i < C::FM; i++) {
+#pragma unroll
+        for (int j = 0; j < C::FN; j++) {
+            const int col = n0 + wn * C::TN + j * 32 + (lane & 31);
+            if (col >= N) continue;
+            const float b = (MODE != OUT_PARTIAL && bias) ? bias[col] : 0.f;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int row = m0 + wm * C::TM + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
+                if (row >= M) continue;
+                const float v = acc[i][j][r] + b;
+                if (MODE == OUT_BF16) {
+                    reinterpret_cast<uint16_t*>(out)[(size_t)row * ldo + col] = bf16_bits(v);
+                } else if (MODE == OUT_F32) {
+                    reinterpret_cast<float*>(out)[(size_t)row * ldo + col] = v;
+                } else if (MODE == OUT_ACC) {
+                    float* dst = reinterpret_cast<float*>(out) + (size_t)row * ldo + col;
+                    *dst += v;
+                } else {
+                    reinterpret_cast<float*>(out)[((size_t)blockIdx.z * M + row) * N + col] = v;
+                }
+            }
+        }
+    }
+}
+
+// Sum of the K splits in ascending order, then bias and the output mode.
+template <int MODE>
+__global__ void gemm_finish_kernel(const float* __restrict__ partial, int splits, const float* __restrict__ bias,
+                                   void* __restrict__ out, int ldo, int M, int N) {
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (size_t)M * N) return;
+    const int row = (int)(idx / N), col = (int)(idx % N);
+    float v = 0.f;
+    for (int s = 0; s < splits; s++) v += partial[(size_t)s * M * N + idx];
+    if (bias) v += bias[col];
+    if (MODE == OUT_BF16)
+        reinterpret_cast<uint16_t*>(out)[(size_t)row * ldo + col] = bf16_bits(v);
+    else if (MODE == OUT_F32)
+        reinterpret_cast<float*>(out)[(size_t)row * ldo + col] = v;
+    else
+        reinterpret_cast<float*>(out)[(size_t)row * ldo + col] += v;
+}
+
+template <int BM, int BN, int BK, int WM, int WN, int MODE>
+static int launch_cfg(const GemmArgs& g, void* out, int splits, int k_per_split) {
+    using C = MfmaCfg<BM, BN, BK, WM, WN>;
+    auto kernel = gemm_mfma_kernel<BM, BN, BK, WM, WN, MODE>;
+    static bool configured = false;
+    if (!configured) {
+        hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM);
+        if (e != hipSuccess) {
+            hfa_set_error("gemm_mfma: cannot reserve %d bytes of LDS: %s", C::SMEM, hipGetErrorString(e));
+            return 2;
+        }
+        configured = true;
+    }
+    const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
+    dim3 grid(tiles_m * tiles_n, 1, splits);
+    kernel<<<grid, C::NT, C::SMEM, g.stream>>>((const uint16_t*)g.a, g.lda, (const uint16_t*)g.w, g.ldw, g.bias, out,
+                                              g.ldo, g.M, g.N, g.K, k_per_split, tiles_m, tiles_n);
+    HFA_LAUNCH_CHECK("gemm_mfma");
+    return 0;
+}
+
+template <int BM, int BN, int BK, int WM, int WN>
+static int launch_mode(const GemmArgs& g, int mode, void* out, int splits, int k_per_split) {
+    switch (mode) {
+        case OUT_BF16: return launch_cfg<BM, BN, BK, WM, WN, OUT_BF16>(g, out, splits, k_per_split);
+        case OUT_F32: return launch_cfg<BM, BN, BK, WM, WN, OUT_F32>(g, out, splits, k_per_split);
+        case OUT_ACC: return launch_cfg<BM, BN, BK, WM, WN, OUT_ACC>(g, out, splits, k_per_split);
+        default: return launch_cfg<BM, BN, BK, WM, WN, OUT_PARTIAL>(g, out, splits, k_per_split);
+    }
+}
+
+bool gemm_mfma_supports(const GemmArgs& g) {
+    return g.a_dtype == HFA_BF16 && g.w_dtype == HFA_BF16 && g.K % 8 == 0 && g.lda % 8 == 0 && g.ldw % 8 == 0 &&
+           ((uintptr_t)g.a & 15) == 0 && ((uintptr_t)g.w & 15) == 0;
+}
+
+int gemm_mfma_launch(const GemmArgs& g, void* workspace, size_t workspace_bytes) {
+    const int mode = g.accumulate ? OUT_ACC : (g.out_dtype == HFA_BF16 ? OUT_BF16 : OUT_F32);
+    const int BK = 64;
+    const int BM = g.M > 64 ? 128 : (g.M > 32 ? 64 : 32), BN = 128;
+    const int tiles = ((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN);
+    const int k_tiles = (g.K + BK - 1) / BK;
+    // Few tiles and a long K: split K so that the machine is full; every split keeps at least 4 steps.
+    int splits = 1;
+    if (g.M <= 64 && tiles < 512) {
+        splits = (512 + tiles - 1) / tiles;
+        const int most = k_tiles / 4 > 0 ? k_tiles / 4 : 1;
+        if (splits > most) splits = most;
+        const size_t per_split = (size_t)g.M * g.N * sizeof(float);
+        if (workspace == nullptr || per_split == 0) splits = 1;
+        else if ((size_t)splits * per_split > workspace_bytes) splits = (int)(workspace_bytes / per_split);
+        if (splits < 1) splits = 1;
+    }
+    int k_per_split = ((k_tiles + splits - 1) / splits) * BK;
+    splits = (g.K + k_per_split - 1) / k_per_split;
+    const int kmode = splits > 1 ? OUT_PARTIAL : mode;
+    void* kout = splits > 1 ? workspace : g.out;
+    int rc;
+    if (BM == 128)
+        rc = launch_mode<128, 128, 64, 2, 2>(g, kmode, kout, splits, k_per_split);
+    else if (BM == 64)
+        rc = launch_mode<64, 128, 64, 2, 2>(g, kmode, kout, splits, k_per_split);
+    else
+        rc = launch_mode<32, 128, 64, 1, 4>(g, kmode, kout, splits, k_per_split);
+    if (rc || splits == 1) return rc;
+    const size_t total = (size_t)g.M * g.N;
+    const int blocks = (int)((total + 255) / 256);
+    const float* part = (const float*)workspace;
+    if (mode == OUT_BF16)
+        gemm_finish_kernel<OUT_BF16><<<blocks, 256, 0, g.stream>>>(part, splits, g.bias, g.out, g.ldo, g.M, g.N);
+    else if (mode == OUT_F32)
+        gemm_finish_kernel<OUT_F32><<<blocks, 256, 0, g.stream>>>(part, splits, g.bias, g.out, g.ldo, g.M, g.N);
+    else
+        gemm_finish_kernel<OUT_ACC><<<blocks, 256, 0, g.stream>>>(part, splits, g.bias, g.out, g.ldo, g.M, g.N);
+    HFA_LAUNCH_CHECK("gemm_finish");
+    return 0;
+}

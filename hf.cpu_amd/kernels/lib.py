@@ -5,7 +5,7 @@ built or loaded the error is raised to the caller.
 """
 import ctypes
 import threading
-from ctypes import c_char_p, c_float, c_int, c_void_p
+from ctypes import c_char_p, c_float, c_int, c_size_t, c_void_p
 
 from . import build as _build
 
@@ -16,7 +16,7 @@ P, I, F = c_void_p, c_int, c_float
 _SIGNATURES = {
     "hfa_embed": [P, I, P, P, I, I, I, P],
     "hfa_rmsnorm": [P, P, P, I, P, I, I, F, P],
-    "hfa_gemm": [P, I, I, P, I, I, P, P, I, I, I, I, I, I, P],
+    "hfa_gemm": [P, I, I, P, I, I, P, P, I, I, I, I, I, I, P, c_size_t, I, P],
     "hfa_rope_store": [P, I, I, P, P, I, I, I, I, P, P, P, I, P],
     "hfa_paged_attention": [P, I, I, P, P, I, P, I, P, P, P, I, I, I, I, I, I, I, F, P],
     "hfa_swiglu": [P, P, I, I, I, P],

@@ -11,6 +11,7 @@ from ..status import EINVAL, ENOTSUP, EngineError, fail
 from .lib import last_error, library
 
 F32, BF16 = 0, 1
+WORKSPACE_BYTES = 64 << 20           # partial sums of matrix products whose K is split
 _CODE = {torch.float32: F32, torch.bfloat16: BF16}
 
 
@@ -44,6 +45,8 @@ class Ops:
         self.act_dtype = act_dtype
         self.lib = library()
         self._scratch = {}
+        self.workspace = torch.empty(WORKSPACE_BYTES, dtype=torch.uint8, device=self.device)
+        self.force_plain_gemm = False        # tests set this to compare the matrix-core path with the plain one
 
     # ---- plumbing ----------------------------------------------------------
     def _stream(self):
@@ -98,7 +101,8 @@ class Ops:
             fail(EINVAL, "gemm: the bias must be contiguous fp32 with one value per output column")
         self._check(self.lib.hfa_gemm(a.data_ptr(), _code(a), lda, w.data_ptr(), _code(w), ldw,
                                       None if bias is None else bias.data_ptr(), out.data_ptr(), _code(out), ldo,
-                                      1 if accumulate else 0, M, N, K, self._stream()))
+                                      1 if accumulate else 0, M, N, K, self.workspace.data_ptr(),
+                                      self.workspace.numel(), 1 if self.force_plain_gemm else 0, self._stream()))
 
     def rope_store(self, qkv, positions, inv_freq, rot_dim, n_heads, n_kv_heads, head_dim, cache, slot_map):
         """Rotates q (and k) inside ``qkv`` and, if ``slot_map`` is given, stores k and v

@@ -94,6 +94,41 @@ def test_gemm(ops32, adt, wdt, odt, M, N, K):
         assert float(wide[:, N:].abs().max()) == 0.0
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 256, 512), (8, 4608, 3584), (8, 3584, 18944), (33, 200, 1000),
+                                   (64, 1000, 4096), (65, 129, 72), (200, 333, 264), (500, 1100, 1024),
+                                   (2048, 512, 3584)])
+def test_gemm_on_matrix_cores(ops16, M, N, K):
+    """bf16 x bf16 with K a multiple of 8 runs on the matrix cores (K split for small M): against
+    fp64 on the rounded operands, against the plain kernel on the same operands, in the three
+    output modes, with operands that are views of wider buffers."""
+    rng = np.random.default_rng(M + N + K)
+    a = rng.standard_normal((M, K)).astype(np.float32)
+    w = (rng.standard_normal((N, K)) / math.sqrt(K)).astype(np.float32)
+    b = rng.standard_normal(N).astype(np.float32)
+    want = rounded(a, torch.bfloat16) @ rounded(w, torch.bfloat16).T
+    wide_a = torch.zeros((M, K + 16), dtype=torch.bfloat16, device="cuda")
+    wide_a[:, 8:K + 8] = dev(a, torch.bfloat16)
+    ta, tw, tb = wide_a[:, 8:K + 8], dev(w, torch.bfloat16), dev(b)
+    out = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    ops16.gemm(ta, tw, out, bias=tb)
+    scale = max(1.0, float(np.max(np.abs(want))))
+    assert np.max(np.abs(out.cpu().numpy() - (want + b))) <= 2e-5 * scale
+    plain_out = torch.empty_like(out)
+    ops16.force_plain_gemm = True
+    try:
+        ops16.gemm(ta, tw, plain_out, bias=tb)
+    finally:
+        ops16.force_plain_gemm = False
+    assert float((out - plain_out).abs().max()) <= 2e-5 * scale
+    o16 = torch.empty((M, N + 8), dtype=torch.bfloat16, device="cuda")[:, :N]
+    ops16.gemm(ta, tw, o16)
+    assert np.max(np.abs(o16.float().cpu().numpy() - want)) <= 0.01 * scale
+    res = rng.standard_normal((M, N)).astype(np.float32)
+    acc = dev(res)
+    ops16.gemm(ta, tw, acc, accumulate=True)
+    assert np.max(np.abs(acc.cpu().numpy() - (want + res))) <= 2e-5 * scale
+
+
 def test_gemm_matches_library_product(ops32):
     """The kernel against the library's fp32 matrix product on the same operands."""
     torch.manual_seed(0)

@@ -6,8 +6,11 @@ import torch
 
 @dataclass
 class PagedView:
-    """What a mixer sees of its cache: row ``page * page_tokens + offset`` of ``k`` and
-    ``v`` belongs to one token; ``group`` names the block table to use."""
+    """What a mixer sees of its cache: row ``page * page_tokens + offset`` of ``k`` belongs to
+    one token; ``v`` has the same size but holds each page transposed (``[page][column][offset]``,
+    so that the attention kernels read the keys of one value column contiguously); ``group``
+    names the block table to use. The memory starts as zeros and only ever holds values that
+    were stored, so a masked read of a stale row never meets a NaN."""
     group: int
     k: torch.Tensor            # [n_pages * page_tokens, k_width]
     v: torch.Tensor            # [n_pages * page_tokens, v_width]
@@ -33,8 +36,8 @@ class CacheStorage:
             rows = pool.n_pages * manager.page_tokens
             for e in g.entries:
                 self.views[e] = PagedView(g.index,
-                                          torch.empty((rows, g.k_width), dtype=dtype, device=device),
-                                          torch.empty((rows, g.v_width), dtype=dtype, device=device),
+                                          torch.zeros((rows, g.k_width), dtype=dtype, device=device),
+                                          torch.zeros((rows, g.v_width), dtype=dtype, device=device),
                                           manager.page_tokens, g.window)
         for e, n_floats in manager.state_entries.items():
             self.views[e] = StateView(torch.zeros((manager.n_slots, n_floats), dtype=torch.float32, device=device))

@@ -32,19 +32,28 @@ int hfa_gemm(const void* a, int a_dtype, int lda, const void* w, int w_dtype, in
 // Rotary position encoding on the q (and k) heads inside qkv rows [q | k | v], split-half
 // pairing, and the store of k (rotated) and v into cache rows slot_map[t] (src/model.c:468-493,
 // 587-600). rot_dim 0: no rotation. n_kv_heads 0: the rows hold q only, nothing is stored.
+// Cache layout: row r = page * page_tokens + offset. Keys: k_cache[r * width + c]. Values lie
+// transposed inside their page, so that the keys of one value column are contiguous:
+// v_cache[page * page_tokens * width + c * page_tokens + offset].
 int hfa_rope_store(void* qkv, int dtype, int ld, const int* positions, const float* inv_freq, int rot_dim,
                    int n_heads, int n_kv_heads, int head_dim, void* k_cache, void* v_cache,
-                   const int* slot_map, int n_tokens, hipStream_t stream);
+                   const int* slot_map, int page_tokens, int n_tokens, hipStream_t stream);
 
 // Softmax attention of each token's query heads over its request's cached keys and values
 // (src/model.c:499-528). Key j of the request in slot s lies in cache row
 // block_table[s, j / page_tokens] * page_tokens + j % page_tokens. A key is visible to the
-// query at position p iff j <= p and (window == 0 or p - j < window).
+// query at position p iff j <= p and (window == 0 or p - j < window). q_start[n_seqs + 1] gives
+// each request's run of tokens (consecutive positions of one slot); max_q_len and max_seq_len
+// bound the runs and the positions. bf16 with head_dim a multiple of 32, page_tokens a multiple
+// of 4 and at most 32 query heads per key/value head runs on the matrix cores, the key range
+// split over `workspace` when there are few queries; everything else, and everything when
+// `force_plain`, runs the plain kernel.
 int hfa_paged_attention(const void* q, int dtype, int ldq, const void* k_cache, const void* v_cache,
                         int kv_width, const int* block_table, int max_blocks, const int* token_slot,
-                        const int* positions, void* out, int ldo, int n_tokens, int n_heads,
-                        int n_kv_heads, int head_dim, int page_tokens, int window, float scale,
-                        hipStream_t stream);
+                        const int* positions, const int* q_start, int n_seqs, int max_q_len, int max_seq_len,
+                        void* out, int ldo, int n_tokens, int n_heads, int n_kv_heads, int head_dim,
+                        int page_tokens, int window, float scale, void* workspace, size_t workspace_bytes,
+                        int force_plain, hipStream_t stream);
 
 // out[t, i] = silu(gate_up[t, i]) * gate_up[t, width + i].  (src/model.c:532-538)
 int hfa_swiglu(const void* gate_up, void* out, int dtype, int n_tokens, int width, hipStream_t stream);

@@ -5,11 +5,9 @@
 // so a token's result depends on its request's cache alone, never on the rest of the batch.
 #include "api.h"
 #include "common.h"
+#include "attention_internal.h"
 
 #define ATT_MAX_D 256
-
-template <typename T> struct Vec8;
-template <> struct Vec8<bf16> { uint4 v; };
 
 __device__ __forceinline__ float dot_row(const float* __restrict__ q_s, const bf16* __restrict__ kp, int D) {
     float dot = 0.f;
@@ -89,11 +87,14 @@ __global__ __launch_bounds__(WAVE) void attn_generic_kernel(
         for (int i = 0; i < ATT_MAX_D / WAVE; i++) acc[i] *= corr;
         for (int jj = first; jj <= last; jj++) {
             const float pj = p_s[jj];
-            const T* vp = vc + (size_t)row_s[jj] * kvw + kvh * D;
+            // values lie transposed inside their page: [page][column][token]
+            const int vr = row_s[jj];
+            const T* vp = vc + (size_t)(vr / page_tokens) * page_tokens * kvw + (size_t)(kvh * D) * page_tokens +
+                          vr % page_tokens;
 #pragma unroll
             for (int i = 0; i < ATT_MAX_D / WAVE; i++) {
                 const int d = lane + WAVE * i;
-                if (d < D) acc[i] = fmaf(pj, to_f32(vp[d]), acc[i]);
+                if (d < D) acc[i] = fmaf(pj, to_f32(vp[(size_t)d * page_tokens]), acc[i]);
             }
         }
         __syncthreads();
@@ -128,9 +129,10 @@ int attn_generic_launch(const void* q, int dtype, int ldq, const void* k_cache, 
 
 extern "C" int hfa_paged_attention(const void* q, int dtype, int ldq, const void* k_cache, const void* v_cache,
                                    int kv_width, const int* block_table, int max_blocks, const int* token_slot,
-                                   const int* positions, void* out, int ldo, int n_tokens, int n_heads,
-                                   int n_kv_heads, int head_dim, int page_tokens, int window, float scale,
-                                   hipStream_t stream) {
+                                   const int* positions, const int* q_start, int n_seqs, int max_q_len,
+                                   int max_seq_len, void* out, int ldo, int n_tokens, int n_heads, int n_kv_heads,
+                                   int head_dim, int page_tokens, int window, float scale, void* workspace,
+                                   size_t workspace_bytes, int force_plain, hipStream_t stream) {
     HFA_REQUIRE(n_tokens > 0 && n_heads > 0 && n_kv_heads > 0 && head_dim > 0 && page_tokens > 0 && max_blocks > 0,
                 "paged_attention: bad sizes");
     HFA_REQUIRE(n_heads % n_kv_heads == 0, "paged_attention: %d heads are not a multiple of %d key/value heads",
@@ -139,6 +141,10 @@ extern "C" int hfa_paged_attention(const void* q, int dtype, int ldq, const void
                 "paged_attention: a row stride is smaller than its row");
     HFA_REQUIRE(window >= 0, "paged_attention: negative window");
     HFA_REQUIRE(dtype == HFA_F32 || dtype == HFA_BF16, "paged_attention: unknown dtype %d", dtype);
+    AttnArgs a = {q, ldq, k_cache, v_cache, kv_width, block_table, max_blocks, token_slot, positions, q_start,
+                  n_seqs, max_q_len, max_seq_len, out, ldo, n_tokens, n_heads, n_kv_heads, head_dim, page_tokens,
+                  window, scale, workspace, workspace_bytes, stream};
+    if (!force_plain && dtype == HFA_BF16 && attn_mfma_supports(a)) return attn_mfma_launch(a);
     return attn_generic_launch(q, dtype, ldq, k_cache, v_cache, kv_width, block_table, max_blocks, token_slot,
                                positions, out, ldo, n_tokens, n_heads, n_kv_heads, head_dim, page_tokens, window,
                                scale, stream);

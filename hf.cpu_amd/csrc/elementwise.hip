@@ -83,7 +83,7 @@ template <typename T>
 __global__ void rope_store_kernel(T* __restrict__ qkv, int ld, const int* __restrict__ positions,
                                   const float* __restrict__ inv_freq, int rot_dim, int H, int G, int D,
                                   T* __restrict__ k_cache, T* __restrict__ v_cache,
-                                  const int* __restrict__ slot_map) {
+                                  const int* __restrict__ slot_map, int page_tokens) {
     __shared__ float cs[ROPE_MAX_HALF], sn[ROPE_MAX_HALF];
     const int t = blockIdx.x;
     const int half = rot_dim / 2;
@@ -126,7 +126,8 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, int ld, const int* __rest
         return;
     }
     T* kdst = k_cache + (size_t)slot * (G * D);
-    T* vdst = v_cache + (size_t)slot * (G * D);
+    // values lie transposed inside their page: element c of the token at offset o is at c * page_tokens + o
+    T* vdst = v_cache + (size_t)(slot / page_tokens) * page_tokens * (G * D) + slot % page_tokens;
     for (int it = threadIdx.x; it < G * half; it += blockDim.x) {
         const int g = it / half, i = it - g * half;
         const T* p = krow + g * D;
@@ -139,12 +140,12 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, int ld, const int* __rest
         const int g = it / rest, i = rot_dim + (it - g * rest);
         kdst[g * D + i] = krow[g * D + i];
     }
-    for (int it = threadIdx.x; it < G * D; it += blockDim.x) vdst[it] = vrow[it];
+    for (int it = threadIdx.x; it < G * D; it += blockDim.x) vdst[(size_t)it * page_tokens] = vrow[it];
 }
 
 extern "C" int hfa_rope_store(void* qkv, int dtype, int ld, const int* positions, const float* inv_freq, int rot_dim,
                               int n_heads, int n_kv_heads, int head_dim, void* k_cache, void* v_cache,
-                              const int* slot_map, int n_tokens, hipStream_t stream) {
+                              const int* slot_map, int page_tokens, int n_tokens, hipStream_t stream) {
     HFA_REQUIRE(n_tokens > 0 && n_heads > 0 && n_kv_heads >= 0 && head_dim > 0, "rope_store: bad sizes");
     HFA_REQUIRE(rot_dim >= 0 && rot_dim % 2 == 0 && rot_dim <= head_dim,
                 "rope_store: rot_dim %d must be even and at most head_dim %d", rot_dim, head_dim);
@@ -152,16 +153,17 @@ extern "C" int hfa_rope_store(void* qkv, int dtype, int ld, const int* positions
                 2 * ROPE_MAX_HALF);
     HFA_REQUIRE(rot_dim == 0 || (positions && inv_freq), "rope_store: positions and inv_freq are needed");
     HFA_REQUIRE(ld >= (n_heads + 2 * n_kv_heads) * head_dim, "rope_store: row stride %d is too small", ld);
-    HFA_REQUIRE(n_kv_heads == 0 || !slot_map || (k_cache && v_cache), "rope_store: no cache to store into");
+    HFA_REQUIRE(n_kv_heads == 0 || !slot_map || (k_cache && v_cache && page_tokens > 0),
+                "rope_store: no cache to store into");
     HFA_REQUIRE(dtype == HFA_F32 || dtype == HFA_BF16, "rope_store: unknown dtype %d", dtype);
     if (dtype == HFA_F32)
         rope_store_kernel<float><<<n_tokens, 256, 0, stream>>>((float*)qkv, ld, positions, inv_freq, rot_dim, n_heads,
                                                                n_kv_heads, head_dim, (float*)k_cache,
-                                                               (float*)v_cache, slot_map);
+                                                               (float*)v_cache, slot_map, page_tokens);
     else
         rope_store_kernel<bf16><<<n_tokens, 256, 0, stream>>>((bf16*)qkv, ld, positions, inv_freq, rot_dim, n_heads,
                                                               n_kv_heads, head_dim, (bf16*)k_cache, (bf16*)v_cache,
-                                                              slot_map);
+                                                              slot_map, page_tokens);
     HFA_LAUNCH_CHECK("rope_store");
     return 0;
 }

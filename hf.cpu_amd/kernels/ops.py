@@ -46,7 +46,8 @@ class Ops:
         self.lib = library()
         self._scratch = {}
         self.workspace = torch.empty(WORKSPACE_BYTES, dtype=torch.uint8, device=self.device)
-        self.force_plain_gemm = False        # tests set this to compare the matrix-core path with the plain one
+        self.force_plain_gemm = False        # tests set these to compare the matrix-core paths with the plain ones
+        self.force_plain_attention = False
 
     # ---- plumbing ----------------------------------------------------------
     def _stream(self):
@@ -106,7 +107,8 @@ class Ops:
 
     def rope_store(self, qkv, positions, inv_freq, rot_dim, n_heads, n_kv_heads, head_dim, cache, slot_map):
         """Rotates q (and k) inside ``qkv`` and, if ``slot_map`` is given, stores k and v
-        rows into ``cache.k`` / ``cache.v`` at the rows it names."""
+        rows into ``cache.k`` / ``cache.v`` at the rows it names (values transposed inside
+        their page, see csrc/api.h)."""
         ld = _rows(qkv, "rope_store qkv")
         T = qkv.shape[0]
         if qkv.shape[1] < (n_heads + 2 * n_kv_heads) * head_dim:
@@ -122,7 +124,8 @@ class Ops:
         self._check(self.lib.hfa_rope_store(
             qkv.data_ptr(), _code(qkv), ld, None if positions is None else _ints(positions, "positions", T),
             None if inv_freq is None else inv_freq.data_ptr(), rot_dim, n_heads, n_kv_heads, head_dim,
-            k_ptr, v_ptr, None if slot_map is None else _ints(slot_map, "slot_map", T), T, self._stream()))
+            k_ptr, v_ptr, None if slot_map is None else _ints(slot_map, "slot_map", T),
+            getattr(cache, "page_tokens", 0) or 0, T, self._stream()))
 
     def paged_attention(self, q, n_heads, n_kv_heads, head_dim, cache, step, window, scale, out):
         """Attention of the first ``n_heads * head_dim`` columns of ``q`` over ``cache``."""
@@ -136,8 +139,10 @@ class Ops:
         self._check(self.lib.hfa_paged_attention(
             q.data_ptr(), _code(q), ldq, cache.k.data_ptr(), cache.v.data_ptr(), cache.k.shape[1],
             g.block_table.data_ptr(), g.block_table.shape[1], _ints(step.token_slot, "token_slot", T),
-            _ints(step.positions, "positions", T), out.data_ptr(), ldo, T, n_heads, n_kv_heads, head_dim,
-            cache.page_tokens, int(window), float(scale), self._stream()))
+            _ints(step.positions, "positions", T), _ints(step.q_start, "q_start", step.n_seqs + 1), step.n_seqs,
+            step.max_q_len, step.max_seq_len, out.data_ptr(), ldo, T, n_heads, n_kv_heads, head_dim,
+            cache.page_tokens, int(window), float(scale), self.workspace.data_ptr(), self.workspace.numel(),
+            1 if self.force_plain_attention else 0, self._stream()))
 
     def swiglu(self, gate_up, out):
         T, F2 = gate_up.shape

@@ -145,12 +145,31 @@ class FakeCache(types.SimpleNamespace):
 
 
 class FakeStep:
+    """Step inputs for a kernel alone: tokens of one request are consecutive in the batch."""
+
     def __init__(self, positions, token_slot, block_table, slot_map):
         self.positions, self.token_slot = positions, token_slot
         self._g = types.SimpleNamespace(block_table=block_table, slot_map=slot_map)
+        slots, pos = token_slot.cpu().tolist(), positions.cpu().tolist()
+        starts = [0] + [i for i in range(1, len(slots)) if slots[i] != slots[i - 1]] + [len(slots)]
+        self.q_start = ints(starts)
+        self.n_seqs = len(starts) - 1
+        self.max_q_len = max(b - a for a, b in zip(starts, starts[1:]))
+        self.max_seq_len = max(pos) + 1
 
     def group(self, i):
         return self._g
+
+
+def to_value_layout(rows, page):
+    """[n_pages * page, width] by token -> the cache's value layout: each page transposed."""
+    n, w = rows.shape
+    return np.ascontiguousarray(rows.reshape(n // page, page, w).transpose(0, 2, 1)).reshape(n, w)
+
+
+def from_value_layout(rows, page):
+    n, w = rows.shape
+    return np.ascontiguousarray(rows.reshape(n // page, w, page).transpose(0, 2, 1)).reshape(n, w)
 
 
 def paged_setup(rng, lengths, G, D, page, dtype, n_pages=None, shuffle=True):
@@ -177,6 +196,7 @@ def paged_setup(rng, lengths, G, D, page, dtype, n_pages=None, shuffle=True):
             vc[pg * page:pg * page + cnt] = v[rows].reshape(cnt, G * D)
         ks.append(k)
         vs.append(v)
+    vc = to_value_layout(vc, page)
     cache = FakeCache(group=0, k=dev(kc, dtype), v=dev(vc, dtype), page_tokens=page, window=0)
     return ks, vs, cache, ints(table)
 
@@ -211,6 +231,47 @@ def test_paged_attention(ops32, dtype, H, G, D, page, window):
     tol = 2e-5 if dtype == torch.float32 else 0.02
     err = np.max(np.abs(out.float().cpu().numpy() - want))
     assert err <= tol, f"max |diff| {err:.3e}"
+    if dtype == torch.bfloat16:          # the plain kernel on the same inputs
+        other = torch.empty_like(out)
+        ops32.force_plain_attention = True
+        try:
+            ops32.paged_attention(qpad[:, :H * D], H, G, D, cache, step, window, 1.0 / math.sqrt(D), other)
+        finally:
+            ops32.force_plain_attention = False
+        assert np.max(np.abs(other.float().cpu().numpy() - want)) <= tol
+
+
+@pytest.mark.parametrize("H,G,D,page,window,lengths,q_lens", [
+    (28, 4, 128, 16, 0, [2100, 700, 64, 1500], [1, 1, 1, 1]),          # decode: keys cut into chunks
+    (28, 4, 128, 16, 0, [600], [600]),                                   # one prompt, whole
+    (14, 2, 64, 16, 300, [1000, 333], [1, 40]),                          # window shorter than the context
+    (8, 1, 96, 8, 0, [257, 31], [9, 31]),                                # one key/value head, 8 query heads
+    (32, 1, 32, 4, 0, [70], [3]),                                        # 32 heads on one key/value head
+])
+def test_paged_attention_on_matrix_cores(ops16, H, G, D, page, window, lengths, q_lens):
+    """bf16 with head_dim a multiple of 32: long contexts (many key blocks, split into chunks when
+    there are few queries), groups of 7, 8 and 32 query heads, tiles that end inside a request."""
+    rng = np.random.default_rng(H + D + len(lengths))
+    dtype = torch.bfloat16
+    ks, vs, cache, table = paged_setup(rng, lengths, G, D, page, dtype)
+    qs, positions, slots, wants = [], [], [], []
+    for s, (n, ql) in enumerate(zip(lengths, q_lens)):
+        q_tail = rng.standard_normal((ql, H, D)).astype(np.float32)
+        q_full = np.zeros((n, H, D), np.float32)
+        q_full[n - ql:] = q_tail
+        full = plain.attention(rounded(q_full, dtype)[n - ql:] if False else rounded(q_full, dtype),
+                               rounded(ks[s], dtype), rounded(vs[s], dtype), window)
+        qs.append(q_tail)
+        wants.append(full[n - ql:])
+        positions += list(range(n - ql, n))
+        slots += [s] * ql
+    q = np.concatenate(qs).reshape(-1, H * D)
+    want = np.concatenate(wants).reshape(-1, H * D)
+    out = torch.empty((q.shape[0], H * D), dtype=dtype, device="cuda")
+    step = FakeStep(ints(positions), ints(slots), table, None)
+    ops16.paged_attention(dev(q, dtype), H, G, D, cache, step, window, 1.0 / math.sqrt(D), out)
+    err = np.max(np.abs(out.float().cpu().numpy() - want))
+    assert err <= 0.02, f"max |diff| {err:.3e}"
 
 
 def test_attention_special_cases(ops32):
@@ -241,7 +302,7 @@ def test_rope_store(ops32, dtype, H, G, D, rot):
     slot_map = [4, 0, 11, 7, 2, 9, 1, 3, 10]
     t_qkv = dev(qkv, dtype)
     cache = FakeCache(group=0, k=torch.zeros((12, G * D), dtype=dtype, device="cuda"),
-                      v=torch.zeros((12, G * D), dtype=dtype, device="cuda"))
+                      v=torch.zeros((12, G * D), dtype=dtype, device="cuda"), page_tokens=4)
     i = np.arange(rot // 2, dtype=np.float64)
     inv_freq = dev((base ** (-2.0 * i / rot)).astype(np.float32))
     ops32.rope_store(t_qkv, ints(positions), inv_freq, rot, H, G, D, cache, ints(slot_map))
@@ -255,7 +316,7 @@ def test_rope_store(ops32, dtype, H, G, D, rot):
     assert np.max(np.abs(got[:, :H * D] - q_want)) <= tol
     small = [t for t, p in enumerate(positions) if p < 100]
     assert np.max(np.abs(got[small, :H * D] - q_want[small])) <= (1e-5 if dtype == torch.float32 else 0.03)
-    kc, vc = cache.k.float().cpu().numpy(), cache.v.float().cpu().numpy()
+    kc, vc = cache.k.float().cpu().numpy(), from_value_layout(cache.v.float().cpu().numpy(), 4)
     assert np.max(np.abs(kc[slot_map] - k_want)) <= tol
     assert np.array_equal(vc[slot_map], v_want.astype(np.float32))
     assert np.array_equal(got[0, :H * D], src[0, :H * D].astype(np.float32)), "position 0 is the identity"
@@ -274,7 +335,8 @@ def test_rope_relative_position(ops32):
     dots = []
     for shift in (0, 5, 100):
         rows = torch.cat([dev(qkv), dev(qkv)])
-        cache = FakeCache(group=0, k=torch.zeros((2, D), device="cuda"), v=torch.zeros((2, D), device="cuda"))
+        cache = FakeCache(group=0, k=torch.zeros((2, D), device="cuda"), v=torch.zeros((2, D), device="cuda"),
+                          page_tokens=2)
         ops32.rope_store(rows, ints([9 + shift, 2 + shift]), inv_freq, D, H, G, D, cache, ints([0, 1]))
         dots.append(float((rows[0, :D].double() * cache.k[1].double()).sum()))
     assert abs(dots[0] - dots[1]) < 1e-4 and abs(dots[0] - dots[2]) < 1e-4

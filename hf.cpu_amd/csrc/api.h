@@ -17,17 +17,26 @@ int hfa_embed(const void* table, int table_dtype, const int* tokens, float* x, i
               int vocab, hipStream_t stream);
 
 // out[r, :] = x[rows ? rows[r] : r, :] * rsqrt(mean(x^2) + eps) * w.  (src/mathx.c:65-75)
-int hfa_rmsnorm(const float* x, const float* w, void* out, int out_dtype, const int* rows, int n_rows,
-                int width, float eps, hipStream_t stream);
+// With splits > 0 (and no rows): first x[r, :] += sum_s partial[s][r][:] + partial_bias, written
+// back: the residual sum of a matrix product that hfa_gemm deferred (src/model.c:609, 623).
+int hfa_rmsnorm(float* x, const float* w, void* out, int out_dtype, const int* rows, int n_rows, int width,
+                float eps, const float* partial, int splits, const float* partial_bias, hipStream_t stream);
 
 // out[m, n] (+)= sum_k a[m, k] * w[n, k] + bias[n].  a: [M, K] row stride lda; w: [N, K] row
 // stride ldw; out row stride ldo. `accumulate` adds into fp32 `out` (the residual sum).
 // bf16 operands with K and the row strides multiples of 8 run on the matrix cores (K split over
 // `workspace` for small M); everything else, and everything when `force_plain`, runs the plain
-// fp32 multiply-add kernel. (src/model.c:408-424)
+// fp32 multiply-add kernel. `epilogue` 1 (matrix cores only): the columns of w come in blocks of
+// 32 gate rows, 32 up rows, and out[m, f] = silu(gate) * up has N / 2 columns (src/model.c:537).
+// `defer`: if K was split, leave the partial sums ([splits][M][N] fp32 at the start of the
+// workspace) for the caller's next kernel and report the number of splits in *pending_splits.
+// (src/model.c:408-424)
 int hfa_gemm(const void* a, int a_dtype, int lda, const void* w, int w_dtype, int ldw, const float* bias,
-             void* out, int out_dtype, int ldo, int accumulate, int M, int N, int K, void* workspace,
-             size_t workspace_bytes, int force_plain, hipStream_t stream);
+             void* out, int out_dtype, int ldo, int accumulate, int epilogue, int M, int N, int K,
+             void* workspace, size_t workspace_bytes, int defer, int* pending_splits, int force_plain,
+             hipStream_t stream);
+int hfa_gemm_finish(const void* partial, int splits, const float* bias, void* out, int out_dtype, int ldo,
+                    int accumulate, int epilogue, int M, int N, hipStream_t stream);
 
 // Rotary position encoding on the q (and k) heads inside qkv rows [q | k | v], split-half
 // pairing, and the store of k (rotated) and v into cache rows slot_map[t] (src/model.c:468-493,
@@ -35,9 +44,13 @@ int hfa_gemm(const void* a, int a_dtype, int lda, const void* w, int w_dtype, in
 // Cache layout: row r = page * page_tokens + offset. Keys: k_cache[r * width + c]. Values lie
 // transposed inside their page, so that the keys of one value column are contiguous:
 // v_cache[page * page_tokens * width + c * page_tokens + offset].
+// With splits > 0 the input is not qkv but the partial sums of a deferred hfa_gemm
+// ([splits][n_tokens][(n_heads + 2 n_kv_heads) * head_dim] fp32) plus partial_bias; the rotated
+// queries are written into qkv.
 int hfa_rope_store(void* qkv, int dtype, int ld, const int* positions, const float* inv_freq, int rot_dim,
                    int n_heads, int n_kv_heads, int head_dim, void* k_cache, void* v_cache,
-                   const int* slot_map, int page_tokens, int n_tokens, hipStream_t stream);
+                   const int* slot_map, int page_tokens, int n_tokens, const float* partial, int splits,
+                   const float* partial_bias, hipStream_t stream);
 
 // Softmax attention of each token's query heads over its request's cached keys and values
 // (src/model.c:499-528). Key j of the request in slot s lies in cache row

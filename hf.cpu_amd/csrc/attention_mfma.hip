@@ -206,19 +206,29 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
 }
 
 // out[t, h, :] = sum_c o_c 2^(m_c - M) / sum_c l_c 2^(m_c - M), chunks in ascending order.
+// Lanes first share the chunks (maximum, weights, sum), then the dimensions; the loads of the
+// second loop do not depend on one another.
+#define MERGE_MAX_CHUNKS 512
 __global__ __launch_bounds__(WAVE) void attn_merge_kernel(const float* __restrict__ partial, uint16_t* __restrict__ out,
                                                           int ldo, int H, int D, int n_chunks) {
-    const int t = blockIdx.x, h = blockIdx.y;
+    __shared__ float w_s[MERGE_MAX_CHUNKS];
+    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
     const float* src = partial + (size_t)(t * H + h) * n_chunks * (D + 2);
     float M = NEG_BIG;
-    for (int c = 0; c < n_chunks; c++) M = fmaxf(M, src[(size_t)c * (D + 2)]);
+    for (int c = lane; c < n_chunks; c += WAVE) M = fmaxf(M, src[(size_t)c * (D + 2)]);
+    M = wave_max(M);
     float L = 0.f;
-    for (int c = 0; c < n_chunks; c++) L += src[(size_t)c * (D + 2) + 1] * exp2f(src[(size_t)c * (D + 2)] - M);
+    for (int c = lane; c < n_chunks; c += WAVE) {
+        const float w = exp2f(src[(size_t)c * (D + 2)] - M);
+        w_s[c] = w;
+        L += src[(size_t)c * (D + 2) + 1] * w;
+    }
+    L = wave_sum(L);
+    __syncthreads();
     const float inv = 1.0f / L;
-    for (int d = threadIdx.x; d < D; d += WAVE) {
+    for (int d = lane; d < D; d += WAVE) {
         float acc = 0.f;
-        for (int c = 0; c < n_chunks; c++)
-            acc += src[(size_t)c * (D + 2) + 2 + d] * exp2f(src[(size_t)c * (D + 2)] - M);
+        for (int c = 0; c < n_chunks; c++) acc = fmaf(src[(size_t)c * (D + 2) + 2 + d], w_s[c], acc);
         out[(size_t)t * ldo + h * D + d] = bf16_bits(acc * inv);
     }
 }
@@ -264,7 +274,7 @@ int attn_mfma_launch(const AttnArgs& a) {
         if (chunk_keys < 64) chunk_keys = 64;
         n_chunks = (a.max_seq_len + chunk_keys - 1) / chunk_keys;
         const size_t need = (size_t)a.n_tokens * a.n_heads * n_chunks * (a.head_dim + 2) * sizeof(float);
-        if (n_chunks < 2 || need > a.workspace_bytes) {
+        if (n_chunks < 2 || n_chunks > MERGE_MAX_CHUNKS || need > a.workspace_bytes) {
             n_chunks = 1;
             chunk_keys = a.max_seq_len;
         }

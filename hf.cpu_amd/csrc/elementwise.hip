@@ -45,32 +45,90 @@ extern "C" int hfa_embed(const void* table, int table_dtype, const int* tokens, 
 // One block per output row. The sum of squares is taken in a fixed order (each thread over
 // its strided elements, then waves, then the block), so a row's result does not depend on
 // which other rows are in the launch.
+//
+// If the matrix product before the norm left its result as partial sums (K split for small
+// M), the kernel first finishes it: x[r, :] += sum over splits + bias, written back, and the
+// norm is taken of the new x. This is the fused residual-add + norm of the decode path.
 template <typename TO>
-__global__ void rmsnorm_kernel(const float* __restrict__ x, const float* __restrict__ w, TO* __restrict__ out,
-                               const int* __restrict__ rows, int width, float eps) {
+__global__ __launch_bounds__(1024) void rmsnorm_kernel(float* __restrict__ x, const float* __restrict__ w,
+                                                      TO* __restrict__ out, const int* __restrict__ rows, int width,
+                                                      float eps, const float* __restrict__ partial, int splits,
+                                                      const float* __restrict__ pbias, int n_rows) {
     __shared__ float red[17];
     const int r = blockIdx.x;
-    const float* src = x + (size_t)(rows ? rows[r] : r) * width;
+    const int xr = rows ? rows[r] : r;
+    float* src = x + (size_t)xr * width;
     float ss = 0.f;
-    for (int i = threadIdx.x; i < width; i += blockDim.x) {
-        float v = src[i];
-        ss += v * v;
+    const bool vec = (width & 3) == 0;
+    if (vec) {
+        for (int i = threadIdx.x * 4; i < width; i += blockDim.x * 4) {
+            float4 v = *reinterpret_cast<const float4*>(src + i);
+            if (splits > 0) {
+                // loads in batches of 8 that do not wait for one another, added in ascending order
+                for (int s0 = 0; s0 < splits; s0 += 8) {
+                    float4 p[8];
+#pragma unroll
+                    for (int u = 0; u < 8; u++)
+                        p[u] = s0 + u < splits
+                                   ? *reinterpret_cast<const float4*>(partial + ((size_t)(s0 + u) * n_rows + xr) * width + i)
+                                   : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+                    for (int u = 0; u < 8; u++) { v.x += p[u].x; v.y += p[u].y; v.z += p[u].z; v.w += p[u].w; }
+                }
+                if (pbias) {
+                    const float4 b = *reinterpret_cast<const float4*>(pbias + i);
+                    v.x += b.x; v.y += b.y; v.z += b.z; v.w += b.w;
+                }
+                *reinterpret_cast<float4*>(src + i) = v;
+            }
+            ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+        }
+    } else {
+        for (int i = threadIdx.x; i < width; i += blockDim.x) {
+            float v = src[i];
+            if (splits > 0) {
+                for (int s = 0; s < splits; s++) v += partial[((size_t)s * n_rows + xr) * width + i];
+                if (pbias) v += pbias[i];
+                src[i] = v;
+            }
+            ss += v * v;
+        }
     }
-    ss = block_sum(ss, red);
+    ss = block_sum(ss, red);            // its barriers also order the writes of x before the reads below
     const float scale = 1.0f / sqrtf(ss / (float)width + eps);
     TO* dst = out + (size_t)r * width;
-    for (int i = threadIdx.x; i < width; i += blockDim.x) dst[i] = from_f32<TO>((src[i] * scale) * w[i]);
+    if (vec) {
+        for (int i = threadIdx.x * 4; i < width; i += blockDim.x * 4) {
+            const float4 v = *reinterpret_cast<const float4*>(src + i);
+            const float4 g = *reinterpret_cast<const float4*>(w + i);
+            dst[i] = from_f32<TO>((v.x * scale) * g.x);
+            dst[i + 1] = from_f32<TO>((v.y * scale) * g.y);
+            dst[i + 2] = from_f32<TO>((v.z * scale) * g.z);
+            dst[i + 3] = from_f32<TO>((v.w * scale) * g.w);
+        }
+    } else {
+        for (int i = threadIdx.x; i < width; i += blockDim.x) dst[i] = from_f32<TO>((src[i] * scale) * w[i]);
+    }
 }
 
-extern "C" int hfa_rmsnorm(const float* x, const float* w, void* out, int out_dtype, const int* rows, int n_rows,
-                           int width, float eps, hipStream_t stream) {
+extern "C" int hfa_rmsnorm(float* x, const float* w, void* out, int out_dtype, const int* rows, int n_rows,
+                           int width, float eps, const float* partial, int splits, const float* partial_bias,
+                           hipStream_t stream) {
     HFA_REQUIRE(n_rows > 0 && width > 0, "rmsnorm: bad sizes rows=%d width=%d", n_rows, width);
     HFA_REQUIRE(out_dtype == HFA_F32 || out_dtype == HFA_BF16, "rmsnorm: unknown dtype %d", out_dtype);
-    const int threads = width >= 1024 ? 256 : (width >= 256 ? 128 : 64);
+    HFA_REQUIRE(splits >= 0 && (splits == 0 || (partial && !rows)),
+                "rmsnorm: partial sums cannot be combined with a choice of rows");
+    int threads = width >= 1024 ? 256 : (width >= 256 ? 128 : 64);
+    if (n_rows <= 64 && (width & 3) == 0) {                 // few rows: one pass of 4 values per thread if possible
+        threads = ((width / 4 + WAVE - 1) / WAVE) * WAVE;
+        threads = threads > 1024 ? 1024 : threads;
+    }
     if (out_dtype == HFA_F32)
-        rmsnorm_kernel<float><<<n_rows, threads, 0, stream>>>(x, w, (float*)out, rows, width, eps);
+        rmsnorm_kernel<float><<<n_rows, threads, 0, stream>>>(x, w, (float*)out, rows, width, eps, partial, splits,
+                                                              partial_bias, n_rows);
     else
-        rmsnorm_kernel<bf16><<<n_rows, threads, 0, stream>>>(x, w, (bf16*)out, rows, width, eps);
+        rmsnorm_kernel<bf16><<<n_rows, threads, 0, stream>>>(x, w, (bf16*)out, rows, width, eps, partial, splits,
+                                                             partial_bias, n_rows);
     HFA_LAUNCH_CHECK("rmsnorm");
     return 0;
 }
@@ -79,13 +137,41 @@ extern "C" int hfa_rmsnorm(const float* x, const float* w, void* out, int out_dt
 // One block per token. Cosines and sines of the token's angles go to LDS once; the angle is
 // the fp32 product of the position and the fp32 inverse frequency.
 #define ROPE_MAX_HALF 256
+// If the q/k/v product left its result as partial sums ([splits][T][width] fp32), the kernel
+// finishes it on the way: every value it reads is the sum over the splits plus the bias, and the
+// rotated queries are written into qkv as if the product had stored them.
+template <typename T>
+struct QkvSource {
+    const T* row;
+    const float* partial;
+    const float* bias;
+    size_t split_stride;
+    int splits;
+    __device__ __forceinline__ float at(int c) const {
+        if (splits == 0) return to_f32(row[c]);
+        float v = 0.f;
+        for (int s0 = 0; s0 < splits; s0 += 8) {           // batches of loads that do not wait for one another
+            float p[8];
+#pragma unroll
+            for (int u = 0; u < 8; u++) p[u] = s0 + u < splits ? partial[(s0 + u) * split_stride + c] : 0.f;
+#pragma unroll
+            for (int u = 0; u < 8; u++) v += p[u];
+        }
+        return bias ? v + bias[c] : v;
+    }
+};
+
 template <typename T>
 __global__ void rope_store_kernel(T* __restrict__ qkv, int ld, const int* __restrict__ positions,
                                   const float* __restrict__ inv_freq, int rot_dim, int H, int G, int D,
                                   T* __restrict__ k_cache, T* __restrict__ v_cache,
-                                  const int* __restrict__ slot_map, int page_tokens) {
+                                  const int* __restrict__ slot_map, int page_tokens,
+                                  const float* __restrict__ partial, int splits, const float* __restrict__ pbias,
+                                  int n_tokens) {
     __shared__ float cs[ROPE_MAX_HALF], sn[ROPE_MAX_HALF];
     const int t = blockIdx.x;
+    const int width = (H + 2 * G) * D;
+    QkvSource<T> in = {qkv + (size_t)t * ld, partial + (size_t)t * width, pbias, (size_t)n_tokens * width, splits};
     const int half = rot_dim / 2;
     if (half > 0) {
         const float pos = (float)positions[t];
@@ -103,22 +189,30 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, int ld, const int* __rest
         for (int it = threadIdx.x; it < H * half; it += blockDim.x) {
             const int h = it / half, i = it - h * half;
             T* p = row + h * D;
-            const float x0 = to_f32(p[i]), x1 = to_f32(p[i + half]);
+            const float x0 = in.at(h * D + i), x1 = in.at(h * D + i + half);
             p[i] = from_f32<T>(x0 * cs[i] - x1 * sn[i]);
             p[i + half] = from_f32<T>(x0 * sn[i] + x1 * cs[i]);
+        }
+    }
+    if (splits > 0) {                                      // dimensions of q that are not rotated still need storing
+        const int rest = D - rot_dim;
+        for (int it = threadIdx.x; it < H * rest; it += blockDim.x) {
+            const int h = it / rest, i = rot_dim + (it - h * rest);
+            row[h * D + i] = from_f32<T>(in.at(h * D + i));
         }
     }
     if (G == 0) return;
     const int slot = slot_map ? slot_map[t] : -1;
     T* krow = row + H * D;
     T* vrow = krow + G * D;
+    const int ko = H * D, vo = (H + G) * D;               // where keys and values start in a row
     if (slot < 0) {
         // no cache row: still leave the rotated keys in place so the caller sees them
         if (half > 0) {
             for (int it = threadIdx.x; it < G * half; it += blockDim.x) {
                 const int g = it / half, i = it - g * half;
                 T* p = krow + g * D;
-                const float x0 = to_f32(p[i]), x1 = to_f32(p[i + half]);
+                const float x0 = in.at(ko + g * D + i), x1 = in.at(ko + g * D + i + half);
                 p[i] = from_f32<T>(x0 * cs[i] - x1 * sn[i]);
                 p[i + half] = from_f32<T>(x0 * sn[i] + x1 * cs[i]);
             }
@@ -130,22 +224,23 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, int ld, const int* __rest
     T* vdst = v_cache + (size_t)(slot / page_tokens) * page_tokens * (G * D) + slot % page_tokens;
     for (int it = threadIdx.x; it < G * half; it += blockDim.x) {
         const int g = it / half, i = it - g * half;
-        const T* p = krow + g * D;
-        const float x0 = to_f32(p[i]), x1 = to_f32(p[i + half]);
+        const float x0 = in.at(ko + g * D + i), x1 = in.at(ko + g * D + i + half);
         kdst[g * D + i] = from_f32<T>(x0 * cs[i] - x1 * sn[i]);
         kdst[g * D + i + half] = from_f32<T>(x0 * sn[i] + x1 * cs[i]);
     }
     const int rest = D - rot_dim;   // dimensions that pass through
     for (int it = threadIdx.x; it < G * rest; it += blockDim.x) {
         const int g = it / rest, i = rot_dim + (it - g * rest);
-        kdst[g * D + i] = krow[g * D + i];
+        kdst[g * D + i] = from_f32<T>(in.at(ko + g * D + i));
     }
-    for (int it = threadIdx.x; it < G * D; it += blockDim.x) vdst[(size_t)it * page_tokens] = vrow[it];
+    for (int it = threadIdx.x; it < G * D; it += blockDim.x)
+        vdst[(size_t)it * page_tokens] = from_f32<T>(in.at(vo + it));
 }
 
 extern "C" int hfa_rope_store(void* qkv, int dtype, int ld, const int* positions, const float* inv_freq, int rot_dim,
                               int n_heads, int n_kv_heads, int head_dim, void* k_cache, void* v_cache,
-                              const int* slot_map, int page_tokens, int n_tokens, hipStream_t stream) {
+                              const int* slot_map, int page_tokens, int n_tokens, const float* partial, int splits,
+                              const float* partial_bias, hipStream_t stream) {
     HFA_REQUIRE(n_tokens > 0 && n_heads > 0 && n_kv_heads >= 0 && head_dim > 0, "rope_store: bad sizes");
     HFA_REQUIRE(rot_dim >= 0 && rot_dim % 2 == 0 && rot_dim <= head_dim,
                 "rope_store: rot_dim %d must be even and at most head_dim %d", rot_dim, head_dim);
@@ -156,14 +251,17 @@ extern "C" int hfa_rope_store(void* qkv, int dtype, int ld, const int* positions
     HFA_REQUIRE(n_kv_heads == 0 || !slot_map || (k_cache && v_cache && page_tokens > 0),
                 "rope_store: no cache to store into");
     HFA_REQUIRE(dtype == HFA_F32 || dtype == HFA_BF16, "rope_store: unknown dtype %d", dtype);
+    HFA_REQUIRE(splits >= 0 && (splits == 0 || partial), "rope_store: partial sums announced but not given");
     if (dtype == HFA_F32)
         rope_store_kernel<float><<<n_tokens, 256, 0, stream>>>((float*)qkv, ld, positions, inv_freq, rot_dim, n_heads,
                                                                n_kv_heads, head_dim, (float*)k_cache,
-                                                               (float*)v_cache, slot_map, page_tokens);
+                                                               (float*)v_cache, slot_map, page_tokens, partial,
+                                                               splits, partial_bias, n_tokens);
     else
         rope_store_kernel<bf16><<<n_tokens, 256, 0, stream>>>((bf16*)qkv, ld, positions, inv_freq, rot_dim, n_heads,
                                                               n_kv_heads, head_dim, (bf16*)k_cache, (bf16*)v_cache,
-                                                              slot_map, page_tokens);
+                                                              slot_map, page_tokens, partial, splits, partial_bias,
+                                                              n_tokens);
     HFA_LAUNCH_CHECK("rope_store");
     return 0;
 }

@@ -9,6 +9,7 @@ struct GemmArgs {
     const float* bias;
     void* out; int out_dtype; int ldo;
     int accumulate;
+    int epilogue;            // 0: none; 1: columns are 32 gate, 32 up, ...: out[m, f] = silu(gate) * up
     int M, N, K;
     hipStream_t stream;
 };
@@ -18,5 +19,10 @@ int gemm_generic_launch(const GemmArgs& g);
 
 // bf16 x bf16 on the matrix cores (K and both row strides multiples of 8, 16-byte aligned bases).
 // `workspace` holds the partial sums when K is split for small M; without one K is not split.
+// With `defer`, a product whose K was split leaves its partial sums in the workspace
+// ([splits][M][N] fp32) and reports the number of splits instead of finishing.
 bool gemm_mfma_supports(const GemmArgs& g);
-int gemm_mfma_launch(const GemmArgs& g, void* workspace, size_t workspace_bytes);
+int gemm_mfma_launch(const GemmArgs& g, void* workspace, size_t workspace_bytes, int defer, int* pending_splits);
+int gemm_mode_of(const GemmArgs& g);
+int gemm_finish_launch(const float* partial, int splits, const float* bias, void* out, int mode, int ldo, int M,
+                       int N, hipStream_t stream);

@@ -27,6 +27,7 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 #define OUT_F32 1
 #define OUT_ACC 2
 #define OUT_PARTIAL 3
+#define OUT_SWIGLU 4      // columns come in blocks of 32 gate, 32 up; out[m, f] = silu(gate) * up as bf16
 
 template <int BM, int BN, int BK, int WM, int WN>
 struct MfmaCfg {
@@ -136,6 +137,26 @@ __global__ __launch_bounds__(WM* WN* WAVE) void gemm_mfma_kernel(
     }
 
     // ---- epilogue: element r of a lane is row 8 * (r / 4) + 4 * (lane / 32) + r % 4, column lane % 32 ----
+    if (MODE == OUT_SWIGLU) {
+        static_assert(MODE != OUT_SWIGLU || C::FN % 2 == 0, "gate and up blocks must meet in one wave");
+#pragma unroll
+        for (int i = 0; i < C::FM; i++) {
+#pragma unroll
+            for (int j = 0; j + 1 < C::FN; j += 2) {
+                const int col = n0 + wn * C::TN + j * 32;          // first gate column of the pair of blocks
+                if (col + (lane & 31) >= N) continue;
+                const int f = col / 2 + (lane & 31);
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int row = m0 + wm * C::TM + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
+                    if (row >= M) continue;
+                    const float gt = acc[i][j][r], up = acc[i][j + 1][r];
+                    reinterpret_cast<uint16_t*>(out)[(size_t)row * ldo + f] = bf16_bits((gt / (1.0f + expf(-gt))) * up);
+                }
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < C::FM; i++) {
 #pragma unroll
@@ -173,7 +194,13 @@ __global__ void gemm_finish_kernel(const float* __restrict__ partial, int splits
     float v = 0.f;
     for (int s = 0; s < splits; s++) v += partial[(size_t)s * M * N + idx];
     if (bias) v += bias[col];
-    if (MODE == OUT_BF16)
+    if (MODE == OUT_SWIGLU) {                 // this thread holds a gate column; its up column is 32 further
+        if ((col & 32) != 0) return;
+        float up = 0.f;
+        for (int s = 0; s < splits; s++) up += partial[(size_t)s * M * N + idx + 32];
+        reinterpret_cast<uint16_t*>(out)[(size_t)row * ldo + (col / 64) * 32 + (col & 31)] =
+            bf16_bits((v / (1.0f + expf(-v))) * up);
+    } else if (MODE == OUT_BF16)
         reinterpret_cast<uint16_t*>(out)[(size_t)row * ldo + col] = bf16_bits(v);
     else if (MODE == OUT_F32)
         reinterpret_cast<float*>(out)[(size_t)row * ldo + col] = v;
@@ -208,6 +235,10 @@ static int launch_mode(const GemmArgs& g, int mode, void* out, int splits, int k
         case OUT_BF16: return launch_cfg<BM, BN, BK, WM, WN, OUT_BF16>(g, out, splits, k_per_split);
         case OUT_F32: return launch_cfg<BM, BN, BK, WM, WN, OUT_F32>(g, out, splits, k_per_split);
         case OUT_ACC: return launch_cfg<BM, BN, BK, WM, WN, OUT_ACC>(g, out, splits, k_per_split);
+        case OUT_SWIGLU:
+            if constexpr ((BN / WN) % 64 == 0) return launch_cfg<BM, BN, BK, WM, WN, OUT_SWIGLU>(g, out, splits, k_per_split);
+            hfa_set_error("gemm_mfma: this tile shape cannot pair gate and up columns");
+            return 1;
         default: return launch_cfg<BM, BN, BK, WM, WN, OUT_PARTIAL>(g, out, splits, k_per_split);
     }
 }
@@ -217,8 +248,34 @@ bool gemm_mfma_supports(const GemmArgs& g) {
            ((uintptr_t)g.a & 15) == 0 && ((uintptr_t)g.w & 15) == 0;
 }
 
-int gemm_mfma_launch(const GemmArgs& g, void* workspace, size_t workspace_bytes) {
-    const int mode = g.accumulate ? OUT_ACC : (g.out_dtype == HFA_BF16 ? OUT_BF16 : OUT_F32);
+int gemm_finish_launch(const float* partial, int splits, const float* bias, void* out, int mode, int ldo, int M,
+                       int N, hipStream_t stream) {
+    const size_t total = (size_t)M * N;
+    const int blocks = (int)((total + 255) / 256);
+    if (mode == OUT_BF16)
+        gemm_finish_kernel<OUT_BF16><<<blocks, 256, 0, stream>>>(partial, splits, bias, out, ldo, M, N);
+    else if (mode == OUT_F32)
+        gemm_finish_kernel<OUT_F32><<<blocks, 256, 0, stream>>>(partial, splits, bias, out, ldo, M, N);
+    else if (mode == OUT_SWIGLU)
+        gemm_finish_kernel<OUT_SWIGLU><<<blocks, 256, 0, stream>>>(partial, splits, bias, out, ldo, M, N);
+    else
+        gemm_finish_kernel<OUT_ACC><<<blocks, 256, 0, stream>>>(partial, splits, bias, out, ldo, M, N);
+    HFA_LAUNCH_CHECK("gemm_finish");
+    return 0;
+}
+
+int gemm_mode_of(const GemmArgs& g) {
+    if (g.epilogue == 1) return OUT_SWIGLU;
+    return g.accumulate ? OUT_ACC : (g.out_dtype == HFA_BF16 ? OUT_BF16 : OUT_F32);
+}
+
+int gemm_mfma_launch(const GemmArgs& g, void* workspace, size_t workspace_bytes, int defer, int* pending_splits) {
+    const int mode = gemm_mode_of(g);
+    if (pending_splits) *pending_splits = 0;
+    if (mode == OUT_SWIGLU && (g.N % 64 != 0 || g.bias != nullptr || g.out_dtype != HFA_BF16)) {
+        hfa_set_error("gemm: the gate/up epilogue needs N a multiple of 64, no bias and a bf16 output");
+        return 1;
+    }
     const int BK = 64;
     const int BM = g.M > 64 ? 128 : (g.M > 32 ? 64 : 32), BN = 128;
     const int tiles = ((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN);
@@ -243,18 +300,14 @@ int gemm_mfma_launch(const GemmArgs& g, void* workspace, size_t workspace_bytes)
         rc = launch_mode<128, 128, 64, 2, 2>(g, kmode, kout, splits, k_per_split);
     else if (BM == 64)
         rc = launch_mode<64, 128, 64, 2, 2>(g, kmode, kout, splits, k_per_split);
+    else if (kmode == OUT_SWIGLU)
+        rc = launch_mode<32, 128, 64, 1, 2>(g, kmode, kout, splits, k_per_split);
     else
         rc = launch_mode<32, 128, 64, 1, 4>(g, kmode, kout, splits, k_per_split);
     if (rc || splits == 1) return rc;
-    const size_t total = (size_t)g.M * g.N;
-    const int blocks = (int)((total + 255) / 256);
-    const float* part = (const float*)workspace;
-    if (mode == OUT_BF16)
-        gemm_finish_kernel<OUT_BF16><<<blocks, 256, 0, g.stream>>>(part, splits, g.bias, g.out, g.ldo, g.M, g.N);
-    else if (mode == OUT_F32)
-        gemm_finish_kernel<OUT_F32><<<blocks, 256, 0, g.stream>>>(part, splits, g.bias, g.out, g.ldo, g.M, g.N);
-    else
-        gemm_finish_kernel<OUT_ACC><<<blocks, 256, 0, g.stream>>>(part, splits, g.bias, g.out, g.ldo, g.M, g.N);
-    HFA_LAUNCH_CHECK("gemm_finish");
-    return 0;
+    if (defer && pending_splits) {             // the caller sums the partial results in its next kernel
+        *pending_splits = splits;
+        return 0;
+    }
+    return gemm_finish_launch((const float*)workspace, splits, g.bias, g.out, mode, g.ldo, g.M, g.N, g.stream);
 }

@@ -58,10 +58,12 @@ class IntStaging:
         self.events = []
         self.dev = None
         self.turn = 0
+        self.generation = 0
         self._grow(capacity)
 
     def _grow(self, capacity):
         torch.cuda.synchronize(self.device)
+        self.generation += 1                      # captured graphs hold the old address
         self.capacity = capacity
         self.host = [torch.empty(capacity, dtype=torch.int32, pin_memory=True) for _ in range(2)]
         self.events = [None, None]

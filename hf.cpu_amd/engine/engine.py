@@ -15,11 +15,17 @@ from .batch import Entry, GroupInputs, IntStaging, StepInputs, as_i32
 
 
 class Engine:
+    GRAPH_MAX_TOKENS = 256        # decode-only steps up to this many requests replay a captured graph
+    GRAPH_LEN_BUCKET = 256        # a graph serves request lengths up to a multiple of this
+
     def __init__(self, model, ops, page_tokens=16, n_pages=None, max_tokens=None, max_seqs=8,
-                 max_context=None):
+                 max_context=None, graphs=True):
         """``n_pages`` pages per group, or ``max_tokens`` (the most tokens live requests
         hold at once, each request's count rounded up to whole pages) from which it follows.
-        ``max_context`` bounds one request's length (default: what the pool can hold)."""
+        ``max_context`` bounds one request's length (default: what the pool can hold).
+        ``graphs``: steps in which every request brings one token (decode) are captured
+        into a HIP graph per (batch size, length bucket) the second time their shape is seen
+        and replayed from then on; the integers of a step still travel before the replay."""
         if n_pages is None:
             if max_tokens is None:
                 fail(EINVAL, "engine: give n_pages or max_tokens")
@@ -32,6 +38,10 @@ class Engine:
         self.staging = IntStaging(ops.device)
         self.vocab_size = model.vocab_size
         self.steps_run = 0
+        self.use_graphs = bool(graphs) and bool(getattr(model, "graph_safe", False))
+        self._graphs = {}
+        self._graph_seen = set()
+        self.graph_replays = 0
 
     # ---- requests ------------------------------------------------------------
     def has(self, req_id):
@@ -81,7 +91,7 @@ class Engine:
             step = self._inputs(entries)
             logits = self.ops.scratch("logits", (max(step.n_logit_rows, 1), self.vocab_size), torch.float32)
             logits = logits[:step.n_logit_rows]
-            self.model.forward(self.ops, step, self.storage.views, logits)
+            self._run(step, logits)
         except BaseException:
             for r in reserved:
                 mgr.rollback(r)
@@ -92,6 +102,34 @@ class Engine:
             mgr.commit(e.req_id, len(e.tokens))
         self.steps_run += 1
         return logits
+
+    def _run(self, step, logits):
+        """The forward pass of the step, eagerly or as a replay of the graph of its shape."""
+        decode_only = step.max_q_len == 1 and step.n_tokens <= self.GRAPH_MAX_TOKENS
+        if not (self.use_graphs and decode_only):
+            return self.model.forward(self.ops, step, self.storage.views, logits)
+        # The kernels use max_seq_len only to choose how the key range is cut, so a graph
+        # captured for a length bucket serves every shorter length too.
+        B = self.GRAPH_LEN_BUCKET
+        step.max_seq_len = min(-(-step.max_seq_len // B) * B, self.manager.max_context)
+        key = (step.n_tokens, step.n_logit_rows, step.max_seq_len)
+        stamp = (self.ops.scratch_generation, self.staging.generation)
+        hit = self._graphs.get(key)
+        if hit is not None and hit[0] == stamp:
+            hit[1].replay()
+            self.graph_replays += 1
+            return
+        if key not in self._graph_seen:          # first sight: run eagerly, which also sizes the work buffers
+            self._graph_seen.add(key)
+            return self.model.forward(self.ops, step, self.storage.views, logits)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            self.model.forward(self.ops, step, self.storage.views, logits)
+        if (self.ops.scratch_generation, self.staging.generation) != stamp:
+            fail(EINVAL, "a work buffer moved while a step was captured")
+        self._graphs[key] = (stamp, graph)
+        graph.replay()
+        self.graph_replays += 1
 
     def _inputs(self, entries):
         mgr = self.manager
@@ -122,12 +160,14 @@ class Engine:
             max_q = max(max_q, n)
             max_len = max(max_len, h.length + n)
             at += n
-        arrays = [tokens, positions, token_slot, q_start, seq_slot, seq_len, as_i32(rows)]
+        # Arrays whose sizes follow from (T, S, R) come first, so that their places in the
+        # device buffer are the same for every step of one shape (a captured graph reads them there).
+        arrays = [tokens, positions, token_slot, q_start, seq_slot, seq_len, as_i32(rows)] + slot_maps
+        G = len(mgr.groups)
         dirty = []
-        for g in range(len(mgr.groups)):
+        for g in range(G):
             app = mgr.drain_appended(g)
             dirty.append(len(app))
-            arrays.append(slot_maps[g])
             arrays.append(as_i32([slot * mgr.max_blocks + block for slot, block, _ in app]))
             arrays.append(as_i32([page for _, _, page in app]))
         views = self.staging.upload(arrays)
@@ -137,8 +177,9 @@ class Engine:
         step.max_q_len, step.max_seq_len = max_q, max_len
         step.host = dict(tokens=tokens, positions=positions, token_slot=token_slot, q_start=q_start,
                          seq_slot=seq_slot, seq_len=seq_len, logit_rows=as_i32(rows))
-        for g in range(len(mgr.groups)):
-            slot_map, idx, val = views[7 + 3 * g:10 + 3 * g]
+        for g in range(G):
+            slot_map = views[7 + g]
+            idx, val = views[7 + G + 2 * g:9 + G + 2 * g]
             table = self.storage.block_tables[g]
             if dirty[g]:
                 self.ops.scatter_i32(table.view(-1), idx, val)

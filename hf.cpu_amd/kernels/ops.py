@@ -1,10 +1,21 @@
 """The kernels as methods on tensors.
 
+A matrix product with few rows splits its K range over the machine and leaves partial sums in
+the workspace. With ``defer=True`` the product does not add them up itself: the next kernel
+that reads the output does (``rmsnorm`` for the residual stream, ``rope_store`` for q/k/v), which
+saves a launch and a pass over memory per product in decode. The pending state lives here; every
+method that could disturb it settles it first, and a part that touches a tensor with anything
+but these methods calls ``settle`` before.
+
+
 ``Ops`` belongs to one device and one compute dtype. Every method checks shapes,
 dtypes and layout on the host, hands raw pointers to the library on the current
 stream, and raises EngineError if the library refuses the call. Nothing here
 computes with a library routine or on the CPU.
 """
+import ctypes
+from dataclasses import dataclass
+
 import torch
 
 from ..status import EINVAL, ENOTSUP, EngineError, fail
@@ -35,6 +46,15 @@ def _ints(t, what, n=None):
     return t.data_ptr()
 
 
+@dataclass
+class Pending:
+    """A matrix product whose partial sums ([splits][M][N] fp32 in the workspace) wait to be added up."""
+    out: torch.Tensor
+    splits: int
+    bias: object
+    accumulate: bool
+
+
 class Ops:
     def __init__(self, act_dtype=torch.bfloat16, device="cuda:0"):
         if not torch.cuda.is_available():
@@ -45,7 +65,11 @@ class Ops:
         self.act_dtype = act_dtype
         self.lib = library()
         self._scratch = {}
+        self.scratch_generation = 0
         self.workspace = torch.empty(WORKSPACE_BYTES, dtype=torch.uint8, device=self.device)
+        self.attn_workspace = torch.empty(WORKSPACE_BYTES, dtype=torch.uint8, device=self.device)
+        self._pending = None
+        self._splits_out = ctypes.c_int(0)
         self.force_plain_gemm = False        # tests set these to compare the matrix-core paths with the plain ones
         self.force_plain_attention = False
 
@@ -66,12 +90,16 @@ class Ops:
         nbytes = max(n, 1) * torch.empty((), dtype=dtype).element_size()
         buf = self._scratch.get(name)
         if buf is None or buf.numel() < nbytes:
+            if torch.cuda.is_current_stream_capturing():
+                fail(EINVAL, f"work buffer '{name}' would have to grow while a graph is being captured")
             buf = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=self.device)
             self._scratch[name] = buf
+            self.scratch_generation += 1          # captured graphs hold the old address
         return buf[:nbytes].view(dtype).view(*shape)
 
     # ---- kernels -----------------------------------------------------------
     def embed(self, table, tokens, out_x):
+        self.settle()
         T = out_x.shape[0]
         if out_x.dtype != torch.float32 or not out_x.is_contiguous() or not table.is_contiguous() \
                 or table.shape[1] != out_x.shape[1]:
@@ -87,28 +115,84 @@ class Ops:
             fail(EINVAL, "rmsnorm: x and weight must be fp32, contiguous, and of one width with out")
         if rows is None and R != x.shape[0]:
             fail(EINVAL, "rmsnorm: without row indices the output must have x's rows")
+        pend = self._take_pending(x) if rows is None else None
+        if pend is None:
+            self.settle()
         self._check(self.lib.hfa_rmsnorm(x.data_ptr(), weight.data_ptr(), out.data_ptr(), _code(out),
                                          None if rows is None else _ints(rows, "rmsnorm rows", R),
-                                         R, E, float(eps), self._stream()))
+                                         R, E, float(eps), None if pend is None else self.workspace.data_ptr(),
+                                         0 if pend is None else pend.splits,
+                                         None if pend is None or pend.bias is None else pend.bias.data_ptr(),
+                                         self._stream()))
 
-    def gemm(self, a, w, out, bias=None, accumulate=False):
-        """out (+)= a @ w.T + bias, fp32 accumulation."""
+    def _take_pending(self, tensor):
+        """The pending product if it is the residual sum of ``tensor`` (whole, contiguous), else None."""
+        p = self._pending
+        if p is not None and p.accumulate and p.out.data_ptr() == tensor.data_ptr() \
+                and p.out.shape == tensor.shape and tensor.is_contiguous():
+            self._pending = None
+            return p
+        return None
+
+    def settle(self, tensor=None):
+        """Adds up a deferred product now (all of them if ``tensor`` is None, else only one that
+        writes ``tensor``)."""
+        p = self._pending
+        if p is None or (tensor is not None and p.out.data_ptr() != tensor.data_ptr()):
+            return
+        self._pending = None
+        M, N = p.out.shape
+        self._check(self.lib.hfa_gemm_finish(self.workspace.data_ptr(), p.splits,
+                                             None if p.bias is None else p.bias.data_ptr(), p.out.data_ptr(),
+                                             _code(p.out), _rows(p.out, "gemm out"), 1 if p.accumulate else 0, 0,
+                                             M, N, self._stream()))
+
+    def gemm(self, a, w, out, bias=None, accumulate=False, defer=False, swiglu=False):
+        """out (+)= a @ w.T + bias, fp32 accumulation. ``defer``: if the kernel split K, leave the
+        partial sums for the next kernel that reads ``out`` (see the module's text).
+        ``swiglu``: w's rows come in blocks of 32 gate, 32 up (``interleave_gate_up``) and
+        out = silu(gate) * up has half as many columns."""
+        self.settle()
         lda, ldw, ldo = _rows(a, "gemm a"), _rows(w, "gemm w"), _rows(out, "gemm out")
         M, K = a.shape
         N = w.shape[0]
-        if w.shape[1] != K or tuple(out.shape) != (M, N):
+        if w.shape[1] != K or tuple(out.shape) != (M, N // 2 if swiglu else N):
             fail(EINVAL, f"gemm: shapes a{tuple(a.shape)} w{tuple(w.shape)} out{tuple(out.shape)} do not fit")
         if bias is not None and (bias.dtype != torch.float32 or bias.numel() != N or not bias.is_contiguous()):
             fail(EINVAL, "gemm: the bias must be contiguous fp32 with one value per output column")
+        self._splits_out.value = 0
         self._check(self.lib.hfa_gemm(a.data_ptr(), _code(a), lda, w.data_ptr(), _code(w), ldw,
                                       None if bias is None else bias.data_ptr(), out.data_ptr(), _code(out), ldo,
-                                      1 if accumulate else 0, M, N, K, self.workspace.data_ptr(),
-                                      self.workspace.numel(), 1 if self.force_plain_gemm else 0, self._stream()))
+                                      1 if accumulate else 0, 1 if swiglu else 0, M, N, K, self.workspace.data_ptr(),
+                                      self.workspace.numel(), 1 if defer else 0, ctypes.byref(self._splits_out),
+                                      1 if self.force_plain_gemm else 0, self._stream()))
+        if self._splits_out.value:
+            self._pending = Pending(out, self._splits_out.value, bias, accumulate)
+
+    def can_fuse_swiglu(self, w_gate, w_up):
+        """Whether gate and up may be interleaved for ``gemm(..., swiglu=True)``: bf16 on the
+        matrix cores, a feature count that is a multiple of 32."""
+        F, E = w_gate.shape
+        return (self.act_dtype == torch.bfloat16 and w_gate.dtype == torch.bfloat16 and w_up.dtype == torch.bfloat16
+                and F % 32 == 0 and E % 8 == 0 and not self.force_plain_gemm)
+
+    @staticmethod
+    def interleave_gate_up(w_gate, w_up):
+        """[2F, E]: rows 0..31 of gate, rows 0..31 of up, rows 32..63 of gate, ..."""
+        F, E = w_gate.shape
+        return torch.stack([w_gate.view(F // 32, 32, E), w_up.view(F // 32, 32, E)], dim=1).reshape(2 * F, E).contiguous()
 
     def rope_store(self, qkv, positions, inv_freq, rot_dim, n_heads, n_kv_heads, head_dim, cache, slot_map):
         """Rotates q (and k) inside ``qkv`` and, if ``slot_map`` is given, stores k and v
         rows into ``cache.k`` / ``cache.v`` at the rows it names (values transposed inside
         their page, see csrc/api.h)."""
+        pend = self._pending
+        if pend is not None and not pend.accumulate and pend.out.data_ptr() == qkv.data_ptr() \
+                and pend.out.shape == qkv.shape and qkv.shape[1] == (n_heads + 2 * n_kv_heads) * head_dim:
+            self._pending = None
+        else:
+            pend = None
+            self.settle()
         ld = _rows(qkv, "rope_store qkv")
         T = qkv.shape[0]
         if qkv.shape[1] < (n_heads + 2 * n_kv_heads) * head_dim:
@@ -125,10 +209,13 @@ class Ops:
             qkv.data_ptr(), _code(qkv), ld, None if positions is None else _ints(positions, "positions", T),
             None if inv_freq is None else inv_freq.data_ptr(), rot_dim, n_heads, n_kv_heads, head_dim,
             k_ptr, v_ptr, None if slot_map is None else _ints(slot_map, "slot_map", T),
-            getattr(cache, "page_tokens", 0) or 0, T, self._stream()))
+            getattr(cache, "page_tokens", 0) or 0, T, None if pend is None else self.workspace.data_ptr(),
+            0 if pend is None else pend.splits,
+            None if pend is None or pend.bias is None else pend.bias.data_ptr(), self._stream()))
 
     def paged_attention(self, q, n_heads, n_kv_heads, head_dim, cache, step, window, scale, out):
         """Attention of the first ``n_heads * head_dim`` columns of ``q`` over ``cache``."""
+        self.settle()
         T = q.shape[0]
         ldq, ldo = _rows(q, "attention q"), _rows(out, "attention out")
         g = step.group(cache.group)
@@ -141,10 +228,12 @@ class Ops:
             g.block_table.data_ptr(), g.block_table.shape[1], _ints(step.token_slot, "token_slot", T),
             _ints(step.positions, "positions", T), _ints(step.q_start, "q_start", step.n_seqs + 1), step.n_seqs,
             step.max_q_len, step.max_seq_len, out.data_ptr(), ldo, T, n_heads, n_kv_heads, head_dim,
-            cache.page_tokens, int(window), float(scale), self.workspace.data_ptr(), self.workspace.numel(),
+            cache.page_tokens, int(window), float(scale), self.attn_workspace.data_ptr(),
+            self.attn_workspace.numel(),
             1 if self.force_plain_attention else 0, self._stream()))
 
     def swiglu(self, gate_up, out):
+        self.settle()
         T, F2 = gate_up.shape
         if not gate_up.is_contiguous() or not out.is_contiguous() or tuple(out.shape) != (T, F2 // 2) \
                 or out.dtype != gate_up.dtype or F2 % 2:
@@ -158,6 +247,7 @@ class Ops:
                                                  _ints(val, "scatter val", n), n, self._stream()))
 
     def argmax(self, logits, out=None):
+        self.settle()
         R, V = logits.shape
         if logits.dtype != torch.float32:
             fail(EINVAL, "argmax: logits must be fp32")
@@ -170,6 +260,7 @@ class Ops:
     def topk(self, logits, k, want_stats=True):
         """(ids [R, k] int32, values [R, k] fp32, stats [R, 2] fp32 = max and log-sum-exp
         above the max), candidates in the order (logit descending, id ascending)."""
+        self.settle()
         R, V = logits.shape
         if logits.dtype != torch.float32:
             fail(EINVAL, "topk: logits must be fp32")

@@ -102,6 +102,13 @@ class Model:
         for p in self._all_parts():
             p.bind_all(params, ops)
 
+    @property
+    def graph_safe(self):
+        """Whether every part (and every part it owns) allows steps to be captured into graphs."""
+        def safe(p):
+            return p.graph_safe and all(safe(q) for q in p.sub_parts())
+        return all(safe(p) for p in self._all_parts())
+
     # ---- what the cache manager needs to know -----------------------------
     def cache_needs(self):
         """For each schedule entry: PagedKV, FixedState, or None (no cache of its own)."""
@@ -128,6 +135,7 @@ class Model:
             cache = caches[i if own else e.cache_of]
             layer.block.forward(ops, step, x, layer.norm1, layer.mixer, layer.norm2, layer.feed_forward,
                                 cache, write_cache=own)
+        ops.settle()
         R = step.n_logit_rows
         if R:
             h = ops.scratch("head_in", (R, self.hidden_size), ops.act_dtype)

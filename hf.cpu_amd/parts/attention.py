@@ -19,6 +19,8 @@ class Attention(Part):
     A key at ``pk`` is visible to a query at ``pq`` iff ``0 <= pq - pk`` and, when
     ``window > 0``, ``pq - pk < window``.
     """
+    graph_safe = True
+
 
     def __init__(self, hidden_size, n_heads, n_kv_heads, head_dim, qkv_bias, window, position,
                  scale=None, out_bias=False, prefix=""):
@@ -70,8 +72,9 @@ class Attention(Part):
         T = h.shape[0]
         width = self.QD + 2 * self.KD if write_cache else self.QD
         qkv = ops.scratch("qkv", (T, width), ops.act_dtype)
-        ops.gemm(h, self.w_qkv[:width], qkv, bias=None if self.b_qkv is None else self.b_qkv[:width])
+        # a product that split K is added up inside the next kernel (position.store, the next norm)
+        ops.gemm(h, self.w_qkv[:width], qkv, bias=None if self.b_qkv is None else self.b_qkv[:width], defer=True)
         self.position.store(ops, step, qkv, self.H, self.G if write_cache else 0, cache, write_cache)
         att = ops.scratch("att", (T, self.QD), ops.act_dtype)
         ops.paged_attention(qkv, self.H, self.G, self.D, cache, step, self.window, self.scale, att)
-        ops.gemm(att, self.w_o, x, bias=self.b_o, accumulate=True)
+        ops.gemm(att, self.w_o, x, bias=self.b_o, accumulate=True, defer=True)

@@ -51,6 +51,10 @@ class FixedState:
 class Part:
     role = None
     kind = None
+    # True if forward() only enqueues kernels whose arguments depend on the step's shape, never
+    # on its values (no host-side loop over the step's tokens, no read-back): only then may the
+    # engine capture a step into a graph and replay it. Parts say so themselves; the default is no.
+    graph_safe = False
 
     def __init__(self, prefix=""):
         self.prefix = prefix

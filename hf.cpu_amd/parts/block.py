@@ -7,6 +7,8 @@ from .base import Part
 class PreNormBlock(Part):
     """``x += mixer(norm1(x)); x += feed_forward(norm2(x))`` (src/model.c:580-623):
     norms in front of each part, nothing after, the residual stream in fp32."""
+    graph_safe = True
+
 
     def __init__(self, hidden_size, prefix=""):
         super().__init__(prefix)
@@ -14,7 +16,9 @@ class PreNormBlock(Part):
 
     def forward(self, ops, step, x, norm1, mixer, norm2, feed_forward, cache, write_cache=True):
         h = ops.scratch("normed", (x.shape[0], self.E), ops.act_dtype)
-        norm1.forward(ops, x, h)
+        norm1.forward(ops, x, h)      # also adds up a product the previous part deferred into x
+        ops.settle(x)                 # (nothing left to do unless the norm could not)
         mixer.forward(ops, step, h, cache, x, write_cache)
         norm2.forward(ops, x, h)
+        ops.settle(x)
         feed_forward.forward(ops, step, h, x)

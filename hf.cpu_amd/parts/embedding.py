@@ -6,6 +6,8 @@ from .base import ParamSpec, Part
 @register_part("embedding", "lookup")
 class Embedding(Part):
     """``x[t, :] = table[token[t], :]`` without scaling (src/model.c:566-571)."""
+    graph_safe = True
+
 
     def __init__(self, vocab_size, hidden_size, prefix=""):
         super().__init__(prefix)
@@ -27,6 +29,8 @@ class LinearHead(Part):
     """``logits = W h`` in fp32, no bias (src/model.c:633-635). With ``tied`` the
     matrix is the embedding table unless the checkpoint holds one of its own, which
     then wins (src/model.c:156-158)."""
+    graph_safe = True
+
 
     def __init__(self, vocab_size, hidden_size, tied, tied_to="", prefix=""):
         super().__init__(prefix)

@@ -11,6 +11,8 @@ class GatedMLP(Part):
     """``x += Wdown (act(Wgate h) * (Wup h))`` with ``act(g) = g / (1 + exp(-g))``
     (src/model.c:612-623, src/mathx.c:34). Gate and up share their input and are held
     as one matrix, gate rows first."""
+    graph_safe = True
+
 
     def __init__(self, hidden_size, intermediate_size, activation="silu", prefix=""):
         super().__init__(prefix)
@@ -18,6 +20,7 @@ class GatedMLP(Part):
             fail(ENOTSUP, f"gated_mlp: activation '{activation}' is not implemented")
         self.E, self.F = hidden_size, intermediate_size
         self.w_gate_up = self.w_down = None
+        self.fused = False
 
     def param_specs(self):
         p = self.prefix
@@ -29,13 +32,22 @@ class GatedMLP(Part):
         p = self.prefix
         g, u = params[p + "gate_proj.weight"], params[p + "up_proj.weight"]
         dt = torch.float32 if torch.float32 in (g.dtype, u.dtype) else g.dtype
-        self.w_gate_up = torch.cat([g.to(dt), u.to(dt)], dim=0).contiguous()
+        # On the matrix cores gate and up rows are interleaved in blocks of 32, so that the product's
+        # last step can form silu(gate) * up without storing gate and up.
+        self.fused = ops.can_fuse_swiglu(g, u)
+        if self.fused:
+            self.w_gate_up = ops.interleave_gate_up(g, u)
+        else:
+            self.w_gate_up = torch.cat([g.to(dt), u.to(dt)], dim=0).contiguous()
         self.w_down = params[p + "down_proj.weight"]
 
     def forward(self, ops, step, h, x):
         T = h.shape[0]
-        gu = ops.scratch("gate_up", (T, 2 * self.F), ops.act_dtype)
-        ops.gemm(h, self.w_gate_up, gu)
         act = ops.scratch("ffn_act", (T, self.F), ops.act_dtype)
-        ops.swiglu(gu, act)
-        ops.gemm(act, self.w_down, x, accumulate=True)
+        if self.fused:
+            ops.gemm(h, self.w_gate_up, act, swiglu=True)
+        else:
+            gu = ops.scratch("gate_up", (T, 2 * self.F), ops.act_dtype)
+            ops.gemm(h, self.w_gate_up, gu)
+            ops.swiglu(gu, act)
+        ops.gemm(act, self.w_down, x, accumulate=True, defer=True)

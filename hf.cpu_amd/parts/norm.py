@@ -7,6 +7,8 @@ from .base import ParamSpec, Part
 class RMSNorm(Part):
     """``y_i = x_i * (1 / sqrt(mean(x^2) + eps)) * w_i`` with the mean of squares in
     fp32 (src/mathx.c:65-75; the reference sums in fp64)."""
+    graph_safe = True
+
 
     def __init__(self, size, eps, prefix=""):
         super().__init__(prefix)

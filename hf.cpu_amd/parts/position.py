@@ -15,6 +15,8 @@ class Rotary(Part):
     product of the position and a table rounded from fp64). Dimensions from
     ``rot_dim`` on pass through. Values are not rotated; keys are stored rotated
     (src/model.c:596-600)."""
+    graph_safe = True
+
 
     def __init__(self, head_dim, rot_dim, theta, pairing="split_half", prefix=""):
         super().__init__(prefix)
@@ -42,6 +44,8 @@ class Rotary(Part):
 @register_part("position", "none")
 class NoPosition(Part):
     """No position encoding: keys and values go to the cache as they are."""
+    graph_safe = True
+
 
     def __init__(self, head_dim, prefix=""):
         super().__init__(prefix)

@@ -158,3 +158,42 @@ def test_step_refusals_leave_no_trace(gpu, tiny):
     toks = reqs["r2"]
     got = helpers.run_trace_in_engine(engine, helpers.trace_whole({"r2": toks}))
     helpers.compare(got, want, TOL["float32"], "after refusals")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_graph_replay_equals_eager(gpu, tiny, dtype):
+    """Decode steps replayed from a captured graph against the same steps run eagerly: many
+    replays, with eager steps of other shapes (a new prompt, a request that ends) in between,
+    every replay compared. The graph is first replayed at its third step of a shape."""
+    name, cfg, d, reqs, want = tiny
+    import hf_cpu_amd
+    runs = {}
+    for graphs in (False, True):
+        engine = hf_cpu_amd.load_engine(d, dtype=dtype, page_tokens=helpers.PAGE[name], max_tokens=1024,
+                                        max_seqs=4, graphs=graphs)
+        rows = []
+        live = {r: 0 for r in ("r2", "r3", "r4")}
+        for r in live:                                        # prompts: all but the last 25 tokens
+            n = len(reqs[r]) - 25
+            engine.step([(r, reqs[r][:n], [])])
+            live[r] = n
+        for i in range(25):
+            if i == 9:                                        # an eager step of another shape in between
+                engine.step([("r1", reqs["r1"], [0])])
+            if i == 15:
+                engine.release("r1")
+            logits = engine.step([(r, [reqs[r][at]], [0]) for r, at in live.items()])
+            rows.append(logits.float().cpu().numpy().copy())
+            for r in live:
+                live[r] += 1
+        runs[graphs] = rows
+        if graphs:
+            assert engine.graph_replays >= 20
+        else:
+            assert engine.graph_replays == 0
+    for i, (a, b) in enumerate(zip(runs[False], runs[True])):
+        scale = float(np.max(np.abs(a)))
+        err = float(np.max(np.abs(a - b))) / scale
+        assert err <= (1e-6 if dtype == "float32" else 1e-2), f"decode step {i}: graph and eager differ by {err:.3e}"
+    got = {("r4", len(reqs["r4"]) - 25 + i): runs[True][i][2] for i in range(25)}
+    helpers.compare(got, want, TOL[dtype], "graph replay")

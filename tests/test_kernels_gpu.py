@@ -129,6 +129,73 @@ def test_gemm_on_matrix_cores(ops16, M, N, K):
     assert np.max(np.abs(acc.cpu().numpy() - (want + res))) <= 2e-5 * scale
 
 
+@pytest.mark.parametrize("M", [1, 8, 64, 100, 300])
+def test_gemm_with_gate_up_epilogue(ops16, M):
+    """Gate and up rows interleaved in blocks of 32; the product's last step forms silu(gate) * up:
+    directly in the tile's epilogue (large M) or when the split K is added up (small M)."""
+    rng = np.random.default_rng(M)
+    E, F = 256, 352
+    x = rng.standard_normal((M, E)).astype(np.float32)
+    wg = (rng.standard_normal((F, E)) / 16).astype(np.float32)
+    wu = (rng.standard_normal((F, E)) / 16).astype(np.float32)
+    tg, tu = dev(wg, torch.bfloat16), dev(wu, torch.bfloat16)
+    assert ops16.can_fuse_swiglu(tg, tu)
+    w = ops16.interleave_gate_up(tg, tu)
+    assert torch.equal(w[:32], tg[:32]) and torch.equal(w[32:64], tu[:32]) and torch.equal(w[64:96], tg[32:64])
+    out = torch.empty((M, F), dtype=torch.bfloat16, device="cuda")
+    ops16.gemm(dev(x, torch.bfloat16), w, out, swiglu=True)
+    xr = rounded(x, torch.bfloat16)
+    want = plain.silu(xr @ rounded(wg, torch.bfloat16).T) * (xr @ rounded(wu, torch.bfloat16).T)
+    assert np.max(np.abs(out.float().cpu().numpy() - want)) <= 0.01 * max(1.0, np.max(np.abs(want)))
+
+
+def test_deferred_products_are_finished_by_the_next_kernel(ops16):
+    """A product with few rows and a long K leaves partial sums; the norm that follows adds them
+    into the residual stream and norms the result; rope_store does the same for q, k and v."""
+    rng = np.random.default_rng(0)
+    M, K, E = 5, 4096, 512
+    a = rng.standard_normal((M, K)).astype(np.float32)
+    w = (rng.standard_normal((E, K)) / 64).astype(np.float32)
+    b = rng.standard_normal(E).astype(np.float32)
+    x0 = rng.standard_normal((M, E)).astype(np.float32)
+    g = (1 + 0.1 * rng.standard_normal(E)).astype(np.float32)
+    x = dev(x0)
+    ops16.gemm(dev(a, torch.bfloat16), dev(w, torch.bfloat16), x, bias=dev(b), accumulate=True, defer=True)
+    assert ops16._pending is not None and ops16._pending.splits > 1, "the case was meant to split K"
+    h = torch.empty((M, E), dtype=torch.bfloat16, device="cuda")
+    ops16.rmsnorm(x, dev(g), 1e-6, h)
+    assert ops16._pending is None
+    x_want = x0 + rounded(a, torch.bfloat16) @ rounded(w, torch.bfloat16).T + b
+    assert np.max(np.abs(x.cpu().numpy() - x_want)) < 1e-4
+    assert np.max(np.abs(h.float().cpu().numpy() - plain.rmsnorm(x_want, g, 1e-6))) < 0.03
+    # the same product, settled explicitly
+    x2 = dev(x0)
+    ops16.gemm(dev(a, torch.bfloat16), dev(w, torch.bfloat16), x2, bias=dev(b), accumulate=True, defer=True)
+    ops16.settle(x2)
+    assert float((x2 - x).abs().max()) < 1e-5          # the same sums in another order
+    # q, k, v: H = 2, G = 1, D = 64 -> width 256
+    H, G, D = 2, 1, 64
+    wq = (rng.standard_normal(((H + 2 * G) * D, K)) / 64).astype(np.float32)
+    bq = rng.standard_normal((H + 2 * G) * D).astype(np.float32)
+    qkv = torch.zeros((M, (H + 2 * G) * D), dtype=torch.bfloat16, device="cuda")
+    ops16.gemm(dev(a, torch.bfloat16), dev(wq, torch.bfloat16), qkv, bias=dev(bq), defer=True)
+    assert ops16._pending is not None
+    cache = FakeCache(group=0, k=torch.zeros((8, G * D), dtype=torch.bfloat16, device="cuda"),
+                      v=torch.zeros((8, G * D), dtype=torch.bfloat16, device="cuda"), page_tokens=4)
+    positions, slot_map = [3, 0, 9, 100, 7], [0, 5, 2, 7, 1]
+    i = np.arange(D // 2, dtype=np.float64)
+    inv_freq = dev((1e4 ** (-2.0 * i / D)).astype(np.float32))
+    ops16.rope_store(qkv, ints(positions), inv_freq, D, H, G, D, cache, ints(slot_map))
+    assert ops16._pending is None
+    full = rounded(a, torch.bfloat16) @ rounded(wq, torch.bfloat16).T + bq
+    q_want = plain.rope(full[:, :H * D].reshape(M, H, D), positions, D, 1e4).reshape(M, H * D)
+    k_want = plain.rope(full[:, H * D:(H + G) * D].reshape(M, G, D), positions, D, 1e4).reshape(M, G * D)
+    assert np.max(np.abs(qkv[:, :H * D].float().cpu().numpy() - q_want)) < 0.05
+    assert np.max(np.abs(cache.k.float().cpu().numpy()[slot_map] - k_want)) < 0.05
+    vc = from_value_layout(cache.v.float().cpu().numpy(), 4)
+    assert np.max(np.abs(vc[slot_map] - full[:, (H + G) * D:])) < 0.05
+
+
 def test_gemm_matches_library_product(ops32):
     """The kernel against the library's fp32 matrix product on the same operands."""
     torch.manual_seed(0)

@@ -98,13 +98,9 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
         for (int ks = 0; ks < KS; ks++) kf[ks].u = *reinterpret_cast<const uint4*>(kp + ks * 16);
     };
 
-    const int first = (k_begin / KB) * KB;
-    Frag kf[KS], kn[KS];
-    if (first <= k_end) load_k(first, kf);
-    for (int key0 = first; key0 <= k_end; key0 += KB) {
-        // values of this block: for product step kk the lane needs keys key0 + 16 kk + 4 half + {0..3}
-        // and the same + 8, for dimension 32 db + col
-        Frag vf[NDB][2];
+    // values of a block: for product step kk the lane needs keys key0 + 16 kk + 4 half + {0..3}
+    // and the same + 8, for dimension 32 db + col
+    auto load_v = [&](int key0, Frag (*vf)[2]) {
 #pragma unroll
         for (int kk = 0; kk < 2; kk++) {
 #pragma unroll
@@ -118,8 +114,22 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
                     vf[db][kk].h[run] = *reinterpret_cast<const uint2*>(vp + (size_t)db * 32 * P);
             }
         }
+    };
+
+    // Keys and values of block b + 1 are requested before block b is worked on, so a wave always
+    // has a block's worth of loads (16 KB at head_dim 128) in flight.
+    const int first = (k_begin / KB) * KB;
+    Frag kf[KS], kn[KS], vf[NDB][2], vn[NDB][2];
+    if (first <= k_end) {
+        load_k(first, kf);
+        load_v(first, vf);
+    }
+    for (int key0 = first; key0 <= k_end; key0 += KB) {
         const bool more = key0 + KB <= k_end;
-        if (more) load_k(key0 + KB, kn);
+        if (more) {
+            load_k(key0 + KB, kn);
+            load_v(key0 + KB, vn);
+        }
 
         floatx16 st;
 #pragma unroll
@@ -171,6 +181,11 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
         if (more) {
 #pragma unroll
             for (int ks = 0; ks < KS; ks++) kf[ks] = kn[ks];
+#pragma unroll
+            for (int db = 0; db < NDB; db++) {
+                vf[db][0] = vn[db][0];
+                vf[db][1] = vn[db][1];
+            }
         }
     }
 

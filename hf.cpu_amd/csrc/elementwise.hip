@@ -134,9 +134,6 @@ extern "C" int hfa_rmsnorm(float* x, const float* w, void* out, int out_dtype, c
 }
 
 // ---- rotary encoding + cache store ------------------------------------------------------------
-// One block per token. Cosines and sines of the token's angles go to LDS once; the angle is
-// the fp32 product of the position and the fp32 inverse frequency.
-#define ROPE_MAX_HALF 256
 // If the q/k/v product left its result as partial sums ([splits][T][width] fp32), the kernel
 // finishes it on the way: every value it reads is the sum over the splits plus the bias, and the
 // rotated queries are written into qkv as if the product had stored them.
@@ -161,80 +158,48 @@ struct QkvSource {
     }
 };
 
+// One block per (token, head slot): slots 0 .. H-1 are the query heads, H .. H+G-1 the key
+// heads, H+G .. H+2G-1 the value heads, so that a single decoded token still spreads over the
+// machine. Cosines and sines of the token's angles are computed by each block that rotates;
+// the angle is the fp32 product of the position and the fp32 inverse frequency.
 template <typename T>
-__global__ void rope_store_kernel(T* __restrict__ qkv, int ld, const int* __restrict__ positions,
-                                  const float* __restrict__ inv_freq, int rot_dim, int H, int G, int D,
-                                  T* __restrict__ k_cache, T* __restrict__ v_cache,
-                                  const int* __restrict__ slot_map, int page_tokens,
-                                  const float* __restrict__ partial, int splits, const float* __restrict__ pbias,
-                                  int n_tokens) {
-    __shared__ float cs[ROPE_MAX_HALF], sn[ROPE_MAX_HALF];
-    const int t = blockIdx.x;
+__global__ __launch_bounds__(128) void rope_store_kernel(
+    T* __restrict__ qkv, int ld, const int* __restrict__ positions, const float* __restrict__ inv_freq, int rot_dim,
+    int H, int G, int D, T* __restrict__ k_cache, T* __restrict__ v_cache, const int* __restrict__ slot_map,
+    int page_tokens, const float* __restrict__ partial, int splits, const float* __restrict__ pbias, int n_tokens) {
+    const int t = blockIdx.x, hs = blockIdx.y;
+    const int half = rot_dim / 2, rest = D - rot_dim;
     const int width = (H + 2 * G) * D;
     QkvSource<T> in = {qkv + (size_t)t * ld, partial + (size_t)t * width, pbias, (size_t)n_tokens * width, splits};
-    const int half = rot_dim / 2;
-    if (half > 0) {
-        const float pos = (float)positions[t];
-        for (int i = threadIdx.x; i < half; i += blockDim.x) {
-            float s, c;
-            sincosf(pos * inv_freq[i], &s, &c);
-            cs[i] = c;
-            sn[i] = s;
-        }
-    }
-    __syncthreads();
     T* row = qkv + (size_t)t * ld;
-    // queries: rotate in place
-    if (half > 0) {
-        for (int it = threadIdx.x; it < H * half; it += blockDim.x) {
-            const int h = it / half, i = it - h * half;
-            T* p = row + h * D;
-            const float x0 = in.at(h * D + i), x1 = in.at(h * D + i + half);
-            p[i] = from_f32<T>(x0 * cs[i] - x1 * sn[i]);
-            p[i + half] = from_f32<T>(x0 * sn[i] + x1 * cs[i]);
+    const int slot = (G > 0 && slot_map) ? slot_map[t] : -1;
+    const int base = hs * D;                                  // first column of this head in the row
+    if (hs >= H + G) {                                        // a value head: copy, transposed inside the page
+        if (slot < 0) {
+            if (splits > 0)
+                for (int i = threadIdx.x; i < D; i += blockDim.x) row[base + i] = from_f32<T>(in.at(base + i));
+            return;
         }
-    }
-    if (splits > 0) {                                      // dimensions of q that are not rotated still need storing
-        const int rest = D - rot_dim;
-        for (int it = threadIdx.x; it < H * rest; it += blockDim.x) {
-            const int h = it / rest, i = rot_dim + (it - h * rest);
-            row[h * D + i] = from_f32<T>(in.at(h * D + i));
-        }
-    }
-    if (G == 0) return;
-    const int slot = slot_map ? slot_map[t] : -1;
-    T* krow = row + H * D;
-    T* vrow = krow + G * D;
-    const int ko = H * D, vo = (H + G) * D;               // where keys and values start in a row
-    if (slot < 0) {
-        // no cache row: still leave the rotated keys in place so the caller sees them
-        if (half > 0) {
-            for (int it = threadIdx.x; it < G * half; it += blockDim.x) {
-                const int g = it / half, i = it - g * half;
-                T* p = krow + g * D;
-                const float x0 = in.at(ko + g * D + i), x1 = in.at(ko + g * D + i + half);
-                p[i] = from_f32<T>(x0 * cs[i] - x1 * sn[i]);
-                p[i + half] = from_f32<T>(x0 * sn[i] + x1 * cs[i]);
-            }
-        }
+        const int c0 = (hs - H - G) * D;
+        T* vdst = v_cache + (size_t)(slot / page_tokens) * page_tokens * (G * D) + slot % page_tokens;
+        for (int i = threadIdx.x; i < D; i += blockDim.x)
+            vdst[(size_t)(c0 + i) * page_tokens] = from_f32<T>(in.at(base + i));
         return;
     }
-    T* kdst = k_cache + (size_t)slot * (G * D);
-    // values lie transposed inside their page: element c of the token at offset o is at c * page_tokens + o
-    T* vdst = v_cache + (size_t)(slot / page_tokens) * page_tokens * (G * D) + slot % page_tokens;
-    for (int it = threadIdx.x; it < G * half; it += blockDim.x) {
-        const int g = it / half, i = it - g * half;
-        const float x0 = in.at(ko + g * D + i), x1 = in.at(ko + g * D + i + half);
-        kdst[g * D + i] = from_f32<T>(x0 * cs[i] - x1 * sn[i]);
-        kdst[g * D + i + half] = from_f32<T>(x0 * sn[i] + x1 * cs[i]);
+    // a query or key head: rotate; keys go to the cache (or stay in the row if there is no cache row)
+    const bool is_key = hs >= H;
+    T* dst = (is_key && slot >= 0) ? k_cache + (size_t)slot * (G * D) + (hs - H) * D : row + base;
+    const float pos = half > 0 ? (float)positions[t] : 0.f;
+    for (int i = threadIdx.x; i < half; i += blockDim.x) {
+        float sn, cs;
+        sincosf(pos * inv_freq[i], &sn, &cs);
+        const float x0 = in.at(base + i), x1 = in.at(base + i + half);
+        dst[i] = from_f32<T>(x0 * cs - x1 * sn);
+        dst[i + half] = from_f32<T>(x0 * sn + x1 * cs);
     }
-    const int rest = D - rot_dim;   // dimensions that pass through
-    for (int it = threadIdx.x; it < G * rest; it += blockDim.x) {
-        const int g = it / rest, i = rot_dim + (it - g * rest);
-        kdst[g * D + i] = from_f32<T>(in.at(ko + g * D + i));
-    }
-    for (int it = threadIdx.x; it < G * D; it += blockDim.x)
-        vdst[(size_t)it * page_tokens] = from_f32<T>(in.at(vo + it));
+    if (splits > 0 || dst != row + base)                      // dimensions that are not rotated pass through
+        for (int i = rot_dim + threadIdx.x; i < D; i += blockDim.x) dst[i] = from_f32<T>(in.at(base + i));
+    (void)rest;
 }
 
 extern "C" int hfa_rope_store(void* qkv, int dtype, int ld, const int* positions, const float* inv_freq, int rot_dim,
@@ -244,21 +209,22 @@ extern "C" int hfa_rope_store(void* qkv, int dtype, int ld, const int* positions
     HFA_REQUIRE(n_tokens > 0 && n_heads > 0 && n_kv_heads >= 0 && head_dim > 0, "rope_store: bad sizes");
     HFA_REQUIRE(rot_dim >= 0 && rot_dim % 2 == 0 && rot_dim <= head_dim,
                 "rope_store: rot_dim %d must be even and at most head_dim %d", rot_dim, head_dim);
-    HFA_REQUIRE(rot_dim / 2 <= ROPE_MAX_HALF, "rope_store: rot_dim %d exceeds the kernel's limit %d", rot_dim,
-                2 * ROPE_MAX_HALF);
     HFA_REQUIRE(rot_dim == 0 || (positions && inv_freq), "rope_store: positions and inv_freq are needed");
     HFA_REQUIRE(ld >= (n_heads + 2 * n_kv_heads) * head_dim, "rope_store: row stride %d is too small", ld);
     HFA_REQUIRE(n_kv_heads == 0 || !slot_map || (k_cache && v_cache && page_tokens > 0),
                 "rope_store: no cache to store into");
     HFA_REQUIRE(dtype == HFA_F32 || dtype == HFA_BF16, "rope_store: unknown dtype %d", dtype);
     HFA_REQUIRE(splits >= 0 && (splits == 0 || partial), "rope_store: partial sums announced but not given");
+    HFA_REQUIRE(n_heads + 2 * n_kv_heads <= 65535, "rope_store: too many heads for the grid");
+    const dim3 grid(n_tokens, n_heads + 2 * n_kv_heads);
+    const int threads = head_dim >= 128 ? 128 : 64;
     if (dtype == HFA_F32)
-        rope_store_kernel<float><<<n_tokens, 256, 0, stream>>>((float*)qkv, ld, positions, inv_freq, rot_dim, n_heads,
+        rope_store_kernel<float><<<grid, threads, 0, stream>>>((float*)qkv, ld, positions, inv_freq, rot_dim, n_heads,
                                                                n_kv_heads, head_dim, (float*)k_cache,
                                                                (float*)v_cache, slot_map, page_tokens, partial,
                                                                splits, partial_bias, n_tokens);
     else
-        rope_store_kernel<bf16><<<n_tokens, 256, 0, stream>>>((bf16*)qkv, ld, positions, inv_freq, rot_dim, n_heads,
+        rope_store_kernel<bf16><<<grid, threads, 0, stream>>>((bf16*)qkv, ld, positions, inv_freq, rot_dim, n_heads,
                                                               n_kv_heads, head_dim, (bf16*)k_cache, (bf16*)v_cache,
                                                               slot_map, page_tokens, partial, splits, partial_bias,
                                                               n_tokens);

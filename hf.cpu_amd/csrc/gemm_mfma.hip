@@ -44,7 +44,7 @@ struct MfmaCfg {
     static_assert(TM % 32 == 0 && TN % 32 == 0 && BK % 16 == 0, "wave tiles are made of 32x32x16 products");
 };
 
-template <int BM, int BN, int BK, int WM, int WN, int MODE>
+template <int BM, int BN, int BK, int WM, int WN, int MODE, int PF>
 __global__ __launch_bounds__(WM* WN* WAVE) void gemm_mfma_kernel(
     const uint16_t* __restrict__ A, int lda, const uint16_t* __restrict__ W, int ldw,
     const float* __restrict__ bias, void* __restrict__ out, int ldo, int M, int N, int K, int k_per_split,
@@ -77,8 +77,11 @@ __global__ __launch_bounds__(WM* WN* WAVE) void gemm_mfma_kernel(
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
-    uint4 ra[C::A_CH], rw[C::W_CH];
-    auto gload = [&](int k0) {
+    // PF = 2 (small M, bandwidth-bound): two register sets, so that while tile t is multiplied out
+    // of LDS, tiles t + 1 and t + 2 are on their way from memory, which doubles the bytes in flight
+    // of a block. PF = 1 (large M): one set, fewer registers, more blocks per CU.
+    uint4 ra0[C::A_CH], rw0[C::W_CH], ra1[PF == 2 ? C::A_CH : 1], rw1[PF == 2 ? C::W_CH : 1];
+    auto gload = [&](uint4* ra, uint4* rw, int k0) {
 #pragma unroll
         for (int i = 0; i < C::A_CH; i++) {
             const int c = tid + i * C::NT, row = c / C::CPR, kk = k0 + (c % C::CPR) * 8;
@@ -94,7 +97,7 @@ __global__ __launch_bounds__(WM* WN* WAVE) void gemm_mfma_kernel(
             rw[i] = kk < kend ? *reinterpret_cast<const uint4*>(W + (size_t)gr * ldw + kk) : make_uint4(0, 0, 0, 0);
         }
     };
-    auto sstore = [&](int stage) {
+    auto sstore = [&](int stage, const uint4* ra, const uint4* rw) {
         uint16_t* sa = smem + stage * C::STAGE;
         uint16_t* sw = sa + BM * C::STRIDE;
 #pragma unroll
@@ -108,16 +111,9 @@ __global__ __launch_bounds__(WM* WN* WAVE) void gemm_mfma_kernel(
             *reinterpret_cast<uint4*>(sw + row * C::STRIDE + kc * 8) = rw[i];
         }
     };
-
-    gload(kbeg);
-    sstore(0);
-    __syncthreads();
-    int cur = 0;
-    for (int k0 = kbeg; k0 < kend; k0 += BK) {
-        const bool more = k0 + BK < kend;
-        if (more) gload(k0 + BK);
-        const uint16_t* sa = smem + cur * C::STAGE + (wm * C::TM + (lane & 31)) * C::STRIDE + (lane >> 5) * 8;
-        const uint16_t* sw = smem + cur * C::STAGE + (BM + wn * C::TN + (lane & 31)) * C::STRIDE + (lane >> 5) * 8;
+    auto compute = [&](int stage) {
+        const uint16_t* sa = smem + stage * C::STAGE + (wm * C::TM + (lane & 31)) * C::STRIDE + (lane >> 5) * 8;
+        const uint16_t* sw = smem + stage * C::STAGE + (BM + wn * C::TN + (lane & 31)) * C::STRIDE + (lane >> 5) * 8;
 #pragma unroll
         for (int kk = 0; kk < BK; kk += 16) {
             bf16x8 fa[C::FM], fw[C::FN];
@@ -131,9 +127,36 @@ __global__ __launch_bounds__(WM* WN* WAVE) void gemm_mfma_kernel(
                 for (int j = 0; j < C::FN; j++)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fw[j], acc[i][j], 0, 0, 0);
         }
-        if (more) sstore(cur ^ 1);
+    };
+
+    const int nk = (kend - kbeg + BK - 1) / BK;
+    gload(ra0, rw0, kbeg);
+    sstore(0, ra0, rw0);
+    if (nk > 1) gload(ra0, rw0, kbeg + BK);
+    if (PF == 2 && nk > 2) gload(ra1, rw1, kbeg + 2 * BK);
+    __syncthreads();
+    if (PF == 1) {
+        for (int t = 0; t < nk; t++) {
+            compute(t & 1);
+            if (t + 1 < nk) sstore((t + 1) & 1, ra0, rw0);
+            if (t + 2 < nk) gload(ra0, rw0, kbeg + (t + 2) * BK);
+            __syncthreads();
+        }
+    }
+    for (int t = 0; PF == 2 && t < nk; t += 2) {
+        compute(0);                                          // tile t
+        if (t + 1 < nk) {
+            sstore(1, ra0, rw0);                             // tile t + 1
+            if (t + 3 < nk) gload(ra0, rw0, kbeg + (t + 3) * BK);
+        }
         __syncthreads();
-        cur ^= 1;
+        if (t + 1 >= nk) break;
+        compute(1);                                          // tile t + 1
+        if (t + 2 < nk) {
+            sstore(0, ra1, rw1);                             // tile t + 2
+            if (t + 4 < nk) gload(ra1, rw1, kbeg + (t + 4) * BK);
+        }
+        __syncthreads();
     }
 
     // ---- epilogue: element r of a lane is row 8 * (r / 4) + 4 * (lane / 32) + r % 4, column lane % 32 ----
@@ -211,7 +234,7 @@ __global__ void gemm_finish_kernel(const float* __restrict__ partial, int splits
 template <int BM, int BN, int BK, int WM, int WN, int MODE>
 static int launch_cfg(const GemmArgs& g, void* out, int splits, int k_per_split) {
     using C = MfmaCfg<BM, BN, BK, WM, WN>;
-    auto kernel = gemm_mfma_kernel<BM, BN, BK, WM, WN, MODE>;
+    auto kernel = gemm_mfma_kernel<BM, BN, BK, WM, WN, MODE, (BM >= 128 ? 1 : 2)>;
     static bool configured = false;
     if (!configured) {
         hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM);

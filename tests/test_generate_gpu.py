@@ -174,3 +174,46 @@ def test_trace_run_program(gpu, models, tmp_path):
                          input=json.dumps({"step": 0, "entries": [{"id": "a", "tokens": list(range(100)), "want": []}],
                                            "end": []}) + "\n", text=True, capture_output=True, timeout=300)
     assert bad.returncode == 1 and "ERANGE" in bad.stderr
+
+
+def test_generation_survives_a_cache_that_is_too_small(gpu, models):
+    """Six requests that together need about twice the pages there are: the scheduler shrinks
+    prompt portions, preempts the newest running request when decoded tokens no longer fit, and
+    recomputes it later. Every request still ends with the tokens it gets when it runs alone."""
+    import hf_cpu_amd.session as S
+    cfg = helpers.CONFIG_A
+    prompts = list(helpers.random_requests(cfg, [30, 44, 25, 51, 38, 47], seed=12).values())
+    roomy = S.Session(models["A"], dtype="float32", ctx_max=128, batch=32, page_size=16, max_seqs=8)
+    want = [roomy.generate(p, temp=0.0, max_tokens=40)[0].tokens for p in prompts]
+    tight = S.Session(models["A"], dtype="float32", ctx_max=128, batch=32, page_size=16, max_seqs=8, kv_tokens=256)
+    gens = tight.generate(prompts, temp=0.0, max_tokens=40)
+    assert [g.tokens for g in gens] == want and all(g.stop == "length" for g in gens)
+    assert sum(g.preemptions for g in gens) > 0, "the cache was meant to run out"
+    tight.engine.manager.check()
+    assert not tight.engine.manager.held and tight.engine.manager.pools[0].reused > 0
+    # a pool smaller than --ctx-max lowers the context limit to what it holds: stop=ctx, not a failure
+    tiny = S.Session(models["A"], dtype="float32", ctx_max=128, batch=32, page_size=16, max_seqs=4, kv_tokens=48)
+    gens = tiny.generate([prompts[0], prompts[1]], temp=0.0, max_tokens=40)
+    assert [g.stop for g in gens] == ["ctx", "ctx"] and all(g.error is None for g in gens)
+    assert [g.prompt_tokens + len(g.tokens) for g in gens] == [48, 48]
+    assert not tiny.engine.manager.held
+
+
+def test_real_layer_sizes_in_both_precisions(gpu, tmp_path):
+    """One layer with the sizes of the 7B shape (hidden 3584, 28 query heads on 4 key/value heads of
+    128, feed-forward 18944; the vocabulary cut to 4096 to keep the plain implementation quick):
+    fp32 against the plain implementation, bf16 against the plain implementation on weights rounded
+    to bf16, with a prompt in portions and decoded tokens. These are the shapes the matrix-core
+    kernels are tuned for and none of the tiny configurations reaches them."""
+    import hf_cpu_amd
+    cfg = dict(architectures=["Qwen2ForCausalLM"], num_hidden_layers=1, hidden_size=3584, num_attention_heads=28,
+               num_key_value_heads=4, head_dim=128, intermediate_size=18944, vocab_size=4096, rope_theta=1e6,
+               rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=512)
+    d = helpers.make_model_dir(str(tmp_path / "m"), cfg, seed=3)
+    reqs = helpers.random_requests(cfg, [70, 45], seed=1)
+    steps = helpers.trace_mixed(reqs, seed=4, max_live=2, decode_tail=6)
+    for dtype, tol, rounded in (("float32", 1e-5, False), ("bfloat16", 2e-2, True)):
+        want = helpers.plain_logits(d, reqs, round_weights_bf16=rounded)
+        engine = hf_cpu_amd.load_engine(d, dtype=dtype, page_tokens=16, max_tokens=256, max_seqs=2)
+        worst = helpers.compare(helpers.run_trace_in_engine(engine, steps), want, tol, "7B layer " + dtype)
+        print(f"7B-sized layer, {dtype}: worst relative difference {worst:.2e}")

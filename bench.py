@@ -63,6 +63,8 @@ def main():
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
     ap.add_argument("--prefill-reps", type=int, default=3)
+    ap.add_argument("--only", choices=["prefill", "decode"], default=None,
+                    help="run one phase only and print a short line (for profiling a phase by itself)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this engine runs on one GPU; --gpus must be 1")
@@ -97,7 +99,7 @@ def main():
 
     # ---- prefill: one prompt of 2,048 tokens in one step, logits for its last token ----
     times = []
-    for rep in range(args.prefill_reps + 1):
+    for rep in range(0 if args.only == "decode" else args.prefill_reps + 1):
         p = prompt()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
@@ -106,8 +108,14 @@ def main():
         torch.cuda.synchronize()
         times.append(time.perf_counter() - t0)
         eng.release("prefill")
-    pre_s = sorted(times[1:])[len(times[1:]) // 2]            # the first run warms up
-    print(f"[bench] prefill {PROMPT} tokens: {pre_s * 1e3:.1f} ms", file=sys.stderr, flush=True)
+    if args.only == "decode":
+        pre_s = float("nan")
+    else:
+        pre_s = sorted(times[1:])[len(times[1:]) // 2]        # the first run warms up
+        print(f"[bench] prefill {PROMPT} tokens: {pre_s * 1e3:.1f} ms", file=sys.stderr, flush=True)
+    if args.only == "prefill":
+        print(json.dumps({"phase": "prefill", "tokens": PROMPT, "ms": round(pre_s * 1e3, 3)}))
+        return 0
 
     def decode(batch, steps, warmup):
         ids = [("d", i) for i in range(batch)]
@@ -135,6 +143,9 @@ def main():
     ms_step = dt / args.steps * 1e3
     value = args.batch * args.steps / dt
     print(f"[bench] decode batch {args.batch}: {ms_step:.3f} ms/step", file=sys.stderr, flush=True)
+    if args.only == "decode":
+        print(json.dumps({"phase": "decode", "batch": args.batch, "ms_per_step": round(ms_step, 4)}))
+        return 0
     mean_ctx = PROMPT + args.warmup + (args.steps + 1) / 2.0
     nbytes = decode_bytes(shape, elem, args.batch, mean_ctx)
     achieved = nbytes / (dt / args.steps) / 1e9

@@ -17,12 +17,13 @@
 //
 // When a step has few columns (decode) the key range is cut into chunks over blockIdx.z; each
 // wave writes (max, sum, unnormalised output) for its chunk and a second kernel merges them in
-// chunk order. No LDS, no barrier: every operand comes from global memory in operand layout.
+// chunk order. Keys and values come from global memory in operand layout, without a barrier.
 #include "attention_internal.h"
 #include "common.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 #define KB 32
 #define NEG_BIG (-1.0e30f)
@@ -75,13 +76,16 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
     int vhi = col_ok ? (pos < k_end ? pos : k_end) : -1;
     const int* bt = block_table + (size_t)token_slot[t0] * max_blocks;
 
-    Frag qf[KS];
+    // The query fragments live in LDS (each lane reads back what it wrote): registers are
+    // needed for the keys and values in flight.
+    __shared__ uint4 q_s[KS * WAVE];
     {
         const uint16_t* qp = q + (size_t)my_tok * ldq + my_head * D + half * 8;
 #pragma unroll
         for (int ks = 0; ks < KS; ks++)
-            qf[ks].u = col_ok ? *reinterpret_cast<const uint4*>(qp + ks * 16) : make_uint4(0, 0, 0, 0);
+            q_s[ks * WAVE + lane] = col_ok ? *reinterpret_cast<const uint4*>(qp + ks * 16) : make_uint4(0, 0, 0, 0);
     }
+    __syncthreads();
     floatx16 o[NDB];
 #pragma unroll
     for (int db = 0; db < NDB; db++)
@@ -89,18 +93,18 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
         for (int r = 0; r < 16; r++) o[db][r] = 0.f;
     float m = NEG_BIG, l = 0.f;
 
-    auto load_k = [&](int key0, Frag* kf) {
+    auto load_k = [&](int key0, Frag (&kf)[KS]) {
         int key = key0 + col;                              // this lane's row of the key block
         key = key < hi ? key : hi;                         // rows past the end repeat the last key; they are masked
         const int page = bt[key / P];
-        const uint16_t* kp = kc + ((size_t)page * P + key % P) * kvw + g * D + half * 8;
+        const unsigned off = (unsigned)(page * P + key % P) * (unsigned)kvw + (unsigned)(g * D + half * 8);
 #pragma unroll
-        for (int ks = 0; ks < KS; ks++) kf[ks].u = *reinterpret_cast<const uint4*>(kp + ks * 16);
+        for (int ks = 0; ks < KS; ks++) kf[ks].u = *reinterpret_cast<const uint4*>(kc + (off + (unsigned)(ks * 16)));
     };
 
     // values of a block: for product step kk the lane needs keys key0 + 16 kk + 4 half + {0..3}
     // and the same + 8, for dimension 32 db + col
-    auto load_v = [&](int key0, Frag (*vf)[2]) {
+    auto load_v = [&](int key0, Frag (&vf)[NDB][2]) {
 #pragma unroll
         for (int kk = 0; kk < 2; kk++) {
 #pragma unroll
@@ -108,35 +112,28 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
                 int ka = key0 + 16 * kk + 8 * run + 4 * half;
                 ka = ka < (hi & ~3) ? ka : (hi & ~3);       // runs past the end are masked; read a valid one
                 const int page = bt[ka / P];
-                const uint16_t* vp = vc + (size_t)page * P * kvw + (size_t)(g * D + col) * P + ka % P;
+                // element offsets fit 32 bits (checked on the host), so one base serves every load
+                const unsigned off = (unsigned)page * (unsigned)(P * kvw) + (unsigned)((g * D + col) * P + ka % P);
 #pragma unroll
                 for (int db = 0; db < NDB; db++)
-                    vf[db][kk].h[run] = *reinterpret_cast<const uint2*>(vp + (size_t)db * 32 * P);
+                    vf[db][kk].h[run] = *reinterpret_cast<const uint2*>(vc + (off + (unsigned)(db * 32 * P)));
             }
         }
     };
 
-    // Keys and values of block b + 1 are requested before block b is worked on, so a wave always
-    // has a block's worth of loads (16 KB at head_dim 128) in flight.
-    const int first = (k_begin / KB) * KB;
-    Frag kf[KS], kn[KS], vf[NDB][2], vn[NDB][2];
-    if (first <= k_end) {
-        load_k(first, kf);
-        load_v(first, vf);
-    }
-    for (int key0 = first; key0 <= k_end; key0 += KB) {
-        const bool more = key0 + KB <= k_end;
-        if (more) {
-            load_k(key0 + KB, kn);
-            load_v(key0 + KB, vn);
-        }
-
+    // One block of 32 keys in two halves, so that the registers of its keys can be refilled as
+    // soon as the scores are formed: scores + online softmax, then weighted values.
+    Frag pf[2];
+    auto scores = [&](int key0, const Frag (&kf)[KS]) {
         floatx16 st;
 #pragma unroll
         for (int r = 0; r < 16; r++) st[r] = 0.f;
 #pragma unroll
-        for (int ks = 0; ks < KS; ks++) st = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ks].v, qf[ks].v, st, 0, 0, 0);
-
+        for (int ks = 0; ks < KS; ks++) {
+            Frag qf;
+            qf.u = q_s[ks * WAVE + lane];
+            st = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ks].v, qf.v, st, 0, 0, 0);
+        }
         // element r of the lane: key key0 + 8 (r / 4) + 4 half + r % 4, this lane's column
         float mx = NEG_BIG;
 #pragma unroll
@@ -163,8 +160,6 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
         for (int db = 0; db < NDB; db++)
 #pragma unroll
             for (int r = 0; r < 16; r++) o[db][r] *= corr;
-
-        Frag pf[2];
 #pragma unroll
         for (int kk = 0; kk < 2; kk++) {
             uint32_t w[4];
@@ -173,20 +168,33 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
                 w[e] = (uint32_t)bf16_bits(st[8 * kk + 2 * e]) | ((uint32_t)bf16_bits(st[8 * kk + 2 * e + 1]) << 16);
             pf[kk].u = make_uint4(w[0], w[1], w[2], w[3]);
         }
+    };
+    auto values = [&](const Frag (&vf)[NDB][2]) {
 #pragma unroll
         for (int kk = 0; kk < 2; kk++)
 #pragma unroll
             for (int db = 0; db < NDB; db++)
                 o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[db][kk].v, pf[kk].v, o[db], 0, 0, 0);
-        if (more) {
-#pragma unroll
-            for (int ks = 0; ks < KS; ks++) kf[ks] = kn[ks];
-#pragma unroll
-            for (int db = 0; db < NDB; db++) {
-                vf[db][0] = vn[db][0];
-                vf[db][1] = vn[db][1];
-            }
-        }
+    };
+
+    // Two register sets in rotation. The keys of block b + 2 are requested as soon as the scores
+    // of block b are formed, its values as soon as block b's values are used, so between one and
+    // two blocks (16 to 32 KB a wave at head_dim 128) are always on their way.
+    const int first = (k_begin / KB) * KB;
+    const int nb = first <= k_end ? (k_end - first) / KB + 1 : 0;
+    Frag k0f[KS], k1f[KS], v0f[NDB][2], v1f[NDB][2];
+    if (nb > 0) { load_k(first, k0f); load_v(first, v0f); }
+    if (nb > 1) { load_k(first + KB, k1f); load_v(first + KB, v1f); }
+    for (int b = 0; b < nb; b += 2) {
+        scores(first + b * KB, k0f);
+        if (b + 2 < nb) load_k(first + (b + 2) * KB, k0f);
+        values(v0f);
+        if (b + 2 < nb) load_v(first + (b + 2) * KB, v0f);
+        if (b + 1 >= nb) break;
+        scores(first + (b + 1) * KB, k1f);
+        if (b + 3 < nb) load_k(first + (b + 3) * KB, k1f);
+        values(v1f);
+        if (b + 3 < nb) load_v(first + (b + 3) * KB, v1f);
     }
 
     if (!col_ok) return;
@@ -220,6 +228,199 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
     }
 }
 
+// ---- prompt portions: four waves share the keys and values of a block through LDS ---------------
+// A block of four waves owns 4 x (tokens per wave) consecutive tokens of one request and one
+// key/value head; wave w takes its own 32 columns as above. Every block of 32 keys is fetched
+// once by the 256 threads (keys as rows of K, values as rows of V^T), stored in LDS with padded
+// rows (272 and 72 bytes: the fragment reads of a wave are conflict-free) and read by all four
+// waves, so L2-to-CU traffic drops fourfold against the kernel above and several waves per SIMD
+// overlap their matrix products and softmax. Two LDS stages, one barrier per key block. Tiles
+// are numbered from the end of each request backwards, so the longest ones start first.
+#define PKS 136      // LDS row of a key: 128 dims + 8 pad (elements)
+#define PVS 36       // LDS row of a value dimension: 32 keys + 4 pad (elements)
+
+template <int NDB>
+__global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) void attn_prefill_kernel(
+    const uint16_t* __restrict__ q, int ldq, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc, int kvw,
+    const int* __restrict__ block_table, int max_blocks, const int* __restrict__ token_slot,
+    const int* __restrict__ positions, const int* __restrict__ q_start, int n_seqs, uint16_t* __restrict__ out,
+    int ldo, int P, int window, float scale_log2e, int tpt, int cpt) {
+    constexpr int D = NDB * 32, KS = D / 16, KROW = D + 8;
+    __shared__ __attribute__((aligned(16))) uint16_t k_s[2][KB * KROW];
+    __shared__ __attribute__((aligned(16))) uint16_t v_s[2][D * PVS];
+    const int tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
+    const int col = lane & 31, half = lane >> 5;
+    const int g = blockIdx.y;
+    const int tile_tokens = 4 * tpt;
+
+    int tile = blockIdx.x, t0 = -1, t_end = 0;
+    for (int s = 0; s < n_seqs; s++) {
+        const int a = q_start[s], b = q_start[s + 1];
+        const int nt = (b - a + tile_tokens - 1) / tile_tokens;
+        if (tile < nt) {
+            const int rt = nt - 1 - tile;                   // last tile of the request first
+            t0 = a + rt * tile_tokens;
+            t_end = t0 + tile_tokens < b ? t0 + tile_tokens : b;
+            break;
+        }
+        tile -= nt;
+    }
+    if (t0 < 0) return;                                    // uniform over the block: no barrier is skipped
+
+    // this wave's tokens and columns
+    const int w0 = t0 + wave * tpt;
+    const int w_end = w0 + tpt < t_end ? w0 + tpt : t_end;
+    const int n_cols = w_end > w0 ? (w_end - w0) * cpt : 0;
+    const bool col_ok = col < n_cols;
+    const int my_tok = col_ok ? w0 + col / cpt : t0;
+    const int my_head = g * cpt + (col_ok ? col % cpt : 0);
+    const int pos = positions[my_tok];
+    const int pos_first = positions[t0], hi = positions[t_end - 1];
+    const int k_begin = window > 0 && pos_first - window + 1 > 0 ? pos_first - window + 1 : 0;
+    const int vlo = window > 0 && pos - window + 1 > k_begin ? pos - window + 1 : k_begin;
+    const int vhi = col_ok ? pos : -1;
+    const int* bt = block_table + (size_t)token_slot[t0] * max_blocks;
+
+    // query fragments in LDS, each lane reading back what it wrote (ordered by the barrier below)
+    __shared__ uint4 q_s[4][KS * WAVE];
+    {
+        const uint16_t* qp = q + (size_t)my_tok * ldq + my_head * D + half * 8;
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++)
+            q_s[wave][ks * WAVE + lane] = col_ok ? *reinterpret_cast<const uint4*>(qp + ks * 16) : make_uint4(0, 0, 0, 0);
+    }
+    floatx16 o[NDB];
+#pragma unroll
+    for (int db = 0; db < NDB; db++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) o[db][r] = 0.f;
+    float m = NEG_BIG, l = 0.f;
+
+    // global -> registers -> LDS. Keys: 32 rows of D elements = 4 D chunks of 16 bytes.
+    // Values: D rows of 32 keys = 4 D chunks of 8 keys. Each thread takes up to NCH of both.
+    constexpr int TOT = 4 * D, NCH = (TOT + 255) / 256;
+    u32x4 rk[NCH];
+    uint2 rv[NCH][2];
+    auto gload = [&](int key0) {
+#pragma unroll
+        for (int i = 0; i < NCH; i++) {
+            const int c = tid + i * 256;
+            if (c >= TOT) break;
+            {   // key chunk: row c / (D / 8), 16-byte piece c % (D / 8)
+                int key = key0 + c / (D / 8);
+                key = key < hi ? key : hi;
+                const int page = bt[key / P];
+                const unsigned off = (unsigned)(page * P + key % P) * (unsigned)kvw + (unsigned)(g * D + (c % (D / 8)) * 8);
+                rk[i] = *reinterpret_cast<const u32x4*>(kc + off);
+            }
+            {   // value chunk: dimension c / 4, keys key0 + 8 (c % 4) .. + 7
+                int ka = key0 + 8 * (c % 4);
+                ka = ka < (hi & ~7) ? ka : (hi & ~7);
+                const int page = bt[ka / P];
+                const unsigned off = (unsigned)page * (unsigned)(P * kvw) + (unsigned)((g * D + c / 4) * P + ka % P);
+                const uint4 v = *reinterpret_cast<const uint4*>(vc + off);
+                rv[i][0] = make_uint2(v.x, v.y);
+                rv[i][1] = make_uint2(v.z, v.w);
+            }
+        }
+    };
+    auto sstore = [&](int stage) {
+#pragma unroll
+        for (int i = 0; i < NCH; i++) {
+            const int c = tid + i * 256;
+            if (c >= TOT) break;
+            *reinterpret_cast<u32x4*>(&k_s[stage][(c / (D / 8)) * KROW + (c % (D / 8)) * 8]) = rk[i];
+            uint2* dst = reinterpret_cast<uint2*>(&v_s[stage][(c / 4) * PVS + 8 * (c % 4)]);
+            dst[0] = rv[i][0];
+            dst[1] = rv[i][1];
+        }
+    };
+
+    const int first = (k_begin / KB) * KB;
+    const int nb = (hi - first) / KB + 1;
+    gload(first);
+    sstore(0);
+    __syncthreads();
+    for (int b = 0; b < nb; b++) {
+        const int key0 = first + b * KB, stage = b & 1;
+        if (b + 1 < nb) gload(key0 + KB);
+        // A wave whose columns all end before this block skips the math. The test is made by all
+        // lanes together: the matrix products need every lane, also those of unused columns.
+        const bool wave_sees = __any(key0 <= vhi) != 0;
+        if (wave_sees) {
+            const uint16_t* ks_ = &k_s[stage][col * KROW + half * 8];
+            floatx16 st;
+#pragma unroll
+            for (int r = 0; r < 16; r++) st[r] = 0.f;
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++) {
+                Frag kf, qf;
+                kf.u = *reinterpret_cast<const uint4*>(ks_ + ks * 16);
+                qf.u = q_s[wave][ks * WAVE + lane];
+                st = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf.v, qf.v, st, 0, 0, 0);
+            }
+            float mx = NEG_BIG;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int kr = key0 + 8 * (r / 4) + 4 * half + (r % 4);
+                const bool vis = kr >= vlo && kr <= vhi;
+                st[r] = vis ? st[r] * scale_log2e : NEG_BIG;
+                mx = fmaxf(mx, st[r]);
+            }
+            mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+            const float mn = fmaxf(m, mx);
+            const float corr = exp2f(m - mn);
+            float psum = 0.f;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const float p = st[r] > 0.5f * NEG_BIG ? exp2f(st[r] - mn) : 0.f;
+                st[r] = p;
+                psum += p;
+            }
+            psum += __shfl_xor(psum, 32, WAVE);
+            l = l * corr + psum;
+            m = mn;
+#pragma unroll
+            for (int db = 0; db < NDB; db++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) o[db][r] *= corr;
+            Frag pf[2];
+#pragma unroll
+            for (int kk = 0; kk < 2; kk++) {
+                uint32_t w[4];
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    w[e] = (uint32_t)bf16_bits(st[8 * kk + 2 * e]) | ((uint32_t)bf16_bits(st[8 * kk + 2 * e + 1]) << 16);
+                pf[kk].u = make_uint4(w[0], w[1], w[2], w[3]);
+            }
+#pragma unroll
+            for (int kk = 0; kk < 2; kk++)
+#pragma unroll
+                for (int db = 0; db < NDB; db++) {
+                    const uint16_t* vs_ = &v_s[stage][(32 * db + col) * PVS + 16 * kk + 4 * half];
+                    Frag vf;
+                    vf.h[0] = *reinterpret_cast<const uint2*>(vs_);
+                    vf.h[1] = *reinterpret_cast<const uint2*>(vs_ + 8);
+                    o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf.v, pf[kk].v, o[db], 0, 0, 0);
+                }
+        }
+        if (b + 1 < nb) sstore(stage ^ 1);
+        __syncthreads();
+    }
+    if (!col_ok) return;
+    const float inv = 1.0f / l;
+    uint16_t* dst = out + (size_t)my_tok * ldo + my_head * D;
+#pragma unroll
+    for (int db = 0; db < NDB; db++)
+#pragma unroll
+        for (int rg = 0; rg < 4; rg++) {
+            uint2 v;
+            v.x = (uint32_t)bf16_bits(o[db][4 * rg] * inv) | ((uint32_t)bf16_bits(o[db][4 * rg + 1] * inv) << 16);
+            v.y = (uint32_t)bf16_bits(o[db][4 * rg + 2] * inv) | ((uint32_t)bf16_bits(o[db][4 * rg + 3] * inv) << 16);
+            *reinterpret_cast<uint2*>(dst + 32 * db + 8 * rg + 4 * half) = v;
+        }
+}
+
 // out[t, h, :] = sum_c o_c 2^(m_c - M) / sum_c l_c 2^(m_c - M), chunks in ascending order.
 // Lanes first share the chunks (maximum, weights, sum), then the dimensions; the loads of the
 // second loop do not depend on one another.
@@ -251,7 +452,8 @@ __global__ __launch_bounds__(WAVE) void attn_merge_kernel(const float* __restric
 bool attn_mfma_supports(const AttnArgs& a) {
     const int group = a.n_heads / a.n_kv_heads;
     return a.head_dim % 32 == 0 && a.head_dim <= 128 && a.page_tokens % 4 == 0 && group <= 32 && a.q_start != nullptr &&
-           a.ldq % 8 == 0 && a.ldo % 4 == 0 && a.kv_width % 8 == 0 && ((uintptr_t)a.q & 15) == 0 &&
+           a.ldq % 8 == 0 && a.ldo % 4 == 0 && a.kv_width % 8 == 0 && a.kv_width * a.page_tokens < (1 << 20) &&
+           ((uintptr_t)a.q & 15) == 0 &&
            ((uintptr_t)a.out & 7) == 0 && ((uintptr_t)a.k_cache & 15) == 0 && ((uintptr_t)a.v_cache & 15) == 0;
 }
 
@@ -273,9 +475,30 @@ static int launch_ndb(const AttnArgs& a, int tiles, int tpt, int cpt, int chunk_
     return 0;
 }
 
+template <int NDB>
+static int launch_prefill(const AttnArgs& a, int tpt, int cpt) {
+    const int tile_tokens = 4 * tpt;
+    dim3 grid((a.n_tokens + tile_tokens - 1) / tile_tokens + a.n_seqs, a.n_kv_heads);
+    attn_prefill_kernel<NDB><<<grid, 4 * WAVE, 0, a.stream>>>(
+        (const uint16_t*)a.q, a.ldq, (const uint16_t*)a.k_cache, (const uint16_t*)a.v_cache, a.kv_width, a.block_table,
+        a.max_blocks, a.token_slot, a.positions, a.q_start, a.n_seqs, (uint16_t*)a.out, a.ldo, a.page_tokens,
+        a.window, a.scale * 1.4426950408889634f, tpt, cpt);
+    HFA_LAUNCH_CHECK("attn_prefill");
+    return 0;
+}
+
 int attn_mfma_launch(const AttnArgs& a) {
     const int cpt = a.n_heads / a.n_kv_heads;              // columns per token: the heads of a group
     const int tpt = 32 / cpt;                              // tokens per tile
+    // Steps with prompt portions: the kernel that shares keys and values between four waves.
+    if (a.max_q_len >= 16 && a.page_tokens % 8 == 0) {
+        switch (a.head_dim / 32) {
+            case 1: return launch_prefill<1>(a, tpt, cpt);
+            case 2: return launch_prefill<2>(a, tpt, cpt);
+            case 3: return launch_prefill<3>(a, tpt, cpt);
+            default: return launch_prefill<4>(a, tpt, cpt);
+        }
+    }
     const int tiles = (a.n_tokens + tpt - 1) / tpt + a.n_seqs;
     // Few waves and long contexts: cut the keys into chunks so that the machine is full.
     const long waves = (long)((a.n_tokens + tpt - 1) / tpt) * a.n_kv_heads;

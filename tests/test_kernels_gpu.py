@@ -314,6 +314,9 @@ def test_paged_attention(ops32, dtype, H, G, D, page, window):
     (14, 2, 64, 16, 300, [1000, 333], [1, 40]),                          # window shorter than the context
     (8, 1, 96, 8, 0, [257, 31], [9, 31]),                                # one key/value head, 8 query heads
     (32, 1, 32, 4, 0, [70], [3]),                                        # 32 heads on one key/value head
+    (28, 4, 128, 16, 0, [700, 90, 333, 64], [100, 90, 17, 1]),           # portions of several prompts beside a decoded token
+    (12, 4, 64, 8, 50, [400, 130], [130, 130]),                          # portions longer than the window
+    (6, 2, 96, 32, 0, [300], [37]),                                      # pages of 32 tokens
 ])
 def test_paged_attention_on_matrix_cores(ops16, H, G, D, page, window, lengths, q_lens):
     """bf16 with head_dim a multiple of 32: long contexts (many key blocks, split into chunks when

@@ -26,6 +26,7 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 #define KB 32
+#define PG_MAX 512
 #define NEG_BIG (-1.0e30f)
 
 union Frag {
@@ -40,13 +41,19 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ token_slot,
     const int* __restrict__ positions, const int* __restrict__ q_start, int n_seqs, uint16_t* __restrict__ out,
     int ldo, float* __restrict__ partial, int H, int P, int window, float scale_log2e, int tpt, int cpt,
-    int chunk_keys, int n_chunks) {
+    int chunk_keys, int n_chunks, int one_tile_each) {
     constexpr int D = NDB * 32, KS = D / 16;
     const int lane = threadIdx.x, col = lane & 31, half = lane >> 5;
     const int g = blockIdx.y, chunk = blockIdx.z;
 
     // ---- the tile's request and tokens: tiles are numbered request by request ----
     int tile = blockIdx.x, t0 = -1, t_end = 0;
+    if (one_tile_each) {                                   // no request has more tokens than a tile: tile s is request s
+        if (tile < n_seqs) {
+            t0 = q_start[tile];
+            t_end = q_start[tile + 1];
+        }
+    } else
     for (int s = 0; s < n_seqs; s++) {
         const int a = q_start[s], b = q_start[s + 1];
         const int nt = (b - a + tpt - 1) / tpt;
@@ -93,10 +100,22 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
         for (int r = 0; r < 16; r++) o[db][r] = 0.f;
     float m = NEG_BIG, l = 0.f;
 
+    // The page ids of the wave's key range go to LDS once (up to PG_MAX pages), so that a block's
+    // loads do not wait for a block-table load first.
+    __shared__ int pg_s[PG_MAX];
+    const int pb0 = ((k_begin / KB) * KB) / P;
+    const int k_top = (k_end / KB) * KB + KB - 1 < hi ? (k_end / KB) * KB + KB - 1 : hi;   // last key any load touches
+    const int n_pg = k_top / P - pb0 + 1;
+    const bool pg_lds = n_pg <= PG_MAX;
+    if (pg_lds)
+        for (int i = lane; i < n_pg; i += WAVE) pg_s[i] = bt[pb0 + i];
+    __syncthreads();
+    auto page_of = [&](int key) { return pg_lds ? pg_s[key / P - pb0] : bt[key / P]; };
+
     auto load_k = [&](int key0, Frag (&kf)[KS]) {
         int key = key0 + col;                              // this lane's row of the key block
         key = key < hi ? key : hi;                         // rows past the end repeat the last key; they are masked
-        const int page = bt[key / P];
+        const int page = page_of(key);
         const unsigned off = (unsigned)(page * P + key % P) * (unsigned)kvw + (unsigned)(g * D + half * 8);
 #pragma unroll
         for (int ks = 0; ks < KS; ks++) kf[ks].u = *reinterpret_cast<const uint4*>(kc + (off + (unsigned)(ks * 16)));
@@ -111,7 +130,7 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
             for (int run = 0; run < 2; run++) {
                 int ka = key0 + 16 * kk + 8 * run + 4 * half;
                 ka = ka < (hi & ~3) ? ka : (hi & ~3);       // runs past the end are masked; read a valid one
-                const int page = bt[ka / P];
+                const int page = page_of(ka);
                 // element offsets fit 32 bits (checked on the host), so one base serves every load
                 const unsigned off = (unsigned)page * (unsigned)(P * kvw) + (unsigned)((g * D + col) * P + ka % P);
 #pragma unroll
@@ -185,16 +204,26 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
     Frag k0f[KS], k1f[KS], v0f[NDB][2], v1f[NDB][2];
     if (nb > 0) { load_k(first, k0f); load_v(first, v0f); }
     if (nb > 1) { load_k(first + KB, k1f); load_v(first + KB, v1f); }
+    // The scheduling barriers keep the compiler from sinking the loads towards their use: they
+    // are issued exactly here, a block and a half ahead.
     for (int b = 0; b < nb; b += 2) {
         scores(first + b * KB, k0f);
+        __builtin_amdgcn_sched_barrier(0);
         if (b + 2 < nb) load_k(first + (b + 2) * KB, k0f);
+        __builtin_amdgcn_sched_barrier(0);
         values(v0f);
+        __builtin_amdgcn_sched_barrier(0);
         if (b + 2 < nb) load_v(first + (b + 2) * KB, v0f);
+        __builtin_amdgcn_sched_barrier(0);
         if (b + 1 >= nb) break;
         scores(first + (b + 1) * KB, k1f);
+        __builtin_amdgcn_sched_barrier(0);
         if (b + 3 < nb) load_k(first + (b + 3) * KB, k1f);
+        __builtin_amdgcn_sched_barrier(0);
         values(v1f);
+        __builtin_amdgcn_sched_barrier(0);
         if (b + 3 < nb) load_v(first + (b + 3) * KB, v1f);
+        __builtin_amdgcn_sched_barrier(0);
     }
 
     if (!col_ok) return;
@@ -296,6 +325,16 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
         for (int r = 0; r < 16; r++) o[db][r] = 0.f;
     float m = NEG_BIG, l = 0.f;
 
+    // page ids of the block's key range in LDS (see above)
+    __shared__ int pg_s[PG_MAX];
+    const int pb0 = ((k_begin / KB) * KB) / P;
+    const int n_pg = hi / P - pb0 + 1;
+    const bool pg_lds = n_pg <= PG_MAX;
+    if (pg_lds)
+        for (int i = tid; i < n_pg; i += 4 * WAVE) pg_s[i] = bt[pb0 + i];
+    __syncthreads();
+    auto page_of = [&](int key) { return pg_lds ? pg_s[key / P - pb0] : bt[key / P]; };
+
     // global -> registers -> LDS. Keys: 32 rows of D elements = 4 D chunks of 16 bytes.
     // Values: D rows of 32 keys = 4 D chunks of 8 keys. Each thread takes up to NCH of both.
     constexpr int TOT = 4 * D, NCH = (TOT + 255) / 256;
@@ -309,14 +348,14 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
             {   // key chunk: row c / (D / 8), 16-byte piece c % (D / 8)
                 int key = key0 + c / (D / 8);
                 key = key < hi ? key : hi;
-                const int page = bt[key / P];
+                const int page = page_of(key);
                 const unsigned off = (unsigned)(page * P + key % P) * (unsigned)kvw + (unsigned)(g * D + (c % (D / 8)) * 8);
                 rk[i] = *reinterpret_cast<const u32x4*>(kc + off);
             }
             {   // value chunk: dimension c / 4, keys key0 + 8 (c % 4) .. + 7
                 int ka = key0 + 8 * (c % 4);
                 ka = ka < (hi & ~7) ? ka : (hi & ~7);
-                const int page = bt[ka / P];
+                const int page = page_of(ka);
                 const unsigned off = (unsigned)page * (unsigned)(P * kvw) + (unsigned)((g * D + c / 4) * P + ka % P);
                 const uint4 v = *reinterpret_cast<const uint4*>(vc + off);
                 rv[i][0] = make_uint2(v.x, v.y);
@@ -465,12 +504,13 @@ static int launch_ndb(const AttnArgs& a, int tiles, int tpt, int cpt, int chunk_
         attn_mfma_kernel<NDB, true><<<grid, WAVE, 0, a.stream>>>(
             (const uint16_t*)a.q, a.ldq, (const uint16_t*)a.k_cache, (const uint16_t*)a.v_cache, a.kv_width,
             a.block_table, a.max_blocks, a.token_slot, a.positions, a.q_start, a.n_seqs, (uint16_t*)a.out, a.ldo,
-            (float*)a.workspace, a.n_heads, a.page_tokens, a.window, sl, tpt, cpt, chunk_keys, n_chunks);
+            (float*)a.workspace, a.n_heads, a.page_tokens, a.window, sl, tpt, cpt, chunk_keys, n_chunks,
+            a.max_q_len <= tpt);
     else
         attn_mfma_kernel<NDB, false><<<grid, WAVE, 0, a.stream>>>(
             (const uint16_t*)a.q, a.ldq, (const uint16_t*)a.k_cache, (const uint16_t*)a.v_cache, a.kv_width,
             a.block_table, a.max_blocks, a.token_slot, a.positions, a.q_start, a.n_seqs, (uint16_t*)a.out, a.ldo,
-            nullptr, a.n_heads, a.page_tokens, a.window, sl, tpt, cpt, chunk_keys, n_chunks);
+            nullptr, a.n_heads, a.page_tokens, a.window, sl, tpt, cpt, chunk_keys, n_chunks, a.max_q_len <= tpt);
     HFA_LAUNCH_CHECK("attn_mfma");
     return 0;
 }
@@ -499,9 +539,9 @@ int attn_mfma_launch(const AttnArgs& a) {
             default: return launch_prefill<4>(a, tpt, cpt);
         }
     }
-    const int tiles = (a.n_tokens + tpt - 1) / tpt + a.n_seqs;
+    const int tiles = a.max_q_len <= tpt ? a.n_seqs : (a.n_tokens + tpt - 1) / tpt + a.n_seqs;
     // Few waves and long contexts: cut the keys into chunks so that the machine is full.
-    const long waves = (long)((a.n_tokens + tpt - 1) / tpt) * a.n_kv_heads;
+    const long waves = (long)(a.max_q_len <= tpt ? a.n_seqs : (a.n_tokens + tpt - 1) / tpt) * a.n_kv_heads;
     const int span = a.window > 0 && a.window + a.max_q_len < a.max_seq_len ? a.window + a.max_q_len : a.max_seq_len;
     int n_chunks = 1, chunk_keys = a.max_seq_len;
     if (waves < 1024 && span > 128 && a.workspace) {

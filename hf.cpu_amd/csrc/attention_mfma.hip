@@ -29,6 +29,15 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 #define PG_MAX 512
 #define NEG_BIG (-1.0e30f)
 
+// 2^x by the hardware instruction (arguments here are <= 0 or the -1e30 sentinel's difference,
+// never subnormal results that matter), and the bf16 bits of a probability in [0, 1]: round to
+// nearest even without the NaN case.
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ uint32_t prob_bits(float p) {
+    const uint32_t u = __float_as_uint(p);
+    return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+}
+
 union Frag {
     uint4 u;
     uint2 h[2];
@@ -164,11 +173,11 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
         }
         mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
         const float mn = fmaxf(m, mx);
-        const float corr = exp2f(m - mn);
+        const float corr = fast_exp2(m - mn);
         float psum = 0.f;
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-            const float p = st[r] > 0.5f * NEG_BIG ? exp2f(st[r] - mn) : 0.f;
+            const float p = st[r] > 0.5f * NEG_BIG ? fast_exp2(st[r] - mn) : 0.f;
             st[r] = p;
             psum += p;
         }
@@ -184,7 +193,7 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
             uint32_t w[4];
 #pragma unroll
             for (int e = 0; e < 4; e++)
-                w[e] = (uint32_t)bf16_bits(st[8 * kk + 2 * e]) | ((uint32_t)bf16_bits(st[8 * kk + 2 * e + 1]) << 16);
+                w[e] = prob_bits(st[8 * kk + 2 * e]) | (prob_bits(st[8 * kk + 2 * e + 1]) << 16);
             pf[kk].u = make_uint4(w[0], w[1], w[2], w[3]);
         }
     };
@@ -408,11 +417,11 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
             }
             mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
             const float mn = fmaxf(m, mx);
-            const float corr = exp2f(m - mn);
+            const float corr = fast_exp2(m - mn);
             float psum = 0.f;
 #pragma unroll
             for (int r = 0; r < 16; r++) {
-                const float p = st[r] > 0.5f * NEG_BIG ? exp2f(st[r] - mn) : 0.f;
+                const float p = st[r] > 0.5f * NEG_BIG ? fast_exp2(st[r] - mn) : 0.f;
                 st[r] = p;
                 psum += p;
             }
@@ -429,7 +438,7 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
                 uint32_t w[4];
 #pragma unroll
                 for (int e = 0; e < 4; e++)
-                    w[e] = (uint32_t)bf16_bits(st[8 * kk + 2 * e]) | ((uint32_t)bf16_bits(st[8 * kk + 2 * e + 1]) << 16);
+                    w[e] = prob_bits(st[8 * kk + 2 * e]) | (prob_bits(st[8 * kk + 2 * e + 1]) << 16);
                 pf[kk].u = make_uint4(w[0], w[1], w[2], w[3]);
             }
 #pragma unroll

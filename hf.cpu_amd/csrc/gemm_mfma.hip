@@ -231,10 +231,10 @@ __global__ void gemm_finish_kernel(const float* __restrict__ partial, int splits
         reinterpret_cast<float*>(out)[(size_t)row * ldo + col] += v;
 }
 
-template <int BM, int BN, int BK, int WM, int WN, int MODE>
+template <int BM, int BN, int BK, int WM, int WN, int MODE, int PF>
 static int launch_cfg(const GemmArgs& g, void* out, int splits, int k_per_split) {
     using C = MfmaCfg<BM, BN, BK, WM, WN>;
-    auto kernel = gemm_mfma_kernel<BM, BN, BK, WM, WN, MODE, (BM >= 128 ? 1 : 2)>;
+    auto kernel = gemm_mfma_kernel<BM, BN, BK, WM, WN, MODE, PF>;
     static bool configured = false;
     if (!configured) {
         hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM);
@@ -252,17 +252,17 @@ static int launch_cfg(const GemmArgs& g, void* out, int splits, int k_per_split)
     return 0;
 }
 
-template <int BM, int BN, int BK, int WM, int WN>
+template <int BM, int BN, int BK, int WM, int WN, int PF = (BM >= 128 ? 1 : 2)>
 static int launch_mode(const GemmArgs& g, int mode, void* out, int splits, int k_per_split) {
     switch (mode) {
-        case OUT_BF16: return launch_cfg<BM, BN, BK, WM, WN, OUT_BF16>(g, out, splits, k_per_split);
-        case OUT_F32: return launch_cfg<BM, BN, BK, WM, WN, OUT_F32>(g, out, splits, k_per_split);
-        case OUT_ACC: return launch_cfg<BM, BN, BK, WM, WN, OUT_ACC>(g, out, splits, k_per_split);
+        case OUT_BF16: return launch_cfg<BM, BN, BK, WM, WN, OUT_BF16, PF>(g, out, splits, k_per_split);
+        case OUT_F32: return launch_cfg<BM, BN, BK, WM, WN, OUT_F32, PF>(g, out, splits, k_per_split);
+        case OUT_ACC: return launch_cfg<BM, BN, BK, WM, WN, OUT_ACC, PF>(g, out, splits, k_per_split);
         case OUT_SWIGLU:
-            if constexpr ((BN / WN) % 64 == 0) return launch_cfg<BM, BN, BK, WM, WN, OUT_SWIGLU>(g, out, splits, k_per_split);
+            if constexpr ((BN / WN) % 64 == 0) return launch_cfg<BM, BN, BK, WM, WN, OUT_SWIGLU, PF>(g, out, splits, k_per_split);
             hfa_set_error("gemm_mfma: this tile shape cannot pair gate and up columns");
             return 1;
-        default: return launch_cfg<BM, BN, BK, WM, WN, OUT_PARTIAL>(g, out, splits, k_per_split);
+        default: return launch_cfg<BM, BN, BK, WM, WN, OUT_PARTIAL, PF>(g, out, splits, k_per_split);
     }
 }
 

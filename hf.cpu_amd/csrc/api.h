@@ -75,7 +75,9 @@ int hfa_swiglu(const void* gate_up, void* out, int dtype, int n_tokens, int widt
 int hfa_scatter_i32(int* dst, const int* idx, const int* val, int n, hipStream_t stream);
 
 // out[r] = first index of the maximum of logits[r, :].  (src/sample.c:72-77)
-int hfa_argmax(const float* logits, int ld, int* out, int n_rows, int vocab, hipStream_t stream);
+// `workspace` holds the candidates of the first of its two stages (n_rows * 64 * 8 bytes).
+int hfa_argmax(const float* logits, int ld, int* out, int n_rows, int vocab, void* workspace,
+               size_t workspace_bytes, hipStream_t stream);
 
 // The k best of each row in the order (logit descending, id ascending) (src/sample.c:59-64),
 // and stats[r] = {max, log(sum(exp(l - max)))} (src/sample.c:25-33). k <= 1024.

@@ -109,17 +109,13 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
         for (int r = 0; r < 16; r++) o[db][r] = 0.f;
     float m = NEG_BIG, l = 0.f;
 
-    // The page ids of the wave's key range go to LDS once (up to PG_MAX pages), so that a block's
-    // loads do not wait for a block-table load first.
+    // Page ids come from LDS, never from the block table inside the loop: a block-table load
+    // whose result feeds an address would have to be waited for, and since loads return in order
+    // that wait would drain every key and value load issued before it. The ids of a window of
+    // PG_MAX pages are fetched at once (pw0 = first page of the window), outside the steady loop.
     __shared__ int pg_s[PG_MAX];
-    const int pb0 = ((k_begin / KB) * KB) / P;
-    const int k_top = (k_end / KB) * KB + KB - 1 < hi ? (k_end / KB) * KB + KB - 1 : hi;   // last key any load touches
-    const int n_pg = k_top / P - pb0 + 1;
-    const bool pg_lds = n_pg <= PG_MAX;
-    if (pg_lds)
-        for (int i = lane; i < n_pg; i += WAVE) pg_s[i] = bt[pb0 + i];
-    __syncthreads();
-    auto page_of = [&](int key) { return pg_lds ? pg_s[key / P - pb0] : bt[key / P]; };
+    int pw0 = 0;
+    auto page_of = [&](int key) { return pg_s[key / P - pw0]; };
 
     auto load_k = [&](int key0, Frag (&kf)[KS]) {
         int key = key0 + col;                              // this lane's row of the key block
@@ -184,10 +180,14 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
         psum += __shfl_xor(psum, 32, WAVE);
         l = l * corr + psum;
         m = mn;
+        // the running maxima settle after a few blocks; the accumulators are rescaled only when
+        // some column's maximum moved (decided by the whole wave together)
+        if (__any(corr != 1.0f)) {
 #pragma unroll
-        for (int db = 0; db < NDB; db++)
+            for (int db = 0; db < NDB; db++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) o[db][r] *= corr;
+                for (int r = 0; r < 16; r++) o[db][r] *= corr;
+        }
 #pragma unroll
         for (int kk = 0; kk < 2; kk++) {
             uint32_t w[4];
@@ -207,32 +207,42 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
 
     // Two register sets in rotation. The keys of block b + 2 are requested as soon as the scores
     // of block b are formed, its values as soon as block b's values are used, so between one and
-    // two blocks (16 to 32 KB a wave at head_dim 128) are always on their way.
+    // two blocks (16 to 32 KB a wave at head_dim 128) are always on their way. Inside a window
+    // every load is issued unconditionally (past the window's end its last block is fetched again
+    // and not used) and there is no branch around a load: the compiler then knows how many loads
+    // are outstanding at each use and waits for exactly those instead of draining all of them.
     const int first = (k_begin / KB) * KB;
     const int nb = first <= k_end ? (k_end - first) / KB + 1 : 0;
-    Frag k0f[KS], k1f[KS], v0f[NDB][2], v1f[NDB][2];
-    if (nb > 0) { load_k(first, k0f); load_v(first, v0f); }
-    if (nb > 1) { load_k(first + KB, k1f); load_v(first + KB, v1f); }
-    // The scheduling barriers keep the compiler from sinking the loads towards their use: they
-    // are issued exactly here, a block and a half ahead.
-    for (int b = 0; b < nb; b += 2) {
-        scores(first + b * KB, k0f);
-        __builtin_amdgcn_sched_barrier(0);
-        if (b + 2 < nb) load_k(first + (b + 2) * KB, k0f);
-        __builtin_amdgcn_sched_barrier(0);
-        values(v0f);
-        __builtin_amdgcn_sched_barrier(0);
-        if (b + 2 < nb) load_v(first + (b + 2) * KB, v0f);
-        __builtin_amdgcn_sched_barrier(0);
-        if (b + 1 >= nb) break;
-        scores(first + (b + 1) * KB, k1f);
-        __builtin_amdgcn_sched_barrier(0);
-        if (b + 3 < nb) load_k(first + (b + 3) * KB, k1f);
-        __builtin_amdgcn_sched_barrier(0);
-        values(v1f);
-        __builtin_amdgcn_sched_barrier(0);
-        if (b + 3 < nb) load_v(first + (b + 3) * KB, v1f);
-        __builtin_amdgcn_sched_barrier(0);
+    const int k_top = first + nb * KB - 1 < hi ? first + nb * KB - 1 : hi;       // last key any load touches
+    const int win_blocks = PG_MAX * P / KB;                                       // key blocks a window of pages covers
+    for (int wb = 0; wb < nb; wb += win_blocks) {
+        const int we = wb + win_blocks < nb ? wb + win_blocks : nb;               // blocks [wb, we)
+        __syncthreads();                                                          // the old window is no longer read
+        pw0 = (first + wb * KB) / P;
+        {
+            const int top = first + we * KB - 1 < k_top ? first + we * KB - 1 : k_top;
+            const int n_pg = top / P - pw0 + 1;
+            for (int i = lane; i < n_pg; i += WAVE) pg_s[i] = bt[pw0 + i];
+        }
+        __syncthreads();
+        const int last = first + (we - 1) * KB;
+        auto at = [&](int b) { const int k = first + b * KB; return k < last ? k : last; };
+        Frag k0f[KS], k1f[KS], v0f[NDB][2], v1f[NDB][2];
+        load_k(at(wb), k0f);
+        load_v(at(wb), v0f);
+        load_k(at(wb + 1), k1f);
+        load_v(at(wb + 1), v1f);
+        for (int b = wb; b < we; b += 2) {
+            scores(first + b * KB, k0f);
+            load_k(at(b + 2), k0f);
+            values(v0f);
+            load_v(at(b + 2), v0f);
+            if (b + 1 >= we) break;
+            scores(first + (b + 1) * KB, k1f);
+            load_k(at(b + 3), k1f);
+            values(v1f);
+            load_v(at(b + 3), v1f);
+        }
     }
 
     if (!col_ok) return;
@@ -334,15 +344,10 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
         for (int r = 0; r < 16; r++) o[db][r] = 0.f;
     float m = NEG_BIG, l = 0.f;
 
-    // page ids of the block's key range in LDS (see above)
+    // page ids in LDS, a window of PG_MAX pages at a time (see the kernel above)
     __shared__ int pg_s[PG_MAX];
-    const int pb0 = ((k_begin / KB) * KB) / P;
-    const int n_pg = hi / P - pb0 + 1;
-    const bool pg_lds = n_pg <= PG_MAX;
-    if (pg_lds)
-        for (int i = tid; i < n_pg; i += 4 * WAVE) pg_s[i] = bt[pb0 + i];
-    __syncthreads();
-    auto page_of = [&](int key) { return pg_lds ? pg_s[key / P - pb0] : bt[key / P]; };
+    int pw0 = 0;
+    auto page_of = [&](int key) { return pg_s[key / P - pw0]; };
 
     // global -> registers -> LDS. Keys: 32 rows of D elements = 4 D chunks of 16 bytes.
     // Values: D rows of 32 keys = 4 D chunks of 8 keys. Each thread takes up to NCH of both.
@@ -386,74 +391,89 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
 
     const int first = (k_begin / KB) * KB;
     const int nb = (hi - first) / KB + 1;
-    gload(first);
-    sstore(0);
-    __syncthreads();
-    for (int b = 0; b < nb; b++) {
-        const int key0 = first + b * KB, stage = b & 1;
-        if (b + 1 < nb) gload(key0 + KB);
-        // A wave whose columns all end before this block skips the math. The test is made by all
-        // lanes together: the matrix products need every lane, also those of unused columns.
-        const bool wave_sees = __any(key0 <= vhi) != 0;
-        if (wave_sees) {
-            const uint16_t* ks_ = &k_s[stage][col * KROW + half * 8];
-            floatx16 st;
-#pragma unroll
-            for (int r = 0; r < 16; r++) st[r] = 0.f;
-#pragma unroll
-            for (int ks = 0; ks < KS; ks++) {
-                Frag kf, qf;
-                kf.u = *reinterpret_cast<const uint4*>(ks_ + ks * 16);
-                qf.u = q_s[wave][ks * WAVE + lane];
-                st = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf.v, qf.v, st, 0, 0, 0);
-            }
-            float mx = NEG_BIG;
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int kr = key0 + 8 * (r / 4) + 4 * half + (r % 4);
-                const bool vis = kr >= vlo && kr <= vhi;
-                st[r] = vis ? st[r] * scale_log2e : NEG_BIG;
-                mx = fmaxf(mx, st[r]);
-            }
-            mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
-            const float mn = fmaxf(m, mx);
-            const float corr = fast_exp2(m - mn);
-            float psum = 0.f;
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const float p = st[r] > 0.5f * NEG_BIG ? fast_exp2(st[r] - mn) : 0.f;
-                st[r] = p;
-                psum += p;
-            }
-            psum += __shfl_xor(psum, 32, WAVE);
-            l = l * corr + psum;
-            m = mn;
-#pragma unroll
-            for (int db = 0; db < NDB; db++)
-#pragma unroll
-                for (int r = 0; r < 16; r++) o[db][r] *= corr;
-            Frag pf[2];
-#pragma unroll
-            for (int kk = 0; kk < 2; kk++) {
-                uint32_t w[4];
-#pragma unroll
-                for (int e = 0; e < 4; e++)
-                    w[e] = prob_bits(st[8 * kk + 2 * e]) | (prob_bits(st[8 * kk + 2 * e + 1]) << 16);
-                pf[kk].u = make_uint4(w[0], w[1], w[2], w[3]);
-            }
-#pragma unroll
-            for (int kk = 0; kk < 2; kk++)
-#pragma unroll
-                for (int db = 0; db < NDB; db++) {
-                    const uint16_t* vs_ = &v_s[stage][(32 * db + col) * PVS + 16 * kk + 4 * half];
-                    Frag vf;
-                    vf.h[0] = *reinterpret_cast<const uint2*>(vs_);
-                    vf.h[1] = *reinterpret_cast<const uint2*>(vs_ + 8);
-                    o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf.v, pf[kk].v, o[db], 0, 0, 0);
-                }
+    const int win_blocks = PG_MAX * P / KB;
+    for (int wb = 0; wb < nb; wb += win_blocks) {
+        const int we = wb + win_blocks < nb ? wb + win_blocks : nb;               // blocks [wb, we)
+        __syncthreads();                                                          // old window and stages are no longer read
+        pw0 = (first + wb * KB) / P;
+        {
+            const int top = first + we * KB - 1 < hi ? first + we * KB - 1 : hi;
+            const int n_pg = top / P - pw0 + 1;
+            for (int i = tid; i < n_pg; i += 4 * WAVE) pg_s[i] = bt[pw0 + i];
         }
-        if (b + 1 < nb) sstore(stage ^ 1);
         __syncthreads();
+        const int last = first + (we - 1) * KB;
+        gload(first + wb * KB);
+        sstore(wb & 1);
+        __syncthreads();
+        for (int b = wb; b < we; b++) {
+            const int key0 = first + b * KB, stage = b & 1;
+            gload(key0 + KB < last ? key0 + KB : last);       // unconditional: the last block is fetched twice
+            // A wave whose columns all end before this block skips the math. The test is made by all
+            // lanes together: the matrix products need every lane, also those of unused columns.
+            const bool wave_sees = __any(key0 <= vhi) != 0;
+            if (wave_sees) {
+                const uint16_t* ks_ = &k_s[stage][col * KROW + half * 8];
+                floatx16 st;
+#pragma unroll
+                for (int r = 0; r < 16; r++) st[r] = 0.f;
+#pragma unroll
+                for (int ks = 0; ks < KS; ks++) {
+                    Frag kf, qf;
+                    kf.u = *reinterpret_cast<const uint4*>(ks_ + ks * 16);
+                    qf.u = q_s[wave][ks * WAVE + lane];
+                    st = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf.v, qf.v, st, 0, 0, 0);
+                }
+                float mx = NEG_BIG;
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int kr = key0 + 8 * (r / 4) + 4 * half + (r % 4);
+                    const bool vis = kr >= vlo && kr <= vhi;
+                    st[r] = vis ? st[r] * scale_log2e : NEG_BIG;
+                    mx = fmaxf(mx, st[r]);
+                }
+                mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+                const float mn = fmaxf(m, mx);
+                const float corr = fast_exp2(m - mn);
+                float psum = 0.f;
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const float p = st[r] > 0.5f * NEG_BIG ? fast_exp2(st[r] - mn) : 0.f;
+                    st[r] = p;
+                    psum += p;
+                }
+                psum += __shfl_xor(psum, 32, WAVE);
+                l = l * corr + psum;
+                m = mn;
+                if (__any(corr != 1.0f)) {                      // see above: only when a maximum moved
+#pragma unroll
+                    for (int db = 0; db < NDB; db++)
+#pragma unroll
+                        for (int r = 0; r < 16; r++) o[db][r] *= corr;
+                }
+                Frag pf[2];
+#pragma unroll
+                for (int kk = 0; kk < 2; kk++) {
+                    uint32_t w[4];
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        w[e] = prob_bits(st[8 * kk + 2 * e]) | (prob_bits(st[8 * kk + 2 * e + 1]) << 16);
+                    pf[kk].u = make_uint4(w[0], w[1], w[2], w[3]);
+                }
+#pragma unroll
+                for (int kk = 0; kk < 2; kk++)
+#pragma unroll
+                    for (int db = 0; db < NDB; db++) {
+                        const uint16_t* vs_ = &v_s[stage][(32 * db + col) * PVS + 16 * kk + 4 * half];
+                        Frag vf;
+                        vf.h[0] = *reinterpret_cast<const uint2*>(vs_);
+                        vf.h[1] = *reinterpret_cast<const uint2*>(vs_ + 8);
+                        o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf.v, pf[kk].v, o[db], 0, 0, 0);
+                    }
+            }
+            sstore(stage ^ 1);
+            __syncthreads();
+        }
     }
     if (!col_ok) return;
     const float inv = 1.0f / l;
@@ -554,7 +574,7 @@ int attn_mfma_launch(const AttnArgs& a) {
     const int span = a.window > 0 && a.window + a.max_q_len < a.max_seq_len ? a.window + a.max_q_len : a.max_seq_len;
     int n_chunks = 1, chunk_keys = a.max_seq_len;
     if (waves < 1024 && span > 128 && a.workspace) {
-        int want = (int)((2048 + waves - 1) / waves);
+        int want = (int)((1024 + waves - 1) / waves);
         const int most = (span + 63) / 64;
         if (want > most) want = most;
         chunk_keys = ((a.max_seq_len + want - 1) / want + KB - 1) / KB * KB;

@@ -31,24 +31,53 @@ __device__ __forceinline__ void block_best(float& v, int& i, float* sv, int* si)
     i = si[16];
 }
 
-__global__ __launch_bounds__(1024) void argmax_kernel(const float* __restrict__ logits, int ld, int* __restrict__ out,
-                                                      int vocab) {
+// Two stages, so that a single row still spreads over the machine: ARGMAX_PARTS blocks per row
+// each find the best of their slice, then one small block per row picks among them. The
+// ordering (larger logit, then smaller id) makes the result independent of the slicing.
+#define ARGMAX_PARTS 64
+__global__ __launch_bounds__(256) void argmax_part_kernel(const float* __restrict__ logits, int ld, int vocab,
+                                                          float* __restrict__ part_v, int* __restrict__ part_i) {
     __shared__ float sv[17];
     __shared__ int si[17];
     const float* row = logits + (size_t)blockIdx.x * ld;
+    const int per = (vocab + ARGMAX_PARTS - 1) / ARGMAX_PARTS;
+    const int lo = blockIdx.y * per, hi = lo + per < vocab ? lo + per : vocab;
     float bv = -INFINITY;
     int bi = 0x7fffffff;
-    for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
+    for (int i = lo + threadIdx.x; i < hi; i += blockDim.x) {
         const float v = row[i];
         if (better(v, i, bv, bi)) { bv = v; bi = i; }
     }
     block_best(bv, bi, sv, si);
-    if (threadIdx.x == 0) out[blockIdx.x] = bi == 0x7fffffff ? 0 : bi;
+    if (threadIdx.x == 0) {
+        part_v[blockIdx.x * ARGMAX_PARTS + blockIdx.y] = bv;
+        part_i[blockIdx.x * ARGMAX_PARTS + blockIdx.y] = bi;
+    }
 }
 
-extern "C" int hfa_argmax(const float* logits, int ld, int* out, int n_rows, int vocab, hipStream_t stream) {
+__global__ __launch_bounds__(WAVE) void argmax_final_kernel(const float* __restrict__ part_v,
+                                                            const int* __restrict__ part_i, int* __restrict__ out) {
+    float v = part_v[blockIdx.x * ARGMAX_PARTS + threadIdx.x];
+    int i = part_i[blockIdx.x * ARGMAX_PARTS + threadIdx.x];
+#pragma unroll
+    for (int off = WAVE / 2; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(v, off, WAVE);
+        const int oi = __shfl_xor(i, off, WAVE);
+        if (better(ov, oi, v, i)) { v = ov; i = oi; }
+    }
+    if (threadIdx.x == 0) out[blockIdx.x] = i == 0x7fffffff ? 0 : i;
+}
+
+extern "C" int hfa_argmax(const float* logits, int ld, int* out, int n_rows, int vocab, void* workspace,
+                          size_t workspace_bytes, hipStream_t stream) {
     HFA_REQUIRE(n_rows > 0 && vocab > 0 && ld >= vocab, "argmax: bad sizes rows=%d vocab=%d ld=%d", n_rows, vocab, ld);
-    argmax_kernel<<<n_rows, 1024, 0, stream>>>(logits, ld, out, vocab);
+    HFA_REQUIRE(workspace && workspace_bytes >= (size_t)n_rows * ARGMAX_PARTS * 8,
+                "argmax: the workspace is smaller than %d x %d candidates", n_rows, ARGMAX_PARTS);
+    static_assert(ARGMAX_PARTS == WAVE, "the second stage is one wave per row");
+    float* part_v = (float*)workspace;
+    int* part_i = (int*)(part_v + (size_t)n_rows * ARGMAX_PARTS);
+    argmax_part_kernel<<<dim3(n_rows, ARGMAX_PARTS), 256, 0, stream>>>(logits, ld, vocab, part_v, part_i);
+    argmax_final_kernel<<<n_rows, WAVE, 0, stream>>>(part_v, part_i, out);
     HFA_LAUNCH_CHECK("argmax");
     return 0;
 }

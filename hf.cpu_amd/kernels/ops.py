@@ -254,7 +254,7 @@ class Ops:
         if out is None:
             out = torch.empty(R, dtype=torch.int32, device=logits.device)
         self._check(self.lib.hfa_argmax(logits.data_ptr(), _rows(logits, "argmax logits"), _ints(out, "argmax out", R),
-                                        R, V, self._stream()))
+                                        R, V, self.workspace.data_ptr(), self.workspace.numel(), self._stream()))
         return out
 
     def topk(self, logits, k, want_stats=True):

@@ -344,6 +344,69 @@ def test_paged_attention_on_matrix_cores(ops16, H, G, D, page, window, lengths, 
     assert err <= 0.02, f"max |diff| {err:.3e}"
 
 
+def tail_attention(q_tail, k, v, window):
+    """Attention of the last queries of a sequence only (float64): q_tail [ql, H, D] stands at
+    positions n-ql .. n-1 of k, v [n, G, D]; key j is visible to position p iff j <= p and,
+    with a window W, p - j < W. The mask is built per query, so that long sequences stay cheap."""
+    ql, H, D = q_tail.shape
+    n, G, _ = k.shape
+    out = np.empty((ql, H, D))
+    k64, v64 = k.astype(np.float64), v.astype(np.float64)
+    for i in range(ql):
+        p = n - ql + i
+        lo = max(0, p - window + 1) if window else 0
+        for h in range(H):
+            g = h // (H // G)
+            s = k64[lo:p + 1, g] @ q_tail[i, h].astype(np.float64) / math.sqrt(D)
+            e = np.exp(s - s.max())
+            out[i, h] = (e / e.sum()) @ v64[lo:p + 1, g]
+    return out
+
+
+@pytest.mark.parametrize("H,G,D,page,window,lengths,q_lens", [
+    (28, 4, 128, 16, 0, [40000, 9000, 17], [1, 1, 1]),       # more pages than one window of page ids holds
+    (8, 2, 64, 16, 0, [20000], [200]),                         # a portion late in a long prompt
+    (4, 4, 32, 8, 5000, [30000, 4999, 5001], [3, 1, 2]),       # a window far into a long sequence
+    (14, 2, 64, 16, 0, [100000], [1]),                         # more chunks of keys than one merge pass takes
+])
+def test_paged_attention_long_contexts(ops16, H, G, D, page, window, lengths, q_lens):
+    """Tens of thousands of keys: the last queries against float64 attention over the same
+    rounded inputs. In each request one far key is made to matter: its dot product with the
+    first query head stands out, so that a chunk that is skipped or read twice shows."""
+    rng = np.random.default_rng(H + D + len(lengths))
+    dtype = torch.bfloat16
+    ks, vs, cache, table = paged_setup(rng, lengths, G, D, page, dtype)
+    qs, positions, slots, wants = [], [], [], []
+    kc = cache.k.float().cpu().numpy()
+    for s, (n, ql) in enumerate(zip(lengths, q_lens)):
+        q_tail = rng.standard_normal((ql, H, D)).astype(np.float32)
+        lo = max(0, n - ql - window + 1) if window else 0
+        far = lo + (n - ql - lo) // 3                         # visible to every query of the tail
+        if n > 100:
+            ks[s][far, 0] = 11.0 * math.sqrt(D) * q_tail[0, 0] / np.dot(q_tail[0, 0], q_tail[0, 0])   # score 11
+            row = int(table[s, far // page].item()) * page + far % page
+            kc[row, :D] = ks[s][far, 0]
+        wants.append(tail_attention(rounded(q_tail, dtype), rounded(ks[s], dtype), rounded(vs[s], dtype), window))
+        qs.append(q_tail)
+        positions += list(range(n - ql, n))
+        slots += [s] * ql
+    cache = FakeCache(group=0, k=dev(kc, dtype), v=cache.v, page_tokens=page, window=0)
+    q = np.concatenate(qs).reshape(-1, H * D)
+    want = np.concatenate(wants).reshape(-1, H * D)
+    out = torch.empty((q.shape[0], H * D), dtype=dtype, device="cuda")
+    step = FakeStep(ints(positions), ints(slots), table, None)
+    ops16.paged_attention(dev(q, dtype), H, G, D, cache, step, window, 1.0 / math.sqrt(D), out)
+    err = np.max(np.abs(out.float().cpu().numpy() - want))
+    assert err <= 0.02, f"max |diff| {err:.3e}"
+    other = torch.empty_like(out)
+    ops16.force_plain_attention = True
+    try:
+        ops16.paged_attention(dev(q, dtype), H, G, D, cache, step, window, 1.0 / math.sqrt(D), other)
+    finally:
+        ops16.force_plain_attention = False
+    assert np.max(np.abs(other.float().cpu().numpy() - want)) <= 0.02
+
+
 def test_attention_special_cases(ops32):
     """A single query at position 0 returns value row 0 exactly; equal scores (zero query)
     return the mean of the visible value rows (softmax of equal numbers)."""

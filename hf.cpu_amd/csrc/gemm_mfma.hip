@@ -44,6 +44,59 @@ struct MfmaCfg {
     static_assert(TM % 32 == 0 && TN % 32 == 0 && BK % 16 == 0, "wave tiles are made of 32x32x16 products");
 };
 
+// Stores a wave's accumulators: element r of a lane is row 8 * (r / 4) + 4 * (lane / 32) + r % 4,
+// column lane % 32 of its 32x32 block.
+template <class C, int MODE>
+__device__ __forceinline__ void gemm_epilogue(floatx16 (&acc)[C::FM][C::FN], const float* __restrict__ bias,
+                                              void* __restrict__ out, int ldo, int M, int N, int m0, int n0, int wm,
+                                              int wn, int lane) {
+    if (MODE == OUT_SWIGLU) {
+        static_assert(MODE != OUT_SWIGLU || C::FN % 2 == 0, "gate and up blocks must meet in one wave");
+#pragma unroll
+        for (int i = 0; i < C::FM; i++) {
+#pragma unroll
+            for (int j = 0; j + 1 < C::FN; j += 2) {
+                const int col = n0 + wn * C::TN + j * 32;          // first gate column of the pair of blocks
+                if (col + (lane & 31) >= N) continue;
+                const int f = col / 2 + (lane & 31);
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int row = m0 + wm * C::TM + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
+                    if (row >= M) continue;
+                    const float gt = acc[i][j][r], up = acc[i][j + 1][r];
+                    reinterpret_cast<uint16_t*>(out)[(size_t)row * ldo + f] = bf16_bits((gt / (1.0f + expf(-gt))) * up);
+                }
+            }
+        }
+        return;
+    }
+#pragma unroll
+    for (int i = 0; i < C::FM; i++) {
+#pragma unroll
+        for (int j = 0; j < C::FN; j++) {
+            const int col = n0 + wn * C::TN + j * 32 + (lane & 31);
+            if (col >= N) continue;
+            const float b = (MODE != OUT_PARTIAL && bias) ? bias[col] : 0.f;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int row = m0 + wm * C::TM + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
+                if (row >= M) continue;
+                const float v = acc[i][j][r] + b;
+                if (MODE == OUT_BF16) {
+                    reinterpret_cast<uint16_t*>(out)[(size_t)row * ldo + col] = bf16_bits(v);
+                } else if (MODE == OUT_F32) {
+                    reinterpret_cast<float*>(out)[(size_t)row * ldo + col] = v;
+                } else if (MODE == OUT_ACC) {
+                    float* dst = reinterpret_cast<float*>(out) + (size_t)row * ldo + col;
+                    *dst += v;
+                } else {
+                    reinterpret_cast<float*>(out)[((size_t)blockIdx.z * M + row) * N + col] = v;
+                }
+            }
+        }
+    }
+}
+
 template <int BM, int BN, int BK, int WM, int WN, int MODE, int PF>
 __global__ __launch_bounds__(WM* WN* WAVE) void gemm_mfma_kernel(
     const uint16_t* __restrict__ A, int lda, const uint16_t* __restrict__ W, int ldw,
@@ -159,51 +212,211 @@ __global__ __launch_bounds__(WM* WN* WAVE) void gemm_mfma_kernel(
         __syncthreads();
     }
 
-    // ---- epilogue: element r of a lane is row 8 * (r / 4) + 4 * (lane / 32) + r % 4, column lane % 32 ----
-    if (MODE == OUT_SWIGLU) {
+    gemm_epilogue<C, MODE>(acc, bias, out, ldo, M, N, m0, n0, wm, wn, lane);
+}
+
+// ---- large M (prompts): operand tiles travel global -> LDS without passing through registers ----
+//
+// A block of 2 x 2 waves owns a BM x BN tile, one block per CU, and keeps STAGES tiles of BK
+// columns of K in LDS. While tile t is multiplied, tile t + STAGES - 1 is requested
+// (global_load_lds_dwordx4: the 64 lanes of a wave fill 1 KB of LDS), one request after every few
+// matrix instructions: the texture path takes about as long for a tile's bytes as the matrix
+// cores take for its products, so the two have to run side by side, and a wave that issues its
+// requests in one burst stands still until the path has taken them all. A load has STAGES - 2
+// whole steps to arrive; the only wait of a step is for the oldest tile. The loads are inline
+// assembly because the wait they need is "all but the newer tiles'", which only the author of
+// the pipeline can state: the compiler, told about such loads, waits for all of them before the
+// next LDS read.
+//
+// LDS rows have no padding (the hardware places the 64 lanes' 16 bytes back to back); instead the
+// 16-byte pieces of a row are stored in swizzled order, which a lane arranges by which piece it
+// asks for: with rows of 128 bytes, piece p of row r lies at p ^ (r % 8); with rows of 64 bytes,
+// at p ^ ((r / 2) % 4). Eight lanes that read the same piece of eight consecutive rows then hit
+// eight different groups of banks.
+template <int BM, int BN, int BK, int WM, int WN>
+struct DmaCfg {
+    static constexpr int NW = WM * WN, NT = NW * WAVE;
+    static constexpr int ROWS = BM + BN;
+    static constexpr int PIECES = BK / 8;                    // 16-byte pieces per row
+    static constexpr int ROWS_PER_LOAD = WAVE / PIECES;
+    static constexpr int STAGE_BYTES = ROWS * BK * 2;
+    static constexpr int LOADS = ROWS / ROWS_PER_LOAD / NW;  // per wave and stage
+    static constexpr int TM = BM / WM, TN = BN / WN;
+    static constexpr int FM = TM / 32, FN = TN / 32;
+    static constexpr int STEPS = BK / 16;
+    static_assert(BK == 32 || BK == 64, "rows of 64 or 128 bytes");
+    static_assert(ROWS % (ROWS_PER_LOAD * NW) == 0 && BM % (ROWS_PER_LOAD * NW) == 0, "rows must spread evenly over the waves");
+    static_assert(TM % 32 == 0 && TN % 32 == 0, "wave tiles are made of 32x32x16 products");
+    static_assert(FM * FN * STEPS >= LOADS, "at most one request after a matrix instruction");
+    __device__ static constexpr int swizzle(int row) { return BK == 64 ? (row & 7) : ((row >> 1) & 3); }
+};
+
+// The block's tile of 16-bit results in LDS: rows of WIDTH columns, 16 bytes of padding.
+template <int BN, int MODE>
+struct DmaOut {
+    static constexpr int PAIR = MODE == OUT_SWIGLU ? 2 : 1;      // 32 gate and 32 up columns give 32 results
+    static constexpr int WIDTH = BN / PAIR, STRIDE = WIDTH + 8;
+    static constexpr int bytes(int bm) { return (MODE == OUT_BF16 || MODE == OUT_SWIGLU) ? bm * STRIDE * 2 : 0; }
+};
+
+template <int BM, int BN, int BK, int WM, int WN, int STAGES, int MODE>
+__global__ __launch_bounds__(WM* WN* WAVE) void gemm_dma_kernel(
+    const uint16_t* __restrict__ A, int lda, const uint16_t* __restrict__ W, int ldw,
+    const float* __restrict__ bias, void* __restrict__ out, int ldo, int M, int N, int K, int tiles_m, int tiles_n) {
+    using C = DmaCfg<BM, BN, BK, WM, WN>;
+    static_assert(STAGES >= 3, "one tile in use, the next one landed, one arriving");
+    extern __shared__ __attribute__((aligned(1024))) uint16_t smem[];
+    const int tid = threadIdx.x, lane = tid & (WAVE - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE);
+    const int wm = wave / WN, wn = wave % WN;
+
+    const int n_tiles = tiles_m * tiles_n;
+    int pid = blockIdx.x;
+    {
+        const int per = n_tiles / N_XCD, rem = n_tiles % N_XCD, x = pid % N_XCD, q = pid / N_XCD;
+        pid = x * per + (x < rem ? x : rem) + q;
+    }
+    const int in_group = GROUP_M * tiles_n;
+    const int group = pid / in_group, first_m = group * GROUP_M;
+    const int gsize = tiles_m - first_m < GROUP_M ? tiles_m - first_m : GROUP_M;
+    const int tm = first_m + (pid % in_group) % gsize, tn = (pid % in_group) / gsize;
+    const int m0 = tm * BM, n0 = tn * BN;
+
+    floatx16 acc[C::FM][C::FN];
+#pragma unroll
+    for (int i = 0; i < C::FM; i++)
+#pragma unroll
+        for (int j = 0; j < C::FN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+
+    // Request i of this wave fills rows (i * NW + wave) * ROWS_PER_LOAD .. of a stage; this lane
+    // supplies the piece stored at lane % PIECES of row lane / PIECES of them. Its address is a
+    // scalar base (the block's first row of A or W, advancing with K) plus a byte offset per lane.
+    const uint16_t* a_base = A + (size_t)m0 * lda;
+    const uint16_t* w_base = W + (size_t)n0 * ldw;
+    uint32_t src[C::LOADS];
+#pragma unroll
+    for (int i = 0; i < C::LOADS; i++) {
+        const int r = (i * C::NW + wave) * C::ROWS_PER_LOAD + lane / C::PIECES;
+        const int piece = (lane % C::PIECES) ^ C::swizzle(r);
+        if ((i * C::NW + wave) * C::ROWS_PER_LOAD < BM) {
+            const int last = M - 1 - m0;                     // rows past the edge repeat the last one
+            src[i] = (uint32_t)(r < last ? r : last) * (uint32_t)lda * 2u + piece * 16;
+        } else {
+            const int last = N - 1 - n0;
+            src[i] = (uint32_t)(r - BM < last ? r - BM : last) * (uint32_t)ldw * 2u + piece * 16;
+        }
+    }
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint16_t*)smem;
+    auto request = [&](int i, int stage, int t) {            // i is a constant after unrolling
+        const uint32_t dst = lds0 + stage * C::STAGE_BYTES + (i * C::NW + wave) * 1024;
+        const bool is_a = (i * C::NW + wave) * C::ROWS_PER_LOAD < BM;      // uniform over the wave
+        const uint16_t* base = (is_a ? a_base : w_base) + (size_t)t * BK;
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(src[i]), "s"(base) : "m0");
+    };
+    // Piece offsets (in elements) of the 16-column steps of a tile for this lane's rows: the rows
+    // a lane reads differ from lane % 32 by multiples of 32, so their swizzle is the lane's.
+    int piece_off[C::STEPS];
+#pragma unroll
+    for (int j = 0; j < C::STEPS; j++) piece_off[j] = ((2 * j + (lane >> 5)) ^ C::swizzle(lane & 31)) * 8;
+
+    // Operand fragments of 16-column step j of the tile in `stage`.
+    auto fragments = [&](int stage, int j, bf16x8 (&fa)[C::FM], bf16x8 (&fw)[C::FN]) {
+        const uint16_t* sa = smem + stage * (C::STAGE_BYTES / 2) + (wm * C::TM + (lane & 31)) * BK + piece_off[j];
+        const uint16_t* sw = smem + stage * (C::STAGE_BYTES / 2) + (BM + wn * C::TN + (lane & 31)) * BK + piece_off[j];
+#pragma unroll
+        for (int i = 0; i < C::FM; i++) fa[i] = *reinterpret_cast<const bf16x8*>(sa + i * 32 * BK);
+#pragma unroll
+        for (int i = 0; i < C::FN; i++) fw[i] = *reinterpret_cast<const bf16x8*>(sw + i * 32 * BK);
+    };
+
+    // The pipeline. Tiles 0 .. STAGES - 2 are requested up front. Step t begins with a wait and a
+    // barrier after which tile t + 1 has landed for every wave and every wave is done with tile
+    // t - 1; tile t + STAGES - 1 is then requested into tile t - 1's stage, a request after every
+    // few matrix instructions. The fragments of a 16-column step are read one step ahead, also
+    // across the barrier (tile t + 1's first ones during tile t's last step), so that the matrix
+    // cores have work the moment a wave leaves the barrier.
+    const int nk = K / BK;
+#pragma unroll
+    for (int p = 0; p < STAGES - 1; p++)
+        if (p < nk) {
+#pragma unroll
+            for (int i = 0; i < C::LOADS; i++) request(i, p, p);
+        }
+    if (nk >= STAGES - 1)
+        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(C::LOADS * (STAGES - 2)) : "memory");
+    else
+        asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+    bf16x8 fa[2][C::FM], fw[2][C::FN];
+    fragments(0, 0, fa[0], fw[0]);
+    constexpr int AHEAD = STAGES - 1;
+    constexpr int PRODUCTS = C::FM * C::FN * C::STEPS;      // matrix instructions per tile and wave
+    // With three stages a load has to arrive within the step after its request: request early.
+    constexpr int SPREAD = STAGES == 3 ? (PRODUCTS / 2 > C::LOADS ? PRODUCTS / 2 : C::LOADS) : PRODUCTS;
+    static_assert(SPREAD >= C::LOADS && SPREAD <= PRODUCTS && C::STEPS % 2 == 0, "at most one request after a matrix instruction");
+    int stage = 0;
+    for (int t = 0; t < nk; t++) {
+        if (t + STAGES - 2 < nk)
+            asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(C::LOADS * (STAGES - 3)) : "memory");
+        else
+            asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+        const bool more = t + AHEAD < nk;
+        const int into = stage + AHEAD < STAGES ? stage + AHEAD : stage + AHEAD - STAGES;
+        const int next = stage + 1 < STAGES ? stage + 1 : 0;
+        int done = 0;
+#pragma unroll
+        for (int j = 0; j < C::STEPS; j++) {
+            if (j + 1 < C::STEPS)
+                fragments(stage, j + 1, fa[(j + 1) & 1], fw[(j + 1) & 1]);
+            else if (t + 1 < nk)
+                fragments(next, 0, fa[0], fw[0]);
+#pragma unroll
+            for (int i = 0; i < C::FM; i++)
+#pragma unroll
+                for (int jj = 0; jj < C::FN; jj++) {
+                    acc[i][jj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[j & 1][i], fw[j & 1][jj], acc[i][jj], 0, 0, 0);
+                    done++;                                  // requests are dealt evenly among the first products
+                    if (done <= SPREAD && done * C::LOADS / SPREAD != (done - 1) * C::LOADS / SPREAD && more)
+                        request(done * C::LOADS / SPREAD - 1, into, t + AHEAD);
+                }
+        }
+        stage = next;
+    }
+    if constexpr (MODE == OUT_BF16 || MODE == OUT_SWIGLU) {
+        // 16-bit results leave through LDS: a lane holds single columns, and a store of 2 bytes per
+        // lane costs the memory path as much as one of 16. The block's tile is put together in
+        // LDS (the operand stages are free now), then written out 16 bytes per lane, whole rows.
+        using O = DmaOut<BN, MODE>;
         static_assert(MODE != OUT_SWIGLU || C::FN % 2 == 0, "gate and up blocks must meet in one wave");
+        __syncthreads();
 #pragma unroll
         for (int i = 0; i < C::FM; i++) {
 #pragma unroll
-            for (int j = 0; j + 1 < C::FN; j += 2) {
-                const int col = n0 + wn * C::TN + j * 32;          // first gate column of the pair of blocks
-                if (col + (lane & 31) >= N) continue;
-                const int f = col / 2 + (lane & 31);
+            for (int j = 0; j < C::FN; j += O::PAIR) {
+                const int col = (wn * C::TN + j * 32) / O::PAIR + (lane & 31);      // within the block's tile
+                const int gcol = n0 + wn * C::TN + j * 32 + (lane & 31);            // column of N (the gate's, if paired)
+                const float b = (MODE == OUT_BF16 && bias && gcol < N) ? bias[gcol] : 0.f;
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
-                    const int row = m0 + wm * C::TM + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
-                    if (row >= M) continue;
-                    const float gt = acc[i][j][r], up = acc[i][j + 1][r];
-                    reinterpret_cast<uint16_t*>(out)[(size_t)row * ldo + f] = bf16_bits((gt / (1.0f + expf(-gt))) * up);
+                    const int row = wm * C::TM + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
+                    float v = acc[i][j][r] + b;
+                    if constexpr (MODE == OUT_SWIGLU) v = (v / (1.0f + expf(-v))) * acc[i][j + 1][r];
+                    smem[row * O::STRIDE + col] = bf16_bits(v);
                 }
             }
         }
-        return;
-    }
-#pragma unroll
-    for (int i = 0; i < C::FM; i++) {
-#pragma unroll
-        for (int j = 0; j < C::FN; j++) {
-            const int col = n0 + wn * C::TN + j * 32 + (lane & 31);
-            if (col >= N) continue;
-            const float b = (MODE != OUT_PARTIAL && bias) ? bias[col] : 0.f;
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int row = m0 + wm * C::TM + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
-                if (row >= M) continue;
-                const float v = acc[i][j][r] + b;
-                if (MODE == OUT_BF16) {
-                    reinterpret_cast<uint16_t*>(out)[(size_t)row * ldo + col] = bf16_bits(v);
-                } else if (MODE == OUT_F32) {
-                    reinterpret_cast<float*>(out)[(size_t)row * ldo + col] = v;
-                } else if (MODE == OUT_ACC) {
-                    float* dst = reinterpret_cast<float*>(out) + (size_t)row * ldo + col;
-                    *dst += v;
-                } else {
-                    reinterpret_cast<float*>(out)[((size_t)blockIdx.z * M + row) * N + col] = v;
-                }
-            }
+        __syncthreads();
+        const int out0 = n0 / O::PAIR, n_out = N / O::PAIR;
+        uint16_t* o16 = reinterpret_cast<uint16_t*>(out);
+        for (int c = tid; c < BM * (O::WIDTH / 8); c += C::NT) {
+            const int row = c / (O::WIDTH / 8), piece = c % (O::WIDTH / 8);
+            if (m0 + row < M && out0 + piece * 8 < n_out)
+                *reinterpret_cast<uint4*>(o16 + (size_t)(m0 + row) * ldo + out0 + piece * 8) =
+                    *reinterpret_cast<const uint4*>(smem + row * O::STRIDE + piece * 8);
         }
+    } else {
+        gemm_epilogue<C, MODE>(acc, bias, out, ldo, M, N, m0, n0, wm, wn, lane);
     }
 }
 
@@ -250,6 +463,37 @@ static int launch_cfg(const GemmArgs& g, void* out, int splits, int k_per_split)
                                               g.ldo, g.M, g.N, g.K, k_per_split, tiles_m, tiles_n);
     HFA_LAUNCH_CHECK("gemm_mfma");
     return 0;
+}
+
+template <int BM, int BN, int BK, int WM, int WN, int STAGES, int MODE>
+static int launch_dma_cfg(const GemmArgs& g) {
+    using C = DmaCfg<BM, BN, BK, WM, WN>;
+    constexpr int SMEM = STAGES * C::STAGE_BYTES > DmaOut<BN, MODE>::bytes(BM) ? STAGES * C::STAGE_BYTES : DmaOut<BN, MODE>::bytes(BM);
+    auto kernel = gemm_dma_kernel<BM, BN, BK, WM, WN, STAGES, MODE>;
+    static bool configured = false;
+    if (!configured) {
+        hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM);
+        if (e != hipSuccess) {
+            hfa_set_error("gemm_dma: cannot reserve %d bytes of LDS: %s", SMEM, hipGetErrorString(e));
+            return 2;
+        }
+        configured = true;
+    }
+    const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
+    kernel<<<dim3(tiles_m * tiles_n), C::NT, SMEM, g.stream>>>((const uint16_t*)g.a, g.lda, (const uint16_t*)g.w, g.ldw,
+                                                              g.bias, g.out, g.ldo, g.M, g.N, g.K, tiles_m, tiles_n);
+    HFA_LAUNCH_CHECK("gemm_dma");
+    return 0;
+}
+
+template <int BM, int BN, int BK, int WM, int WN, int STAGES>
+static int launch_dma(const GemmArgs& g, int mode) {
+    switch (mode) {
+        case OUT_BF16: return launch_dma_cfg<BM, BN, BK, WM, WN, STAGES, OUT_BF16>(g);
+        case OUT_F32: return launch_dma_cfg<BM, BN, BK, WM, WN, STAGES, OUT_F32>(g);
+        case OUT_ACC: return launch_dma_cfg<BM, BN, BK, WM, WN, STAGES, OUT_ACC>(g);
+        default: return launch_dma_cfg<BM, BN, BK, WM, WN, STAGES, OUT_SWIGLU>(g);
+    }
 }
 
 template <int BM, int BN, int BK, int WM, int WN, int PF = (BM >= 128 ? 1 : 2)>
@@ -319,7 +563,18 @@ int gemm_mfma_launch(const GemmArgs& g, void* workspace, size_t workspace_bytes,
     const int kmode = splits > 1 ? OUT_PARTIAL : mode;
     void* kout = splits > 1 ? workspace : g.out;
     int rc;
-    if (BM == 128)
+    // Long prompts: tiles of 256 rows fed by direct loads into LDS, if the rows they waste past M
+    // cost less than they gain (they run about a quarter faster than the 128 x 128 tiles).
+    const int rows256 = (g.M + 255) / 256 * 256, rows128 = (g.M + 127) / 128 * 128;
+    const bool dma_ok = BM == 128 && splits == 1 && g.K % 64 == 0 && g.lda < (1 << 22) && g.ldw < (1 << 22) &&
+                        (size_t)rows256 * 100 <= (size_t)rows128 * 128 &&
+                        (g.out_dtype != HFA_BF16 || (g.ldo % 8 == 0 && g.N % 16 == 0 && ((uintptr_t)g.out & 15) == 0));
+    const int tiles256 = (rows256 / 256) * ((g.N + 255) / 256);
+    if (dma_ok && tiles256 >= 128)
+        rc = launch_dma<256, 256, 32, 2, 4, 4>(g, kmode);
+    else if (dma_ok && 2 * tiles256 >= 128)
+        rc = launch_dma<256, 128, 64, 2, 2, 3>(g, kmode);
+    else if (BM == 128)
         rc = launch_mode<128, 128, 64, 2, 2>(g, kmode, kout, splits, k_per_split);
     else if (BM == 64)
         rc = launch_mode<64, 128, 64, 2, 2>(g, kmode, kout, splits, k_per_split);

@@ -96,11 +96,14 @@ def test_gemm(ops32, adt, wdt, odt, M, N, K):
 
 @pytest.mark.parametrize("M,N,K", [(1, 256, 512), (8, 4608, 3584), (8, 3584, 18944), (33, 200, 1000),
                                    (64, 1000, 4096), (65, 129, 72), (200, 333, 264), (500, 1100, 1024),
-                                   (2048, 512, 3584)])
+                                   (2048, 512, 3584), (2048, 4608, 1024), (1000, 8200, 512), (700, 5408, 640),
+                                   (2048, 3584, 1024), (1024, 8192, 64), (2048, 3584, 64), (512, 4096, 128)])
 def test_gemm_on_matrix_cores(ops16, M, N, K):
-    """bf16 x bf16 with K a multiple of 8 runs on the matrix cores (K split for small M): against
-    fp64 on the rounded operands, against the plain kernel on the same operands, in the three
-    output modes, with operands that are views of wider buffers."""
+    """bf16 x bf16 with K a multiple of 8 runs on the matrix cores (K split for small M; tiles of
+    256 rows loaded straight into LDS for long prompts and wide outputs, with edges in M and N
+    and as few as one or two steps of K): against fp64 on the rounded operands, against the
+    plain kernel on the same operands, in the three output modes, with operands that are views
+    of wider buffers."""
     rng = np.random.default_rng(M + N + K)
     a = rng.standard_normal((M, K)).astype(np.float32)
     w = (rng.standard_normal((N, K)) / math.sqrt(K)).astype(np.float32)
@@ -129,12 +132,12 @@ def test_gemm_on_matrix_cores(ops16, M, N, K):
     assert np.max(np.abs(acc.cpu().numpy() - (want + res))) <= 2e-5 * scale
 
 
-@pytest.mark.parametrize("M", [1, 8, 64, 100, 300])
-def test_gemm_with_gate_up_epilogue(ops16, M):
+@pytest.mark.parametrize("M,E,F", [(1, 256, 352), (8, 256, 352), (64, 256, 352), (100, 256, 352), (300, 256, 352),
+                                   (1500, 192, 16416), (600, 320, 4512)])
+def test_gemm_with_gate_up_epilogue(ops16, M, E, F):
     """Gate and up rows interleaved in blocks of 32; the product's last step forms silu(gate) * up:
     directly in the tile's epilogue (large M) or when the split K is added up (small M)."""
     rng = np.random.default_rng(M)
-    E, F = 256, 352
     x = rng.standard_normal((M, E)).astype(np.float32)
     wg = (rng.standard_normal((F, E)) / 16).astype(np.float32)
     wu = (rng.standard_normal((F, E)) / 16).astype(np.float32)

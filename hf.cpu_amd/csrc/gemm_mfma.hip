@@ -573,7 +573,7 @@ int gemm_mfma_launch(const GemmArgs& g, void* workspace, size_t workspace_bytes,
     if (dma_ok && tiles256 >= 128)
         rc = launch_dma<256, 256, 32, 2, 4, 4>(g, kmode);
     else if (dma_ok && 2 * tiles256 >= 128)
-        rc = launch_dma<256, 128, 64, 2, 2, 3>(g, kmode);
+        rc = launch_dma<256, 128, 32, 4, 2, 6>(g, kmode);
     else if (BM == 128)
         rc = launch_mode<128, 128, 64, 2, 2>(g, kmode, kout, splits, k_per_split);
     else if (BM == 64)

@@ -543,6 +543,18 @@ int gemm_mfma_launch(const GemmArgs& g, void* workspace, size_t workspace_bytes,
         hfa_set_error("gemm: the gate/up epilogue needs N a multiple of 64, no bias and a bf16 output");
         return 1;
     }
+    if (g.M <= 64) {
+        const int slots = gemm_stream_slots(g, workspace ? workspace_bytes : 0);
+        if (slots > 0) {
+            const int rc = gemm_stream_launch(g, workspace, slots);
+            if (rc) return rc;
+            if (defer && pending_splits) {
+                *pending_splits = slots;
+                return 0;
+            }
+            return gemm_finish_launch((const float*)workspace, slots, g.bias, g.out, mode, g.ldo, g.M, g.N, g.stream);
+        }
+    }
     const int BK = 64;
     const int BM = g.M > 64 ? 128 : (g.M > 32 ? 64 : 32), BN = 128;
     const int tiles = ((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN);

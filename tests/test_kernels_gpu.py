@@ -97,11 +97,13 @@ def test_gemm(ops32, adt, wdt, odt, M, N, K):
 @pytest.mark.parametrize("M,N,K", [(1, 256, 512), (8, 4608, 3584), (8, 3584, 18944), (33, 200, 1000),
                                    (64, 1000, 4096), (65, 129, 72), (200, 333, 264), (500, 1100, 1024),
                                    (2048, 512, 3584), (2048, 4608, 1024), (1000, 8200, 512), (700, 5408, 640),
-                                   (2048, 3584, 1024), (1024, 8192, 64), (2048, 3584, 64), (512, 4096, 128)])
+                                   (2048, 3584, 1024), (1024, 8192, 64), (2048, 3584, 64), (512, 4096, 128),
+                                   (64, 4608, 3584), (48, 3584, 18944), (33, 37888, 256), (40, 1024, 8192)])
 def test_gemm_on_matrix_cores(ops16, M, N, K):
     """bf16 x bf16 with K a multiple of 8 runs on the matrix cores (K split for small M; tiles of
     256 rows loaded straight into LDS for long prompts and wide outputs, with edges in M and N
-    and as few as one or two steps of K): against fp64 on the rounded operands, against the
+    and as few as one or two steps of K; for 33 to 64 rows one stream of tile-and-K units cut
+    evenly over the CUs, with runs shorter and longer than a tile's K): against fp64 on the rounded operands, against the
     plain kernel on the same operands, in the three output modes, with operands that are views
     of wider buffers."""
     rng = np.random.default_rng(M + N + K)
@@ -152,11 +154,12 @@ def test_gemm_with_gate_up_epilogue(ops16, M, E, F):
     assert np.max(np.abs(out.float().cpu().numpy() - want)) <= 0.01 * max(1.0, np.max(np.abs(want)))
 
 
-def test_deferred_products_are_finished_by_the_next_kernel(ops16):
-    """A product with few rows and a long K leaves partial sums; the norm that follows adds them
-    into the residual stream and norms the result; rope_store does the same for q, k and v."""
+@pytest.mark.parametrize("M,K,E", [(5, 4096, 512), (40, 8192, 1024)])
+def test_deferred_products_are_finished_by_the_next_kernel(ops16, M, K, E):
+    """A product with few rows and a long K leaves partial sums (for 40 rows: the planes of the
+    streamed product); the norm that follows adds them into the residual stream and norms the
+    result; rope_store does the same for q, k and v."""
     rng = np.random.default_rng(0)
-    M, K, E = 5, 4096, 512
     a = rng.standard_normal((M, K)).astype(np.float32)
     w = (rng.standard_normal((E, K)) / 64).astype(np.float32)
     b = rng.standard_normal(E).astype(np.float32)
@@ -183,9 +186,11 @@ def test_deferred_products_are_finished_by_the_next_kernel(ops16):
     qkv = torch.zeros((M, (H + 2 * G) * D), dtype=torch.bfloat16, device="cuda")
     ops16.gemm(dev(a, torch.bfloat16), dev(wq, torch.bfloat16), qkv, bias=dev(bq), defer=True)
     assert ops16._pending is not None
-    cache = FakeCache(group=0, k=torch.zeros((8, G * D), dtype=torch.bfloat16, device="cuda"),
-                      v=torch.zeros((8, G * D), dtype=torch.bfloat16, device="cuda"), page_tokens=4)
-    positions, slot_map = [3, 0, 9, 100, 7], [0, 5, 2, 7, 1]
+    rows = (M + 3 + 3) // 4 * 4
+    cache = FakeCache(group=0, k=torch.zeros((rows, G * D), dtype=torch.bfloat16, device="cuda"),
+                      v=torch.zeros((rows, G * D), dtype=torch.bfloat16, device="cuda"), page_tokens=4)
+    positions = [int(p) for p in rng.integers(0, 200, M)]
+    slot_map = [int(p) for p in rng.permutation(M + 3)[:M]]
     i = np.arange(D // 2, dtype=np.float64)
     inv_freq = dev((1e4 ** (-2.0 * i / D)).astype(np.float32))
     ops16.rope_store(qkv, ints(positions), inv_freq, D, H, G, D, cache, ints(slot_map))

@@ -14,6 +14,9 @@ src/model.c:217-230). Here pages come from shared pools:
 * Pages go back to the pool when the request is released, and, in a group with a
   window ``W``, as soon as every position on the page is ``<= next_pos - W`` for the
   request's next position: no later query can see them.
+* ``fork`` gives a new request the cache of another (src/model.c:271-301): whole pages are
+  shared and counted, the last, partly filled page is copied, because both will write there.
+  A shared page is never written: a request writes only at and beyond its own length.
 * Every request also holds one **state slot** (an index below ``n_slots``) from
   admission to release, for parts that keep per-request state of fixed size; the
   device block tables are indexed by it as well.
@@ -92,6 +95,43 @@ class CacheManager:
         for g, table in enumerate(h.tables):
             self.pools[g].give_back([p for p in table if p >= 0])
         self._free_slots.append(h.slot)
+
+    def fork(self, src_id, new_id):
+        """Admits ``new_id`` with the cache contents of ``src_id``: the same length, the whole
+        pages shared, a page of its own for the last, partly filled block. All or nothing.
+        Returns what the caller has to copy in device memory before either request runs again:
+        ``(page_copies, slot_copy)`` with page_copies = [(group, from_page, to_page)] and
+        slot_copy = (from_slot, to_slot)."""
+        src = self.held.get(src_id)
+        if src is None:
+            fail(EINVAL, f"request {src_id!r} is forked but not admitted")
+        if new_id in self.held:
+            fail(EINVAL, f"request {new_id!r} is already admitted")
+        if src.reserved:
+            fail(EINVAL, f"request {src_id!r} is forked in the middle of a step")
+        if not self._free_slots:
+            raise EngineError(ENOMEM, f"no state slot is free ({self.n_slots} in use)")
+        P = self.page_tokens
+        full, partial = src.length // P, src.length % P != 0
+        if partial:
+            for g, pool in enumerate(self.pools):
+                if pool.n_free < 1:
+                    raise OutOfPages(f"fork of {src_id!r}: group {g} has no page for the last block")
+        h = Held(new_id, self._free_slots.pop(), length=src.length, tables=[])
+        copies = []
+        for g, pool in enumerate(self.pools):
+            table = list(src.tables[g][:full])
+            pool.share([p for p in table if p >= 0])
+            if partial:
+                own = pool.take(1)[0]
+                copies.append((g, src.tables[g][full], own))
+                table.append(own)
+            for b, page in enumerate(table):
+                if page >= 0:
+                    self.appended[g].append((h.slot, b, page))
+            h.tables.append(table)
+        self.held[new_id] = h
+        return copies, (src.slot, h.slot)
 
     # ---- pages ---------------------------------------------------------------
     def _first_needed_block(self, group, next_pos):
@@ -180,6 +220,11 @@ class CacheManager:
             first = self._first_needed_block(g, length)
             if any(p < 0 for p in h.tables[g.index][first:-(-length // self.page_tokens)]):
                 fail(ENOTSUP, f"request {req_id!r}: the window has released pages before {length}")
+        if length % self.page_tokens:
+            for g, pool in enumerate(self.pools):
+                page = h.tables[g][length // self.page_tokens]
+                if page >= 0 and pool.holders(page) > 1:
+                    fail(ENOTSUP, f"request {req_id!r}: position {length} lies on a page shared with a fork")
         h.length = length
         self.rollback(req_id)
 
@@ -208,13 +253,22 @@ class CacheManager:
                 "slots_held": self.n_slots - len(self._free_slots), "requests": len(self.held)}
 
     def check(self):
-        """Raises AssertionError unless every page is either free or held by exactly one
-        request, and every slot likewise."""
+        """Raises AssertionError unless every page is either free or held by exactly as many
+        requests as the pool counts for it (one, unless forks share it), no page beyond a
+        request's last whole block is shared, and every slot is free or held once."""
         for g, pool in enumerate(self.pools):
             pool.check()
-            held = [p for h in self.held.values() for p in h.tables[g] if p >= 0]
-            assert len(held) == len(set(held)), f"group {g}: a page is held twice"
-            assert len(held) == pool.n_held, f"group {g}: {pool.n_held} pages out, {len(held)} in tables"
+            count = {}
+            for h in self.held.values():
+                own = [p for p in h.tables[g] if p >= 0]
+                assert len(own) == len(set(own)), f"group {g}: request {h.req_id!r} holds a page twice"
+                for p in own:
+                    count[p] = count.get(p, 0) + 1
+                for p in h.tables[g][h.length // self.page_tokens:]:
+                    assert p < 0 or pool.holders(p) == 1, f"group {g}: a page that will be written is shared"
+            assert len(count) == pool.n_held, f"group {g}: {pool.n_held} pages out, {len(count)} in tables"
+            for p, n in count.items():
+                assert pool.holders(p) == n, f"group {g}: page {p} has {pool.holders(p)} holders, {n} tables name it"
         slots = [h.slot for h in self.held.values()]
         assert len(slots) == len(set(slots)), "a state slot is held twice"
         assert sorted(slots + self._free_slots) == list(range(self.n_slots)), "a state slot is lost"

@@ -91,7 +91,7 @@ class Cli:
             state["prefilled"] += 1
             if state["prefilled"] == nseq or not multi:
                 dt = time.monotonic() - t0
-                ntok = sum(len(p) for p in prompts) * eff["n"]
+                ntok = sum(len(p) for p in prompts)        # each prompt is computed once, whatever --n
                 self.out.event("prefill", tokens=ntok, cached=0, ms=f"{dt * 1e3:.1f}",
                                tok_per_s=f"{ntok / dt if dt > 0 else 0:.2f}",
                                kv_bytes=s.engine.storage.nbytes())
@@ -137,11 +137,12 @@ class Cli:
             sch = real_scheduler()
             orig_submit = sch.submit
 
-            def submit(r):
-                cli.current.append(r)
-                if cli.cancel:
-                    r.cancel = True
-                return orig_submit(r)
+            def submit(r, forks=()):
+                for q in (r, *forks):
+                    cli.current.append(q)
+                    if cli.cancel:
+                        q.cancel = True
+                return orig_submit(r, forks=forks)
             sch.submit = submit
             return sch
         s.scheduler = watched

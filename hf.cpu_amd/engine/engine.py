@@ -54,6 +54,21 @@ class Engine:
         """The request is finished: its pages and its slot are given back."""
         self.manager.release(req_id)
 
+    def fork(self, src_id, new_id):
+        """Admits ``new_id`` holding what ``src_id`` holds (src/model.c:271-301): whole pages are
+        shared, the last, partly filled page and the state slot are copied. Both requests go on
+        independently afterwards. On an error (no page, no slot) nothing is taken."""
+        copies, (from_slot, to_slot) = self.manager.fork(src_id, new_id)
+        P = self.manager.page_tokens
+        for group, src, dst in copies:
+            for e in self.manager.groups[group].entries:
+                view = self.storage.views[e]
+                view.k[dst * P:(dst + 1) * P].copy_(view.k[src * P:(src + 1) * P])
+                view.v[dst * P:(dst + 1) * P].copy_(view.v[src * P:(src + 1) * P])    # a page's block, whatever its inner order
+        for e in self.manager.state_entries:
+            state = self.storage.views[e].state
+            state[to_slot].copy_(state[from_slot])
+
     # ---- one step ------------------------------------------------------------
     def step(self, entries):
         """``entries``: a list of Entry or (req_id, tokens, want). A request seen for the

@@ -21,6 +21,12 @@ Each step:
     the queue to be recomputed as a prompt, which starts once pages for all its tokens are
     free again (so it is not thrown out again at once). A request that does not fit even
     alone fails with ERANGE.
+
+Several continuations of one prompt (``--n``, src/ops.c:808-825): the prompt is computed once;
+when its last portion is done the other continuations are forked from the first one's cache
+(whole pages shared), and each samples its own first token from the same logits with its own
+seed. A continuation for which no slot or page is free at that moment waits in the queue
+and computes the prompt itself.
 """
 import time
 from collections import deque
@@ -28,7 +34,7 @@ from dataclasses import dataclass, field
 
 from ..cache import OutOfPages
 from ..sampling import Rng, SamplerParams
-from ..status import ECANCEL, EINVAL, ERANGE, EngineError, fail
+from ..status import ECANCEL, EINVAL, ENOMEM, ERANGE, EngineError, fail
 
 WAITING, RUNNING, FINISHED = "waiting", "running", "finished"
 
@@ -59,6 +65,7 @@ class Request:
     t_first: float = None                    # when the prompt was done (first logits)
     t_done: float = None
     admitted_at: int = -1                    # admission order, for the preemption choice
+    forks: list = field(default_factory=list)     # continuations of the same prompt, forked when it is done
 
     @property
     def unfed(self):
@@ -92,7 +99,19 @@ class Scheduler:
         self.on_prefill = None        # callback(request)
 
     # ---- submission --------------------------------------------------------
-    def submit(self, req):
+    def submit(self, req, forks=()):
+        """Queues ``req``. ``forks`` are further requests with the same prompt (other seeds):
+        they do not queue, but start from ``req``'s cache when its prompt is done."""
+        for c in forks:
+            if list(c.prompt) != list(req.prompt):
+                fail(EINVAL, "a fork must have the prompt of the request it is forked from")
+            self._prepare(c)
+        self._prepare(req)
+        req.forks = list(forks)
+        self.waiting.append(req)
+        return req
+
+    def _prepare(self, req):
         if len(req.prompt) == 0:
             fail(EINVAL, "the prompt is empty")                                     # src/ops.c:752
         if len(req.prompt) >= self.ctx_max:
@@ -109,8 +128,6 @@ class Scheduler:
         req.rng = Rng(req.seed)
         req.status = WAITING
         req.t_submit = self.clock()
-        self.waiting.append(req)
-        return req
 
     @property
     def idle(self):
@@ -204,6 +221,9 @@ class Scheduler:
         self.finished.append(r)
         if self.on_finish:
             self.on_finish(r)
+        pending, r.forks = r.forks, []
+        for c in pending:                      # the prompt never got done: its other continuations end with it
+            self._finish(c, stop=stop, error=error)
 
     # ---- one step ------------------------------------------------------------
     def step(self):
@@ -239,9 +259,34 @@ class Scheduler:
             r.n_fed += n
         if sampled:
             choices = self.sampler.sample(logits, [(r.params, r.rng, r.logprobs) for r in sampled])
-            for r, ch in zip(sampled, choices):
+            for i, (r, ch) in enumerate(zip(sampled, choices)):
+                forked = self._fork(r, logits[i:i + 1]) if r.forks and r.t_first is None else []
                 self._accept(r, ch)
+                for c, cch in forked:
+                    self._accept(c, cch)
         return plan
+
+    def _fork(self, r, row):
+        """``r``'s prompt is done: its other continuations take its cache and draw their first
+        token from the same logits. Returns [(request, choice)] of those that could be forked."""
+        pending, r.forks = r.forks, []
+        out = []
+        for c in pending:
+            try:
+                if len(self.running) >= self.max_seqs:
+                    raise OutOfPages("as many sequences are live as may be")
+                self.engine.fork(r.req_id, c.req_id)
+            except EngineError as e:
+                if e.code != ENOMEM:
+                    raise
+                self.waiting.append(c)         # no room now: it computes the prompt itself later
+                continue
+            c.status, c.n_fed = RUNNING, r.n_fed
+            c.admitted_at = self._admissions
+            self._admissions += 1
+            self.running.append(c)
+            out.append((c, self.sampler.sample(row, [(c.params, c.rng, c.logprobs)])[0]))
+        return out
 
     def _accept(self, r, ch):
         if r.t_first is None:

@@ -97,11 +97,12 @@ class Session:
         params = SamplerParams(float(temp), int(top_k), float(top_p), float(min_p)).check()
         sched = self.scheduler()
         eos = self.eos_ids if eos_ids is None else tuple(eos_ids)
-        reqs = []
+        reqs, families = [], []
         for p in prompts:
-            for i in range(n):
-                reqs.append(Request(len(reqs), list(p), params, int(max_tokens), int(seed) + i,
-                                    min(int(logprobs), 64), eos, float(timeout)))
+            family = [Request(len(reqs) + i, list(p), params, int(max_tokens), int(seed) + i,
+                              min(int(logprobs), 64), eos, float(timeout)) for i in range(n)]
+            reqs += family
+            families.append(family)
         if on_token:
             sched.on_token = lambda r, ch: on_token(r.req_id, len(r.generated) - 1, ch)
         if on_prefill:
@@ -109,8 +110,8 @@ class Session:
         if on_finish:
             sched.on_finish = lambda r: on_finish(r.req_id, r)
         try:
-            for r in reqs:
-                sched.submit(r)
+            for family in families:            # the prompt is computed once, the others fork from it
+                sched.submit(family[0], forks=family[1:])
             sched.run()
         finally:
             for r in reqs:                     # an error mid-way leaves nothing behind (src/ops.c:930)

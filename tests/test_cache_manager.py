@@ -1,5 +1,6 @@
-"""The cache manager's books (no GPU): no page is lost, held twice or freed twice, under
-random orders of requests; the window gives pages back; reservations are all-or-nothing."""
+"""The cache manager's books (no GPU): no page is lost, held by more requests than the pool
+counts, or freed twice, under random orders of requests (new ones, forks, steps, releases);
+the window gives pages back; reservations and forks are all-or-nothing."""
 import random
 
 import pytest
@@ -114,8 +115,25 @@ def test_random_orders_keep_the_books(seed):
         if (r < 0.25 and len(live) < 4) or not live:
             name = f"q{counter}"
             counter += 1
-            m.admit(name)
-            live[name] = 0
+            if live and rng.random() < 0.4:    # start from another request's cache
+                src = rng.choice(list(live))
+                before = [p.n_free for p in m.pools]
+                try:
+                    copies, (s_from, s_to) = m.fork(src, name)
+                except OutOfPages:
+                    m.check()
+                    assert name not in m.held and [p.n_free for p in m.pools] == before
+                    continue
+                live[name] = live[src]
+                assert m.held[name].length == live[src] and s_from == m.held[src].slot and s_to == m.held[name].slot
+                assert len(copies) == (len(m.groups) if live[src] % 4 else 0)
+                for g, a, b in copies:         # the last, partly filled block: a page of its own
+                    assert m.held[src].tables[g][live[src] // 4] == a and m.held[name].tables[g][live[src] // 4] == b != a
+                for g in m.groups:             # whole blocks: the same pages
+                    assert m.held[name].tables[g.index][:live[src] // 4] == m.held[src].tables[g.index][:live[src] // 4]
+            else:
+                m.admit(name)
+                live[name] = 0
         elif r < 0.85:
             name = rng.choice(list(live))
             n = rng.choice([1, 1, 1, 2, 3, 5, 9, 14])
@@ -149,3 +167,64 @@ def test_random_orders_keep_the_books(seed):
         m.release(name)
     m.check()
     assert all(p.n_held == 0 for p in m.pools) and any(p.reused > 0 for p in m.pools)
+
+
+def test_fork_shares_whole_pages_and_copies_the_last():
+    m = manager(n_pages=8, page=4, slots=3, window=0, ctx=32)
+    m.admit("a")
+    m.reserve("a", 10)
+    m.commit("a", 10)
+    for g in range(len(m.groups)):
+        m.drain_appended(g)
+    copies, slots = m.fork("a", "b")
+    a, b = m.held["a"], m.held["b"]
+    assert b.length == 10 and slots == (a.slot, b.slot) and a.slot != b.slot
+    for g in range(len(m.groups)):
+        assert b.tables[g][:2] == a.tables[g][:2] and b.tables[g][2] != a.tables[g][2]
+        assert (g, a.tables[g][2], b.tables[g][2]) in copies
+        assert all(m.pools[g].holders(p) == 2 for p in a.tables[g][:2])
+        assert sorted(m.drain_appended(g)) == sorted((b.slot, i, p) for i, p in enumerate(b.tables[g]))
+        assert m.pools[g].n_held == 4                  # three of a's, one more for b
+    m.check()
+    # both go on independently; a shared page returns to the pool when its last holder lets go
+    m.reserve("b", 3)
+    m.commit("b", 3)
+    m.reserve("a", 1)
+    m.commit("a", 1)
+    m.check()
+    m.release("a")
+    for g in range(len(m.groups)):
+        assert m.pools[g].n_held == 4 and all(m.pools[g].holders(p) == 1 for p in b.tables[g])
+    m.check()
+    with pytest.raises(EngineError):                   # the name is taken
+        m.fork("b", "b")
+    m.truncate("b", 6)                                 # the page of position 6 is b's alone by now
+    m.release("b")
+    m.check()
+    assert all(p.n_held == 0 for p in m.pools)
+
+
+def test_fork_is_all_or_nothing_and_guards_shared_pages():
+    m = manager(n_pages=3, page=4, slots=2, window=0, ctx=12)
+    m.admit("a")
+    m.reserve("a", 10)
+    m.commit("a", 10)                                  # all three pages
+    with pytest.raises(OutOfPages):
+        m.fork("a", "b")                               # the copy of the last block needs a page
+    assert "b" not in m.held and m.held["a"].length == 10
+    m.check()
+    m.truncate("a", 8)                                 # two whole pages: nothing to copy
+    copies, _ = m.fork("a", "b")
+    assert copies == [] and all(m.pools[g].n_held == 2 for g in range(len(m.groups)))
+    with pytest.raises(EngineError) as e:              # a third request: no slot
+        m.fork("a", "c")
+    assert e.value.code == "ENOMEM"
+    with pytest.raises(EngineError) as e:              # writing at position 6 would change b's keys too
+        m.truncate("a", 6)
+    assert e.value.code == "ENOTSUP"
+    m.truncate("a", 4)                                 # a page boundary: a lets go of the second page, b keeps it
+    m.check()
+    m.reserve("a", 2)
+    m.commit("a", 2)
+    assert m.held["a"].tables[0][1] != m.held["b"].tables[0][1]
+    m.check()

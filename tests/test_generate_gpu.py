@@ -88,6 +88,33 @@ def test_sampling_is_reproducible_and_follows_the_plain_sampler(gpu, models):
         toks.append(t)
 
 
+@pytest.mark.parametrize("name,length", [("A", 21), ("B", 43), ("B", 150)])
+def test_continuations_fork_from_one_prompt(gpu, models, name, length):
+    """``n`` continuations: the prompt is computed once (counted in steps), the others start
+    from its cache (whole pages shared, the last, partly filled page copied; in B some layers
+    have a window that has already given pages back at 150 tokens), and continuation i gives
+    what it gives alone with seed + i (tests/e2e.pl:224: alone or in a fan-out, the same)."""
+    import hf_cpu_amd.session as S
+    cfg = helpers.CONFIGS[name]
+    prompt = helpers.random_requests(cfg, [length], seed=length)["r0"]
+    s = S.Session(models[name], dtype="float32", ctx_max=256, batch=16, page_size=helpers.PAGE[name], max_seqs=4)
+    before = s.engine.steps_run
+    fan = s.generate(prompt, n=4, temp=0.9, seed=3, max_tokens=12)
+    assert all(g.stop == "length" for g in fan) and not s.engine.manager.held
+    assert s.engine.steps_run - before == -(-length // 16) + 11
+    s.engine.manager.check()
+    assert len({tuple(g.tokens) for g in fan}) > 1
+    for i, g in enumerate(fan):
+        assert s.generate(prompt, n=1, temp=0.9, seed=3 + i, max_tokens=12)[0].tokens == g.tokens, f"continuation {i}"
+    # greedy continuations are all the plain implementation's
+    want, _ = plain_greedy(models[name], prompt, 6)
+    assert [g.tokens for g in s.generate(prompt, n=3, temp=0.0, max_tokens=6)] == [want] * 3
+    # bf16: the forked caches serve too (each continuation against itself alone)
+    s16 = S.Session(models[name], dtype="bfloat16", ctx_max=256, batch=16, page_size=helpers.PAGE[name], max_seqs=4)
+    fan16 = s16.generate(prompt, n=3, temp=0.0, max_tokens=8)
+    assert fan16[0].tokens == fan16[1].tokens == fan16[2].tokens
+
+
 def run_cli(args, stdin=""):
     r = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "hfamd")] + args, input=stdin, text=True,
                        capture_output=True, timeout=300)

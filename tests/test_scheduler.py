@@ -23,6 +23,10 @@ class FakeEngine:
     def release(self, r):
         self.manager.release(r)
 
+    def fork(self, src, new):
+        self.manager.fork(src, new)
+        self.log.append([("fork", src, new)])
+
     def step(self, entries):
         m = self.manager
         for r, toks, want in entries:
@@ -219,3 +223,46 @@ def test_windowed_group_frees_pages_for_others():
     # 33 tokens need 9 pages in the full group: it fails there, but the windowed group never held more than 3
     assert eng.manager.pools[1].high_water <= 3
     assert r.error is not None and r.error.code == "ERANGE"
+
+
+def test_continuations_of_one_prompt_fork_from_its_cache():
+    eng, s = make(budget=8, n_pages=16, slots=4)
+    fam = [Request(f"c{i}", list(range(10)), greedy(), max_tokens=3, seed=i) for i in range(3)]
+    s.submit(fam[0], forks=fam[1:])
+    assert list(s.waiting) == [fam[0]]                 # the others do not queue
+    s.step()
+    assert eng.log[-1] == [("c0", 8, [])]
+    s.step()                                           # the prompt's end: the others take its cache
+    assert eng.log[-3:] == [[("c0", 2, [1])], [("fork", "c0", "c1")], [("fork", "c0", "c2")]]
+    assert [r.req_id for r in s.running] == ["c0", "c1", "c2"] and all(len(r.generated) == 1 for r in fam)
+    assert all(r.n_fed == 10 for r in fam)
+    m = eng.manager
+    assert m.held["c1"].tables[0][:2] == m.held["c0"].tables[0][:2] and m.held["c1"].tables[0][2] != m.held["c0"].tables[0][2]
+    s.step()
+    assert eng.log[-1] == [("c0", 1, [0]), ("c1", 1, [0]), ("c2", 1, [0])]      # the prompt was computed once
+    s.run()
+    assert all(r.stop == "length" and len(r.generated) == 3 for r in fam)
+    assert all(p.n_held == 0 for p in m.pools)
+    m.check()
+
+
+def test_a_continuation_without_room_computes_the_prompt_itself():
+    eng, s = make(budget=16, n_pages=16, slots=2)
+    fam = [Request(f"c{i}", list(range(6)), greedy(), max_tokens=2, seed=i) for i in range(3)]
+    s.submit(fam[0], forks=fam[1:])
+    s.step()                                           # two slots: c1 forks, c2 has to wait
+    assert [r.req_id for r in s.running] == ["c0", "c1"] and list(s.waiting) == [fam[2]]
+    s.run()
+    assert all(r.stop == "length" and len(r.generated) == 2 for r in fam)
+    assert any(step == [("c2", 6, [5])] or ("c2", 6, [5]) in step for step in eng.log)
+    eng.manager.check()
+
+
+def test_continuations_end_with_a_prompt_that_fails():
+    eng, s = make(budget=8, n_pages=2, page=4, ctx=64)
+    fam = [Request(f"c{i}", list(range(20)), greedy(), max_tokens=2, seed=i) for i in range(2)]
+    s.submit(fam[0], forks=fam[1:])
+    s.run()
+    assert all(r.error is not None and r.error.code == "ERANGE" for r in fam)
+    with pytest.raises(EngineError):
+        s.submit(Request("x", [1, 2], greedy()), forks=[Request("y", [1, 3], greedy())])

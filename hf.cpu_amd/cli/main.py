@@ -107,10 +107,13 @@ class Cli:
 
         try:
             self.busy = True
+            if eff["profile"]:
+                s.engine.profile_start()
             gens = self._run_generate(s, prompts, eff, eos, on_token, on_prefill)
         finally:
             self.busy = False
             self.current = []
+            times = s.engine.profile_stop() if eff["profile"] else None
         dt = time.monotonic() - (state["t_dec0"] or t0)
         total = 0
         for g in gens:
@@ -123,6 +126,9 @@ class Cli:
             self.out.event("genall", sequences=nseq, tokens=total, ms=f"{dt * 1e3:.1f}",
                            tok_per_s=f"{total / dt if dt > 0 else 0:.2f}")
         if eff["profile"]:
+            for stage in ("prefill", "decode"):        # the reference's fields, src/ops.c:593-603
+                self.out.event("profile", stage=stage, **{k: f"{times[stage].get(k, 0.0):.3f}" for k in
+                               ("embed", "glue", "qkv", "attn", "wo", "gate_up", "silu", "down", "head", "sample")})
             st = s.engine.manager.stats()
             self.out.event("profile", stage="cache", steps=s.engine.steps_run,
                            pages_high_water=max((g["high_water"] for g in st["groups"]), default=0),

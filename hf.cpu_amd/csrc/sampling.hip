@@ -82,48 +82,178 @@ extern "C" int hfa_argmax(const float* logits, int ld, int* out, int n_rows, int
     return 0;
 }
 
-// One block per row. Pass c finds the best candidate that comes after the one chosen in
-// pass c-1 in the ordering, so nothing is modified and the order is exact.
-__global__ __launch_bounds__(1024) void topk_kernel(const float* __restrict__ logits, int ld, int* __restrict__ ids,
-                                                    float* __restrict__ vals, float* __restrict__ stats, int vocab,
-                                                    int k) {
-    __shared__ float sv[17];
-    __shared__ int si[17];
+// Ordered best-k of a row, one block of 1024 threads per row, in a fixed number of passes over
+// the row (which stays in L2) whatever k is:
+//  1. the k-th largest value is found by three histogram passes over the order-preserving
+//     integer image of the floats (11 + 11 + 10 bits); pass 1 also finds the maximum, pass 2
+//     also adds up exp(l - max) for the log-sum-exp;
+//  2. two sweeps collect the values above it and, of the values equal to it, those with the
+//     smallest ids until k are together: each wave owns a contiguous segment of the row and
+//     walks it 64 ids at a time, so ballots and counts give every candidate its place in id
+//     order without atomics;
+//  3. the k candidates are sorted in LDS (bitonic) by (logit descending, id ascending).
+#define TOPK_THREADS 1024
+#define TOPK_MAX 1024
+
+__device__ __forceinline__ uint32_t float_key(float v) {     // larger float <=> larger key
+    const uint32_t u = __float_as_uint(v);
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+// Among the histogram's bins, from the top: the bin that holds the `rank`-th largest element
+// (rank counts from 1). Returns the bin; `rank` becomes the rank inside that bin. All threads
+// call it; `hist` and `pick` are LDS.
+__device__ int topk_find_bin(const uint32_t* hist, int n_bins, int& rank, int* pick) {
+    __syncthreads();
+    if (threadIdx.x < WAVE) {
+        const int per = n_bins / WAVE, lane = threadIdx.x;
+        uint32_t c = 0;
+        for (int j = 0; j < per; j++) c += hist[lane * per + j];
+        // elements in chunks above this lane's
+        uint32_t above = 0;
+        for (int l = WAVE - 1; l >= 0; l--) {
+            const uint32_t cl = __shfl(c, l, WAVE);
+            if (l > lane) above += cl;
+        }
+        if (above < (uint32_t)rank && (uint32_t)rank <= above + c) {     // exactly one lane
+            uint32_t seen = above;
+            int bin = lane * per + per - 1;
+            for (; bin > lane * per; bin--) {
+                if (seen + hist[bin] >= (uint32_t)rank) break;
+                seen += hist[bin];
+            }
+            pick[0] = bin;
+            pick[1] = rank - (int)seen;
+        }
+    }
+    __syncthreads();
+    rank = pick[1];
+    return pick[0];
+}
+
+__global__ __launch_bounds__(TOPK_THREADS) void topk_kernel(const float* __restrict__ logits, int ld,
+                                                            int* __restrict__ ids, float* __restrict__ vals,
+                                                            float* __restrict__ stats, int vocab, int k) {
+    __shared__ uint32_t hist[2048];
+    __shared__ float cand_v[TOPK_MAX];
+    __shared__ int cand_i[TOPK_MAX];
+    __shared__ int pick[2];
+    __shared__ int wave_above[TOPK_THREADS / WAVE + 1], wave_equal[TOPK_THREADS / WAVE + 1];
     __shared__ float red[17];
     const float* row = logits + (size_t)blockIdx.x * ld;
-    float pv = INFINITY;
-    int pi = -1;
-    float mx = 0.f;
-    for (int c = 0; c < k; c++) {
-        float bv = -INFINITY;
-        int bi = 0x7fffffff;
-        for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
-            const float v = row[i];
-            const bool after = v < pv || (v == pv && i > pi);
-            if (after && better(v, i, bv, bi)) { bv = v; bi = i; }
-        }
-        block_best(bv, bi, sv, si);
-        if (threadIdx.x == 0) {
-            ids[(size_t)blockIdx.x * k + c] = bi == 0x7fffffff ? -1 : bi;
-            vals[(size_t)blockIdx.x * k + c] = bv;
-        }
-        if (c == 0) mx = bv;
-        pv = bv;
-        pi = bi;
+    const int tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
+    constexpr int NW = TOPK_THREADS / WAVE;
+
+    // ---- pass 1: top 11 bits, and the maximum ----
+    for (int i = tid; i < 2048; i += TOPK_THREADS) hist[i] = 0;
+    __syncthreads();
+    float mx = -INFINITY;
+    for (int i = tid; i < vocab; i += TOPK_THREADS) {
+        const float v = row[i];
+        mx = fmaxf(mx, v);
+        if (k > 0) atomicAdd(&hist[float_key(v) >> 21], 1u);
     }
-    if (stats) {
-        if (k == 0) {
-            float bv = -INFINITY;
-            for (int i = threadIdx.x; i < vocab; i += blockDim.x) bv = fmaxf(bv, row[i]);
-            mx = block_max(bv, red);
+    mx = block_max(mx, red);
+    uint32_t prefix = 0;
+    int rank = k;
+    if (k > 0) prefix = (uint32_t)topk_find_bin(hist, 2048, rank, pick);
+
+    // ---- pass 2: the next 11 bits among the elements of that bin, and the sum of exp(l - max) ----
+    for (int i = tid; i < 2048; i += TOPK_THREADS) hist[i] = 0;
+    __syncthreads();
+    float sum = 0.f;
+    for (int i = tid; i < vocab; i += TOPK_THREADS) {
+        const float v = row[i];
+        sum += expf(v - mx);
+        const uint32_t key = float_key(v);
+        if (k > 0 && (key >> 21) == prefix) atomicAdd(&hist[(key >> 10) & 0x7ffu], 1u);
+    }
+    sum = block_sum(sum, red);
+    if (stats && tid == 0) {
+        stats[2 * blockIdx.x] = mx;
+        stats[2 * blockIdx.x + 1] = logf(sum);
+    }
+    if (k == 0) return;
+    prefix = (prefix << 11) | (uint32_t)topk_find_bin(hist, 2048, rank, pick);
+
+    // ---- pass 3: the last 10 bits ----
+    for (int i = tid; i < 1024; i += TOPK_THREADS) hist[i] = 0;
+    __syncthreads();
+    for (int i = tid; i < vocab; i += TOPK_THREADS) {
+        const uint32_t key = float_key(row[i]);
+        if ((key >> 10) == prefix) atomicAdd(&hist[key & 0x3ffu], 1u);
+    }
+    const uint32_t kth = (prefix << 10) | (uint32_t)topk_find_bin(hist, 1024, rank, pick);
+    const int n_equal = rank, n_above = k - rank;            // of the values equal to the k-th, the `rank` smallest ids
+
+    // ---- sweep 1: how many candidates each wave's segment holds ----
+    const int seg = (vocab + NW - 1) / NW;
+    const int lo = wave * seg, hi = lo + seg < vocab ? lo + seg : vocab;
+    int above = 0, equal = 0;
+    for (int i = lo + lane; i < hi; i += WAVE) {
+        const uint32_t key = float_key(row[i]);
+        above += key > kth;
+        equal += key == kth;
+    }
+#pragma unroll
+    for (int off = WAVE / 2; off > 0; off >>= 1) {
+        above += __shfl_xor(above, off, WAVE);
+        equal += __shfl_xor(equal, off, WAVE);
+    }
+    if (lane == 0) { wave_above[wave] = above; wave_equal[wave] = equal; }
+    __syncthreads();
+    int base_above = 0, base_equal = 0;                      // candidates in the segments before this wave's
+    for (int w = 0; w < wave; w++) { base_above += wave_above[w]; base_equal += wave_equal[w]; }
+
+    // ---- sweep 2: every candidate to its place: the values above first, then the ties in id order ----
+    for (int i0 = lo; i0 < hi; i0 += WAVE) {
+        const int i = i0 + lane;
+        const float v = i < hi ? row[i] : 0.f;
+        const uint32_t key = float_key(v);
+        const bool is_above = i < hi && key > kth, is_equal = i < hi && key == kth;
+        const unsigned long long ma = __ballot(is_above), me = __ballot(is_equal);
+        const unsigned long long below = (1ull << lane) - 1ull;
+        if (is_above) {
+            const int at = base_above + __popcll(ma & below);
+            cand_v[at] = v;
+            cand_i[at] = i;
         }
-        float s = 0.f;
-        for (int i = threadIdx.x; i < vocab; i += blockDim.x) s += expf(row[i] - mx);
-        s = block_sum(s, red);
-        if (threadIdx.x == 0) {
-            stats[2 * blockIdx.x] = mx;
-            stats[2 * blockIdx.x + 1] = logf(s);
+        if (is_equal) {
+            const int r = base_equal + __popcll(me & below);
+            if (r < n_equal) {
+                cand_v[n_above + r] = v;
+                cand_i[n_above + r] = i;
+            }
         }
+        base_above += __popcll(ma);
+        base_equal += __popcll(me);
+    }
+    int n = 2;
+    while (n < k) n <<= 1;
+    for (int i = k + tid; i < n; i += TOPK_THREADS) {        // padding sorts to the end
+        cand_v[i] = -INFINITY;
+        cand_i[i] = 0x7fffffff;
+    }
+
+    // ---- sort: bitonic network over n <= 1024 entries, one thread per entry ----
+    for (int size = 2; size <= n; size <<= 1)
+        for (int stride = size >> 1; stride > 0; stride >>= 1) {
+            __syncthreads();
+            const int j = tid ^ stride;
+            if (tid < n && j > tid) {
+                const bool forward = (tid & size) == 0;      // this pair's better entry goes first
+                const float va = cand_v[tid], vb = cand_v[j];
+                const int ia = cand_i[tid], ib = cand_i[j];
+                if (better(vb, ib, va, ia) == forward) {
+                    cand_v[tid] = vb; cand_i[tid] = ib;
+                    cand_v[j] = va; cand_i[j] = ia;
+                }
+            }
+        }
+    __syncthreads();
+    for (int c = tid; c < k; c += TOPK_THREADS) {
+        ids[(size_t)blockIdx.x * k + c] = cand_i[c] == 0x7fffffff ? -1 : cand_i[c];
+        vals[(size_t)blockIdx.x * k + c] = cand_v[c];
     }
 }
 
@@ -132,7 +262,7 @@ extern "C" int hfa_topk(const float* logits, int ld, int* ids, float* vals, floa
     HFA_REQUIRE(n_rows > 0 && vocab > 0 && ld >= vocab, "topk: bad sizes rows=%d vocab=%d ld=%d", n_rows, vocab, ld);
     HFA_REQUIRE(k >= 0 && k <= 1024 && k <= vocab, "topk: k=%d is outside 0..min(1024, vocab)", k);
     HFA_REQUIRE(k == 0 || (ids && vals), "topk: no output for the candidates");
-    topk_kernel<<<n_rows, 1024, 0, stream>>>(logits, ld, ids, vals, stats, vocab, k);
+    topk_kernel<<<n_rows, TOPK_THREADS, 0, stream>>>(logits, ld, ids, vals, stats, vocab, k);
     HFA_LAUNCH_CHECK("topk");
     return 0;
 }

@@ -42,6 +42,7 @@ class Engine:
         self._graphs = {}
         self._graph_seen = set()
         self.graph_replays = 0
+        self.profile = None           # while timing: {"prefill" | "decode": {part: milliseconds}}
 
     # ---- requests ------------------------------------------------------------
     def has(self, req_id):
@@ -68,6 +69,28 @@ class Engine:
         for e in self.manager.state_entries:
             state = self.storage.views[e].state
             state[to_slot].copy_(state[from_slot])
+
+    # ---- timing by part (src/model.h:75-79; reported by --profile, src/ops.c:593-603) ----
+    def profile_start(self):
+        """From now on every step's device time is booked by part (embed, qkv, attn, wo, gate_up,
+        silu, down, head; the rest, norms, rotary, cache stores and partial sums, as glue),
+        under ``prefill`` if the step holds a prompt portion, else under ``decode``. Steps run
+        eagerly and the host waits for each, so the total is larger than without timing."""
+        self.ops.timing(True)
+        self.profile = {"prefill": {}, "decode": {}}
+
+    def profile_stop(self):
+        out, self.profile = self.profile, None
+        self.ops.timing(False)
+        return out
+
+    def _book_times(self, stage):
+        times = self.ops.take_times()
+        book = self.profile[stage]
+        named = sum(v for k, v in times.items() if k != "total")
+        times["glue"] = max(times.pop("total", 0.0) - named, 0.0)
+        for k, v in times.items():
+            book[k] = book.get(k, 0.0) + v
 
     # ---- one step ------------------------------------------------------------
     def step(self, entries):
@@ -107,6 +130,8 @@ class Engine:
             logits = self.ops.scratch("logits", (max(step.n_logit_rows, 1), self.vocab_size), torch.float32)
             logits = logits[:step.n_logit_rows]
             self._run(step, logits)
+            if self.profile is not None:
+                self._book_times("prefill" if step.max_q_len > 1 else "decode")
         except BaseException:
             for r in reserved:
                 mgr.rollback(r)
@@ -121,7 +146,7 @@ class Engine:
     def _run(self, step, logits):
         """The forward pass of the step, eagerly or as a replay of the graph of its shape."""
         decode_only = step.max_q_len == 1 and step.n_tokens <= self.GRAPH_MAX_TOKENS
-        if not (self.use_graphs and decode_only):
+        if not (self.use_graphs and decode_only) or self.profile is not None:
             return self.model.forward(self.ops, step, self.storage.views, logits)
         # The kernels use max_seq_len only to choose how the key range is cut, so a graph
         # captured for a length bucket serves every shorter length too.

@@ -258,7 +258,12 @@ class Scheduler:
         for r, n, _ in plan.entries:
             r.n_fed += n
         if sampled:
+            t0 = time.perf_counter()
             choices = self.sampler.sample(logits, [(r.params, r.rng, r.logprobs) for r in sampled])
+            book = getattr(self.engine, "profile", None)
+            if book is not None:               # sampling is timed on the host, as in src/ops.c:845-847
+                stage = book["prefill" if any(n > 1 for _, n, _ in plan.entries) else "decode"]
+                stage["sample"] = stage.get("sample", 0.0) + (time.perf_counter() - t0) * 1e3
             for i, (r, ch) in enumerate(zip(sampled, choices)):
                 forked = self._fork(r, logits[i:i + 1]) if r.forks and r.t_first is None else []
                 self._accept(r, ch)

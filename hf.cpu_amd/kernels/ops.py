@@ -55,6 +55,35 @@ class Pending:
     accumulate: bool
 
 
+class _NoSection:
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_SECTION = _NoSection()
+
+
+class _Section:
+    """Device time between entering and leaving, booked under a name."""
+
+    def __init__(self, ops, name):
+        self.ops, self.name = ops, name
+
+    def __enter__(self):
+        self.start = torch.cuda.Event(enable_timing=True)
+        self.start.record()
+        return self
+
+    def __exit__(self, *exc):
+        end = torch.cuda.Event(enable_timing=True)
+        end.record()
+        self.ops._sections.append((self.name, self.start, end))
+        return False
+
+
 class Ops:
     def __init__(self, act_dtype=torch.bfloat16, device="cuda:0"):
         if not torch.cuda.is_available():
@@ -70,8 +99,28 @@ class Ops:
         self.attn_workspace = torch.empty(WORKSPACE_BYTES, dtype=torch.uint8, device=self.device)
         self._pending = None
         self._splits_out = ctypes.c_int(0)
+        self._sections = None                # while timing: (name, start event, end event) of every section left
         self.force_plain_gemm = False        # tests set these to compare the matrix-core paths with the plain ones
         self.force_plain_attention = False
+
+    # ---- timing (the reference's hfc_prof_enable / hfc_prof_take, src/model.h:75-79) ----
+    def section(self, name):
+        """``with ops.section("qkv"): ...`` books the device time of the kernels enqueued inside
+        under ``name`` while timing is on; otherwise it costs nothing."""
+        return _NO_SECTION if self._sections is None else _Section(self, name)
+
+    def timing(self, on):
+        self._sections = [] if on else None
+
+    def take_times(self):
+        """Milliseconds per section name since the last call; waits for the device."""
+        out = {}
+        if self._sections:
+            torch.cuda.synchronize(self.device)
+            for name, start, end in self._sections:
+                out[name] = out.get(name, 0.0) + start.elapsed_time(end)
+            self._sections = []
+        return out
 
     # ---- plumbing ----------------------------------------------------------
     def _stream(self):

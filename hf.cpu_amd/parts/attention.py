@@ -73,8 +73,11 @@ class Attention(Part):
         width = self.QD + 2 * self.KD if write_cache else self.QD
         qkv = ops.scratch("qkv", (T, width), ops.act_dtype)
         # a product that split K is added up inside the next kernel (position.store, the next norm)
-        ops.gemm(h, self.w_qkv[:width], qkv, bias=None if self.b_qkv is None else self.b_qkv[:width], defer=True)
+        with ops.section("qkv"):
+            ops.gemm(h, self.w_qkv[:width], qkv, bias=None if self.b_qkv is None else self.b_qkv[:width], defer=True)
         self.position.store(ops, step, qkv, self.H, self.G if write_cache else 0, cache, write_cache)
         att = ops.scratch("att", (T, self.QD), ops.act_dtype)
-        ops.paged_attention(qkv, self.H, self.G, self.D, cache, step, self.window, self.scale, att)
-        ops.gemm(att, self.w_o, x, bias=self.b_o, accumulate=True, defer=True)
+        with ops.section("attn"):
+            ops.paged_attention(qkv, self.H, self.G, self.D, cache, step, self.window, self.scale, att)
+        with ops.section("wo"):
+            ops.gemm(att, self.w_o, x, bias=self.b_o, accumulate=True, defer=True)

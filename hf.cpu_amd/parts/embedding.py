@@ -21,7 +21,8 @@ class Embedding(Part):
         self.table = params[self.prefix + "weight"]
 
     def forward(self, ops, step, out_x):
-        ops.embed(self.table, step.tokens, out_x)
+        with ops.section("embed"):
+            ops.embed(self.table, step.tokens, out_x)
 
 
 @register_part("head", "linear")
@@ -47,4 +48,5 @@ class LinearHead(Part):
         self.weight = own if own is not None else params[self.tied_to]
 
     def forward(self, ops, h, out_logits):
-        ops.gemm(h, self.weight, out_logits)
+        with ops.section("head"):
+            ops.gemm(h, self.weight, out_logits)

@@ -45,9 +45,13 @@ class GatedMLP(Part):
         T = h.shape[0]
         act = ops.scratch("ffn_act", (T, self.F), ops.act_dtype)
         if self.fused:
-            ops.gemm(h, self.w_gate_up, act, swiglu=True)
+            with ops.section("gate_up"):           # the activation is the product's last step
+                ops.gemm(h, self.w_gate_up, act, swiglu=True)
         else:
             gu = ops.scratch("gate_up", (T, 2 * self.F), ops.act_dtype)
-            ops.gemm(h, self.w_gate_up, gu)
-            ops.swiglu(gu, act)
-        ops.gemm(act, self.w_down, x, accumulate=True, defer=True)
+            with ops.section("gate_up"):
+                ops.gemm(h, self.w_gate_up, gu)
+            with ops.section("silu"):
+                ops.swiglu(gu, act)
+        with ops.section("down"):
+            ops.gemm(act, self.w_down, x, accumulate=True, defer=True)

@@ -44,38 +44,38 @@ class SamplerParams:
         return self.temp <= 0
 
 
-def pick(ids, logits, params, rng):
-    """The draw among candidates already ordered (logit descending, id ascending) and cut
-    to top_k: steps 3 to 6 of the pipeline, in fp32 (src/sample.c:99-114)."""
+def pick_rows(ids, logits, params, rngs):
+    """The draw for several rows with the same parameters: ``ids`` and ``logits`` are [R, k]
+    candidates already ordered (logit descending, id ascending) and cut to top_k; ``rngs[r]``
+    is row r's generator. Steps 3 to 6 of the pipeline in fp32 (src/sample.c:99-114): every
+    sum is a running fp32 sum in candidate order, as in the reference's loops (``cumsum``
+    adds one element at a time in the array's precision)."""
     logits = np.asarray(logits, dtype=f32)
-    p = np.exp((logits - logits[0]) / f32(params.temp), dtype=f32)
-    total = f32(0)
-    for v in p:
-        total = f32(total + v)
-    p = (p / total).astype(f32)
-    kept = len(p)
+    ids = np.asarray(ids)
+    R, k = logits.shape
+    col = np.arange(k)[None, :]
+    p = np.exp((logits - logits[:, :1]) / f32(params.temp), dtype=f32)
+    p = (p / np.cumsum(p, axis=1, dtype=f32)[:, -1:]).astype(f32)
+    kept = np.full(R, k)
     if params.min_p > 0:
-        kept = 0
-        while kept < len(p) and p[kept] >= f32(params.min_p) * p[0]:
-            kept += 1
-        kept = max(kept, 1)
+        below = p < f32(params.min_p) * p[:, :1]                 # p does not increase along the order
+        kept = np.maximum(np.where(below.any(axis=1), below.argmax(axis=1), k), 1)
     if 0 < params.top_p < 1:
-        cum = f32(0)
-        for i in range(kept):
-            cum = f32(cum + p[i])
-            if cum >= f32(params.top_p):
-                kept = i + 1
-                break
-    total = f32(0)
-    for i in range(kept):
-        total = f32(total + p[i])
-    r = f32(rng.uniform() * total)
-    cum = f32(0)
-    for i in range(kept):
-        cum = f32(cum + p[i])
-        if r < cum:
-            return int(ids[i])
-    return int(ids[kept - 1])
+        live = col < kept[:, None]
+        reached = (np.cumsum(np.where(live, p, f32(0)), axis=1, dtype=f32) >= f32(params.top_p)) & live
+        kept = np.where(reached.any(axis=1), reached.argmax(axis=1) + 1, kept)
+    live = col < kept[:, None]
+    cum = np.cumsum(np.where(live, p, f32(0)), axis=1, dtype=f32)
+    u = np.array([rng.uniform() for rng in rngs], dtype=f32)     # 24 random bits: exact in fp32
+    r = u * cum[np.arange(R), kept - 1]
+    over = (r[:, None] < cum) & live
+    at = np.where(over.any(axis=1), over.argmax(axis=1), kept - 1)
+    return [int(t) for t in ids[np.arange(R), at]]
+
+
+def pick(ids, logits, params, rng):
+    """One row of ``pick_rows``."""
+    return pick_rows(np.asarray(ids)[None, :], np.asarray(logits, dtype=f32)[None, :], params, [rng])[0]
 
 
 def order_on_host(row, top_k):
@@ -114,16 +114,23 @@ class Sampler:
         arg = self.ops.argmax(logits).cpu().numpy() if greedy else None
         ids = vals = stats = None
         if need_k or any(n for _, _, n in wants):
-            ids, vals, stats = self.ops.topk(logits, need_k)
-            ids, vals, stats = ids.cpu().numpy(), vals.cpu().numpy(), stats.cpu().numpy()
+            ids, vals, stats = (t.cpu().numpy() for t in self.ops.topk(logits, need_k))
+        toks = [None] * R
+        groups = {}                               # rows drawn from the device's candidates, by parameters
         for i, (params, rng, n_lp) in enumerate(wants):
             if params.greedy:
-                tok = int(arg[i])
+                toks[i] = int(arg[i])
             elif 0 < params.top_k <= TOPK_KERNEL_MAX and params.top_k < logits.shape[1]:
-                tok = pick(ids[i, :params.top_k], vals[i, :params.top_k], params, rng)
+                groups.setdefault(params, []).append(i)
             else:
                 cand, cl = order_on_host(logits[i].cpu().numpy(), params.top_k)
-                tok = pick(cand, cl, params, rng)
+                toks[i] = pick(cand, cl, params, rng)
+        for params, rows in groups.items():
+            drawn = pick_rows(ids[rows, :params.top_k], vals[rows, :params.top_k], params, [wants[i][1] for i in rows])
+            for i, t in zip(rows, drawn):
+                toks[i] = t
+        for i, (params, rng, n_lp) in enumerate(wants):
+            tok = toks[i]
             ch = Choice(tok)
             if n_lp:
                 mx, lse = float(stats[i, 0]), float(stats[i, 1])

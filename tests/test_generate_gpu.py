@@ -171,6 +171,25 @@ def test_command_line_generate(gpu, models):
     assert rc == 1 and "code=EIO" in out
 
 
+def test_command_line_profile(gpu, models):
+    """``--profile`` adds the reference's two @profile events (docs/PROTOCOL.md:93): per stage the
+    milliseconds by part of the forward pass, plus sampling; the tokens are the same as without."""
+    base = ["--stdin-mode", "none", "--model", models["A"], "--dtype", "float32", "--prompt-ids",
+            " ".join(str(3 + i) for i in range(40)), "--temp", "0", "--max-tokens", "5", "--batch", "16"]
+    rc, out, err = run_cli(base + ["--profile"])
+    assert rc == 0, err
+    ev = events(out)
+    prof = {e[1]["stage"]: e[1] for e in ev if e[0] == "profile"}
+    parts = ("embed", "glue", "qkv", "attn", "wo", "gate_up", "silu", "down", "head", "sample")
+    for stage in ("prefill", "decode"):
+        assert all(k in prof[stage] for k in parts), prof[stage]
+        assert all(float(prof[stage][k]) > 0 for k in ("glue", "qkv", "attn", "wo", "gate_up", "down", "head", "sample"))
+    rc2, out2, _ = run_cli(base)
+    assert rc2 == 0 and [e[1]["id"] for e in events(out2) if e[0] == "token"] == \
+        [e[1]["id"] for e in ev if e[0] == "token"]
+    assert not any(e[0] == "profile" for e in events(out2))
+
+
 def test_trace_run_program(gpu, models, tmp_path):
     """bin/trace_run as a user calls it: steps on stdin, ``done <step>`` lines, <step>.f32 files;
     a mixed trace with few pages, in both dtypes, against the plain implementation."""

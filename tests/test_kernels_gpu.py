@@ -518,8 +518,23 @@ def test_argmax_and_topk(ops32):
         mx = logits[r].max()
         lse = np.log(np.sum(np.exp(logits[r].astype(np.float64) - mx)))
         assert float(stats[r, 0]) == mx and abs(float(stats[r, 1]) - lse) < 1e-5
-    big = dev(rng.standard_normal((2, 152064)).astype(np.float32))
+    big_np = rng.standard_normal((3, 152064)).astype(np.float32)
+    big_np[1, ::7] = 2.5                        # thousands of ties around the cut
+    big_np[2] = np.round(big_np[2] * 4) / 4     # few distinct values, negative ones among them
+    big_np[2, 5] = -np.inf
+    big = dev(big_np)
     assert ops32.argmax(big).cpu().tolist() == big.argmax(dim=1).cpu().tolist()
+    for k in (1, 2, 40, 333, 1024):             # the ordered best-k at other k, with ties across the cut
+        ids, vals, stats = ops32.topk(big, k)
+        for r in range(3):
+            order = np.lexsort((np.arange(152064), -big_np[r]))[:k]
+            assert np.array_equal(ids[r].cpu().numpy(), order), f"k={k} row {r}"
+            assert np.array_equal(vals[r].cpu().numpy(), big_np[r, order])
+    small = rng.standard_normal((2, 37)).astype(np.float32)     # fewer ids than threads; k = all of them
+    ids, vals, stats = ops32.topk(dev(small), 37)
+    assert ids.cpu().tolist() == [list(np.lexsort((np.arange(37), -r))) for r in small]
+    _, _, stats = ops32.topk(dev(small), 0)
+    assert abs(float(stats[1, 1]) - np.log(np.sum(np.exp(small[1].astype(np.float64) - small[1].max())))) < 1e-5
 
 
 def test_kernels_refuse_what_they_cannot_do(ops32):

@@ -31,6 +31,25 @@ def test_pick_follows_the_plain_pipeline(params):
         assert a == b
 
 
+@pytest.mark.parametrize("params", [(0.8, 40, 0.95, 0.05), (0.3, 5, 0.5, 0.0), (2.0, 64, 0.9, 0.2), (1.0, 7, 1.0, 0.0)])
+def test_rows_drawn_together_are_drawn_as_alone(params):
+    """Many rows of one step in one call: each row's token is what the plain sampler draws for
+    that row with that row's generator, whatever the other rows hold (a row that keeps one
+    candidate beside rows that keep all of them)."""
+    from hf_cpu_amd.sampling.sampler import pick_rows
+    rng = np.random.default_rng(1)
+    temp, top_k, top_p, min_p = params
+    logits = (rng.standard_normal((17, 500)) * 3).astype(np.float32)
+    logits[3, 100] = 40.0                           # one candidate takes all the mass
+    logits[4] = 0.25                                # all equal
+    logits[5, 7] = logits[5, 300] = logits[5].max() + 1
+    cands = [order_on_host(r, top_k) for r in logits]
+    got = pick_rows(np.stack([c[0] for c in cands]), np.stack([c[1] for c in cands]),
+                    SamplerParams(temp, top_k, top_p, min_p), [Rng(100 + i) for i in range(17)])
+    want = [plain.sample(logits[i], temp, top_k, top_p, min_p, plain.Rng(100 + i)) for i in range(17)]
+    assert got == want
+
+
 def test_option_layers_and_syntax(tmp_path):
     o = O.defaults()
     assert (o["temp"], o["top-k"], o["top-p"], o["min-p"], o["max-tokens"], o["batch"], o["ctx-max"], o["n"]) == \

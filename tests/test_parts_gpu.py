@@ -1,5 +1,6 @@
-"""Each part alone, a schedule that is more than a list of layers, and a toy mixer with
-state of its own that is registered, built and stepped without touching the package."""
+"""Each part alone, a schedule that is more than a list of layers, and toy parts that are
+registered, built and stepped without touching the package: a mixer with state of its own, a
+feed-forward with routing, another position encoding."""
 import dataclasses
 import json
 import math
@@ -254,4 +255,188 @@ def test_toy_mixer_with_state_and_a_schedule_that_repeats(gpu, tmp_path):
                                         max_seqs=3)
         got = helpers.run_trace_in_engine(engine, steps)
         helpers.compare(got, want, 2e-5, "toy model")
+        assert not engine.manager.held
+
+
+def routed_plan_factory():
+    """Registers a toy feed-forward with routing (top-1 of four experts, the router in fp32), a toy
+    position encoding (a learned vector per position added to queries and keys) and an
+    architecture that uses them in some layers and the package's parts in others. Nothing in
+    the package is edited for this; the toy parts use the package's products and cache store
+    and plain tensor arithmetic for the rest."""
+
+    @register_part("position", "toy_learned")
+    class ToyLearned(Part):
+        """q_t += table[pos_t], k_t += table[pos_t] for every head; values as they are."""
+
+        def __init__(self, head_dim, max_positions, prefix=""):
+            super().__init__(prefix)
+            self.head_dim, self.n = head_dim, max_positions
+
+        def param_specs(self):
+            return [ParamSpec(self.prefix + "pos.weight", (self.n, self.head_dim), "matrix", ("normal", 0.5))]
+
+        def bind(self, params, ops):
+            self.table = params[self.prefix + "pos.weight"]
+
+        def store(self, ops, step, qkv, n_heads, n_kv_heads, cache, write):
+            ops.settle()                                       # the product before may have left partial sums
+            add = self.table[step.positions.long()].to(qkv.dtype)
+            for h in range(n_heads + n_kv_heads):              # queries, then keys
+                qkv[:, h * self.head_dim:(h + 1) * self.head_dim] += add
+            if write:
+                ops.rope_store(qkv, step.positions, None, 0, n_heads, n_kv_heads, self.head_dim, cache,
+                               step.group(cache.group).slot_map)
+
+    @register_part("feed_forward", "toy_routed")
+    class ToyRouted(Part):
+        """x_t += p_e * down_e(relu(up_e(h_t))) with e = argmax of the router's logits and p_e its
+        softmax probability, both in fp32."""
+
+        def __init__(self, hidden_size, intermediate_size, n_experts, prefix=""):
+            super().__init__(prefix)
+            self.E, self.F, self.n = hidden_size, intermediate_size, n_experts
+
+        def param_specs(self):
+            out = [ParamSpec(self.prefix + "router.weight", (self.n, self.E), "matrix", ("normal", 0.5))]
+            for e in range(self.n):
+                out.append(ParamSpec(f"{self.prefix}experts.{e}.up.weight", (self.F, self.E), "matrix", ("normal", 0.3)))
+                out.append(ParamSpec(f"{self.prefix}experts.{e}.down.weight", (self.E, self.F), "matrix", ("normal", 0.3)))
+            return out
+
+        def bind(self, params, ops):
+            self.router = params[self.prefix + "router.weight"]
+            self.up = [params[f"{self.prefix}experts.{e}.up.weight"] for e in range(self.n)]
+            self.down = [params[f"{self.prefix}experts.{e}.down.weight"] for e in range(self.n)]
+
+        def forward(self, ops, step, h, x):
+            T = h.shape[0]
+            logits = torch.empty((T, self.n), dtype=torch.float32, device=h.device)
+            ops.gemm(h, self.router, logits)
+            ops.settle()
+            prob, expert = torch.softmax(logits, dim=1).max(dim=1)
+            for e in range(self.n):
+                rows = torch.nonzero(expert == e).flatten()
+                if rows.numel() == 0:
+                    continue
+                he = h.index_select(0, rows).contiguous()
+                mid = torch.empty((rows.numel(), self.F), dtype=h.dtype, device=h.device)
+                ops.gemm(he, self.up[e], mid)
+                out = torch.empty((rows.numel(), self.E), dtype=torch.float32, device=h.device)
+                ops.gemm(torch.relu(mid), self.down[e], out)
+                ops.settle()
+                x.index_add_(0, rows, out * prob[rows, None])
+
+    @dataclasses.dataclass(frozen=True)
+    class RoutedConfig:
+        architecture: str
+        vocab_size: int
+        hidden_size: int
+        n_experts: int
+        max_positions: int
+
+        @classmethod
+        def from_dict(cls, obj, origin="config.json"):
+            return cls(obj["architectures"][0], obj["vocab_size"], obj["hidden_size"], obj["n_experts"],
+                       obj["max_positions"])
+
+    def routed_plan(cfg):
+        E = cfg.hidden_size
+
+        def attention(l, position, window):
+            return PartSpec("attention", dict(hidden_size=E, n_heads=3, n_kv_heads=1, head_dim=16, qkv_bias=True,
+                                              window=window, prefix=f"layers.{l}.attn.", position=position))
+
+        def layer(l, mixer, ffn):
+            pre = f"layers.{l}."
+            return hf_cpu_amd.LayerPlan(
+                label=pre, block=PartSpec("prenorm", dict(hidden_size=E)),
+                norm1=PartSpec("rmsnorm", dict(size=E, eps=1e-6, prefix=pre + "norm1.")), mixer=mixer,
+                norm2=PartSpec("rmsnorm", dict(size=E, eps=1e-6, prefix=pre + "norm2.")), feed_forward=ffn)
+        learned = PartSpec("toy_learned", dict(head_dim=16, max_positions=cfg.max_positions, prefix="layers.0.attn."))
+        rotary = PartSpec("rotary", dict(head_dim=16, rot_dim=8, theta=100.0))
+        dense = PartSpec("gated_mlp", dict(hidden_size=E, intermediate_size=40, prefix="layers.0.mlp."))
+        routed = PartSpec("toy_routed", dict(hidden_size=E, intermediate_size=24, n_experts=cfg.n_experts,
+                                             prefix="layers.1.moe."))
+        return hf_cpu_amd.ModelPlan(
+            hidden_size=E, vocab_size=cfg.vocab_size,
+            embedding=PartSpec("lookup", dict(vocab_size=cfg.vocab_size, hidden_size=E, prefix="embed.")),
+            layers=(layer(0, attention(0, learned, 0), dense), layer(1, attention(1, rotary, 9), routed)),
+            schedule=(ScheduleEntry(0), ScheduleEntry(1)),
+            final_norm=PartSpec("rmsnorm", dict(size=E, eps=1e-6, prefix="final.")),
+            head=PartSpec("linear", dict(vocab_size=cfg.vocab_size, hidden_size=E, tied=False, prefix="head.")))
+    register_architecture("ToyRoutedForCausalLM", RoutedConfig, routed_plan)
+
+
+def routed_reference(w, toks, n_experts):
+    """The toy model over a whole sequence, written out directly (float64)."""
+    T = len(toks)
+    x = w["embed.weight"][toks]
+
+    def attn(x, l, window):
+        pre = f"layers.{l}.attn."
+        h = plain.rmsnorm(x, w[f"layers.{l}.norm1.weight"], 1e-6)
+        q = plain.linear(h, w[pre + "q_proj.weight"], w[pre + "q_proj.bias"]).reshape(T, 3, 16)
+        k = plain.linear(h, w[pre + "k_proj.weight"], w[pre + "k_proj.bias"]).reshape(T, 1, 16)
+        v = plain.linear(h, w[pre + "v_proj.weight"], w[pre + "v_proj.bias"]).reshape(T, 1, 16)
+        if l == 0:
+            q = q + w[pre + "pos.weight"][:T, None, :]
+            k = k + w[pre + "pos.weight"][:T, None, :]
+        else:
+            q, k = plain.rope(q, range(T), 8, 100.0), plain.rope(k, range(T), 8, 100.0)
+        return plain.linear(plain.attention(q, k, v, window).reshape(T, 48), w[pre + "o_proj.weight"])
+    x = x + attn(x, 0, 0)
+    x = x + plain.swiglu_mlp(plain.rmsnorm(x, w["layers.0.norm2.weight"], 1e-6), w["layers.0.mlp.gate_proj.weight"],
+                             w["layers.0.mlp.up_proj.weight"], w["layers.0.mlp.down_proj.weight"])
+    x = x + attn(x, 1, 9)
+    h = plain.rmsnorm(x, w["layers.1.norm2.weight"], 1e-6)
+    logits = h @ w["layers.1.moe.router.weight"].T
+    prob = plain.softmax(logits)
+    used = set()
+    for t in range(T):
+        e = int(np.argmax(logits[t]))
+        used.add(e)
+        mid = np.maximum(w[f"layers.1.moe.experts.{e}.up.weight"] @ h[t], 0.0)
+        x[t] = x[t] + prob[t, e] * (w[f"layers.1.moe.experts.{e}.down.weight"] @ mid)
+    out = plain.linear(plain.rmsnorm(x, w["final.weight"], 1e-6), w["head.weight"])
+    return out, used
+
+
+def test_toy_routed_feed_forward_and_toy_position_encoding(gpu, tmp_path):
+    """Another feed-forward (with routing) and another position encoding, registered from
+    here, in a model whose two layers differ in position encoding, window and feed-forward:
+    whole, in portions and mixed with few pages, against the model written out directly."""
+    routed_plan_factory()
+    cfg = {"architectures": ["ToyRoutedForCausalLM"], "vocab_size": 70, "hidden_size": 20, "n_experts": 4,
+           "max_positions": 64}
+    d = str(tmp_path / "routed")
+    os.makedirs(d)
+    with open(os.path.join(d, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    model = hf_cpu_amd.Model.from_config(hf_cpu_amd.config_from_dict(cfg))
+    needs = model.cache_needs()
+    assert [type(n).__name__ for n in needs] == ["PagedKV", "PagedKV"] and (needs[0].window, needs[1].window) == (0, 9)
+    names = {s.name for s in model.param_specs()}
+    assert "layers.1.moe.experts.3.down.weight" in names and "layers.0.attn.pos.weight" in names
+    rng = np.random.default_rng(5)
+    w = {}
+    for s in model.param_specs():
+        if s.optional:
+            continue
+        std = {"embed.weight": 0.5, "layers.1.moe.router.weight": 1.0}.get(s.name, 0.3 if s.kind == "matrix" else 0.1)
+        w[s.name] = ((1.0 if s.kind == "vector" and s.name.endswith("norm1.weight") or s.name.endswith("norm2.weight")
+                      or s.name == "final.weight" else 0.0) + rng.standard_normal(s.shape) * std).astype(np.float32)
+    helpers.write_safetensors(os.path.join(d, "model.safetensors"), w)
+    reqs = {f"r{i}": [int(t) for t in rng.integers(0, 70, n)] for i, n in enumerate([6, 25, 44, 33])}
+    w64 = {k: v.astype(np.float64) for k, v in w.items()}
+    want, used = {}, set()
+    for r, t in reqs.items():
+        want[r], u = routed_reference(w64, t, 4)
+        used |= u
+    assert len(used) >= 3, "the inputs were meant to reach most experts"
+    for steps in (helpers.trace_whole(reqs), helpers.trace_portions(reqs), helpers.trace_mixed(reqs, seed=4, max_live=3)):
+        engine = hf_cpu_amd.load_engine(d, dtype="float32", page_tokens=4, max_tokens=helpers.max_live_tokens(steps),
+                                        max_seqs=3)
+        got = helpers.run_trace_in_engine(engine, steps)
+        helpers.compare(got, want, 2e-5, "toy routed model")
         assert not engine.manager.held

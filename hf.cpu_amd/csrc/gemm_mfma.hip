@@ -262,7 +262,8 @@ struct DmaOut {
 template <int BM, int BN, int BK, int WM, int WN, int STAGES, int MODE>
 __global__ __launch_bounds__(WM* WN* WAVE) void gemm_dma_kernel(
     const uint16_t* __restrict__ A, int lda, const uint16_t* __restrict__ W, int ldw,
-    const float* __restrict__ bias, void* __restrict__ out, int ldo, int M, int N, int K, int tiles_m, int tiles_n) {
+    const float* __restrict__ bias, void* __restrict__ out, int ldo, int M, int N, int K, int k_per_split,
+    int tiles_m, int tiles_n) {
     using C = DmaCfg<BM, BN, BK, WM, WN>;
     static_assert(STAGES >= 3, "one tile in use, the next one landed, one arriving");
     extern __shared__ __attribute__((aligned(1024))) uint16_t smem[];
@@ -293,8 +294,10 @@ __global__ __launch_bounds__(WM* WN* WAVE) void gemm_dma_kernel(
     // Request i of this wave fills rows (i * NW + wave) * ROWS_PER_LOAD .. of a stage; this lane
     // supplies the piece stored at lane % PIECES of row lane / PIECES of them. Its address is a
     // scalar base (the block's first row of A or W, advancing with K) plus a byte offset per lane.
-    const uint16_t* a_base = A + (size_t)m0 * lda;
-    const uint16_t* w_base = W + (size_t)n0 * ldw;
+    const int kbeg = blockIdx.z * k_per_split;               // K may be split over blockIdx.z (narrow outputs)
+    const int kend = kbeg + k_per_split < K ? kbeg + k_per_split : K;
+    const uint16_t* a_base = A + (size_t)m0 * lda + kbeg;
+    const uint16_t* w_base = W + (size_t)n0 * ldw + kbeg;
     uint32_t src[C::LOADS];
 #pragma unroll
     for (int i = 0; i < C::LOADS; i++) {
@@ -337,7 +340,7 @@ __global__ __launch_bounds__(WM* WN* WAVE) void gemm_dma_kernel(
     // few matrix instructions. The fragments of a 16-column step are read one step ahead, also
     // across the barrier (tile t + 1's first ones during tile t's last step), so that the matrix
     // cores have work the moment a wave leaves the barrier.
-    const int nk = K / BK;
+    const int nk = (kend - kbeg) / BK;
 #pragma unroll
     for (int p = 0; p < STAGES - 1; p++)
         if (p < nk) {
@@ -466,7 +469,7 @@ static int launch_cfg(const GemmArgs& g, void* out, int splits, int k_per_split)
 }
 
 template <int BM, int BN, int BK, int WM, int WN, int STAGES, int MODE>
-static int launch_dma_cfg(const GemmArgs& g) {
+static int launch_dma_cfg(const GemmArgs& g, void* out, int splits, int k_per_split) {
     using C = DmaCfg<BM, BN, BK, WM, WN>;
     constexpr int SMEM = STAGES * C::STAGE_BYTES > DmaOut<BN, MODE>::bytes(BM) ? STAGES * C::STAGE_BYTES : DmaOut<BN, MODE>::bytes(BM);
     auto kernel = gemm_dma_kernel<BM, BN, BK, WM, WN, STAGES, MODE>;
@@ -480,19 +483,21 @@ static int launch_dma_cfg(const GemmArgs& g) {
         configured = true;
     }
     const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
-    kernel<<<dim3(tiles_m * tiles_n), C::NT, SMEM, g.stream>>>((const uint16_t*)g.a, g.lda, (const uint16_t*)g.w, g.ldw,
-                                                              g.bias, g.out, g.ldo, g.M, g.N, g.K, tiles_m, tiles_n);
+    kernel<<<dim3(tiles_m * tiles_n, 1, splits), C::NT, SMEM, g.stream>>>(
+        (const uint16_t*)g.a, g.lda, (const uint16_t*)g.w, g.ldw, g.bias, out, g.ldo, g.M, g.N, g.K, k_per_split, tiles_m,
+        tiles_n);
     HFA_LAUNCH_CHECK("gemm_dma");
     return 0;
 }
 
 template <int BM, int BN, int BK, int WM, int WN, int STAGES>
-static int launch_dma(const GemmArgs& g, int mode) {
+static int launch_dma(const GemmArgs& g, int mode, void* out, int splits, int k_per_split) {
     switch (mode) {
-        case OUT_BF16: return launch_dma_cfg<BM, BN, BK, WM, WN, STAGES, OUT_BF16>(g);
-        case OUT_F32: return launch_dma_cfg<BM, BN, BK, WM, WN, STAGES, OUT_F32>(g);
-        case OUT_ACC: return launch_dma_cfg<BM, BN, BK, WM, WN, STAGES, OUT_ACC>(g);
-        default: return launch_dma_cfg<BM, BN, BK, WM, WN, STAGES, OUT_SWIGLU>(g);
+        case OUT_BF16: return launch_dma_cfg<BM, BN, BK, WM, WN, STAGES, OUT_BF16>(g, out, splits, k_per_split);
+        case OUT_F32: return launch_dma_cfg<BM, BN, BK, WM, WN, STAGES, OUT_F32>(g, out, splits, k_per_split);
+        case OUT_ACC: return launch_dma_cfg<BM, BN, BK, WM, WN, STAGES, OUT_ACC>(g, out, splits, k_per_split);
+        case OUT_PARTIAL: return launch_dma_cfg<BM, BN, BK, WM, WN, STAGES, OUT_PARTIAL>(g, out, splits, k_per_split);
+        default: return launch_dma_cfg<BM, BN, BK, WM, WN, STAGES, OUT_SWIGLU>(g, out, splits, k_per_split);
     }
 }
 
@@ -582,10 +587,23 @@ int gemm_mfma_launch(const GemmArgs& g, void* workspace, size_t workspace_bytes,
                         (size_t)rows256 * 100 <= (size_t)rows128 * 128 &&
                         (g.out_dtype != HFA_BF16 || (g.ldo % 8 == 0 && g.N % 16 == 0 && ((uintptr_t)g.out & 15) == 0));
     const int tiles256 = (rows256 / 256) * ((g.N + 255) / 256);
+    // A narrow output has too few 256 x 256 tiles for the CUs: K is cut in two and the halves' sums
+    // go to the workspace, if it holds them; otherwise tiles of 256 x 128.
+    const bool halves = dma_ok && tiles256 < 128 && 2 * tiles256 >= 128 && g.K % 128 == 0 && g.K >= 2048 &&
+                        mode != OUT_SWIGLU && workspace != nullptr &&
+                        2 * (size_t)g.M * g.N * sizeof(float) <= workspace_bytes;
     if (dma_ok && tiles256 >= 128)
-        rc = launch_dma<256, 256, 32, 2, 4, 4>(g, kmode);
-    else if (dma_ok && 2 * tiles256 >= 128)
-        rc = launch_dma<256, 128, 32, 4, 2, 6>(g, kmode);
+        rc = launch_dma<256, 256, 32, 2, 4, 4>(g, kmode, kout, 1, g.K);
+    else if (halves) {
+        rc = launch_dma<256, 256, 32, 2, 4, 4>(g, OUT_PARTIAL, workspace, 2, g.K / 2);
+        if (rc) return rc;
+        if (defer && pending_splits) {
+            *pending_splits = 2;
+            return 0;
+        }
+        return gemm_finish_launch((const float*)workspace, 2, g.bias, g.out, mode, g.ldo, g.M, g.N, g.stream);
+    } else if (dma_ok && 2 * tiles256 >= 128)
+        rc = launch_dma<256, 128, 32, 4, 2, 6>(g, kmode, kout, 1, g.K);
     else if (BM == 128)
         rc = launch_mode<128, 128, 64, 2, 2>(g, kmode, kout, splits, k_per_split);
     else if (BM == 64)

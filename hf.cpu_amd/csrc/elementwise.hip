@@ -202,6 +202,86 @@ __global__ __launch_bounds__(128) void rope_store_kernel(
     (void)rest;
 }
 
+// The same for prompt portions in bf16: a block takes 8 consecutive tokens. The angles of a token
+// are computed once (not once per head), queries and keys move 16 bytes per lane, and the
+// values of the 8 tokens go through LDS so that, where the tokens' cache rows are 8 consecutive
+// rows of one page, every value column is written with one 16-byte store instead of eight
+// 2-byte stores 2 * page_tokens bytes apart.
+#define ROPE_TOKENS 8
+__global__ __launch_bounds__(256) void rope_store_rows_kernel(
+    uint16_t* __restrict__ qkv, int ld, const int* __restrict__ positions, const float* __restrict__ inv_freq,
+    int rot_dim, int H, int G, int D, uint16_t* __restrict__ k_cache, uint16_t* __restrict__ v_cache,
+    const int* __restrict__ slot_map, int page_tokens, int n_tokens) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char rope_lds[];
+    const int half = rot_dim / 2, KD = G * D;
+    float* cs = reinterpret_cast<float*>(rope_lds);                          // [ROPE_TOKENS][half] cosines, then sines
+    float* sn = cs + ROPE_TOKENS * half;
+    uint16_t* vt = reinterpret_cast<uint16_t*>(sn + ROPE_TOKENS * half);     // [ROPE_TOKENS][KD] values
+    int* slots = reinterpret_cast<int*>(vt + ROPE_TOKENS * KD);              // [ROPE_TOKENS]
+    const int t0 = blockIdx.x * ROPE_TOKENS;
+    const int nt = n_tokens - t0 < ROPE_TOKENS ? n_tokens - t0 : ROPE_TOKENS;
+    const int tid = threadIdx.x;
+    const bool store = G > 0 && slot_map != nullptr;
+    for (int i = tid; i < nt * half; i += blockDim.x) {
+        const int t = i / half, j = i % half;
+        sincosf((float)positions[t0 + t] * inv_freq[j], &sn[i], &cs[i]);
+    }
+    if (tid < ROPE_TOKENS) slots[tid] = (store && tid < nt) ? slot_map[t0 + tid] : -1;
+    if (store)                                                               // values: rows into LDS
+        for (int i = tid; i < nt * (KD / 8); i += blockDim.x) {
+            const int t = i / (KD / 8), c = (i % (KD / 8)) * 8;
+            *reinterpret_cast<uint4*>(vt + t * KD + c) =
+                *reinterpret_cast<const uint4*>(qkv + (size_t)(t0 + t) * ld + (H + G) * D + c);
+        }
+    __syncthreads();
+    // queries and keys: 8 pairs (i, i + half) per item
+    const int heads = H + G, per_head = half / 8;
+    for (int i = tid; i < nt * heads * per_head; i += blockDim.x) {
+        const int t = i / (heads * per_head), r = i % (heads * per_head), h = r / per_head, j = (r % per_head) * 8;
+        uint16_t* src = qkv + (size_t)(t0 + t) * ld + h * D;
+        uint16_t* dst = src;
+        if (h >= H && store) dst = k_cache + (size_t)slots[t] * KD + (h - H) * D;
+        uint4 a = *reinterpret_cast<const uint4*>(src + j), b = *reinterpret_cast<const uint4*>(src + j + half);
+        uint16_t* pa = reinterpret_cast<uint16_t*>(&a);
+        uint16_t* pb = reinterpret_cast<uint16_t*>(&b);
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            const float x0 = __uint_as_float((uint32_t)pa[u] << 16), x1 = __uint_as_float((uint32_t)pb[u] << 16);
+            const float c = cs[t * half + j + u], s1 = sn[t * half + j + u];
+            pa[u] = bf16_bits(x0 * c - x1 * s1);
+            pb[u] = bf16_bits(x0 * s1 + x1 * c);
+        }
+        *reinterpret_cast<uint4*>(dst + j) = a;
+        *reinterpret_cast<uint4*>(dst + j + half) = b;
+    }
+    if (!store) return;
+    // dimensions of the keys that are not rotated pass through to the cache
+    const int rest = (D - rot_dim) / 8;
+    for (int i = tid; i < nt * G * rest; i += blockDim.x) {
+        const int t = i / (G * rest), r = i % (G * rest), g = r / rest, j = rot_dim + (r % rest) * 8;
+        *reinterpret_cast<uint4*>(k_cache + (size_t)slots[t] * KD + g * D + j) =
+            *reinterpret_cast<const uint4*>(qkv + (size_t)(t0 + t) * ld + (H + g) * D + j);
+    }
+    // values, transposed inside their page
+    bool run = nt == ROPE_TOKENS && page_tokens % 8 == 0 && slots[0] % 8 == 0;
+    for (int t = 1; run && t < ROPE_TOKENS; t++) run = slots[t] == slots[0] + t;
+    if (run) {
+        uint16_t* page = v_cache + (size_t)(slots[0] / page_tokens) * page_tokens * KD + slots[0] % page_tokens;
+        for (int c = tid; c < KD; c += blockDim.x) {
+            uint4 out;
+            uint16_t* po = reinterpret_cast<uint16_t*>(&out);
+#pragma unroll
+            for (int t = 0; t < ROPE_TOKENS; t++) po[t] = vt[t * KD + c];
+            *reinterpret_cast<uint4*>(page + (size_t)c * page_tokens) = out;
+        }
+    } else {
+        for (int i = tid; i < nt * KD; i += blockDim.x) {
+            const int t = i / KD, c = i % KD, slot = slots[t];
+            v_cache[(size_t)(slot / page_tokens) * page_tokens * KD + (size_t)c * page_tokens + slot % page_tokens] = vt[i];
+        }
+    }
+}
+
 extern "C" int hfa_rope_store(void* qkv, int dtype, int ld, const int* positions, const float* inv_freq, int rot_dim,
                               int n_heads, int n_kv_heads, int head_dim, void* k_cache, void* v_cache,
                               const int* slot_map, int page_tokens, int n_tokens, const float* partial, int splits,
@@ -216,6 +296,17 @@ extern "C" int hfa_rope_store(void* qkv, int dtype, int ld, const int* positions
     HFA_REQUIRE(dtype == HFA_F32 || dtype == HFA_BF16, "rope_store: unknown dtype %d", dtype);
     HFA_REQUIRE(splits >= 0 && (splits == 0 || partial), "rope_store: partial sums announced but not given");
     HFA_REQUIRE(n_heads + 2 * n_kv_heads <= 65535, "rope_store: too many heads for the grid");
+    const int kd = n_kv_heads * head_dim;
+    const size_t rows_lds = (size_t)ROPE_TOKENS * rot_dim * sizeof(float) + (size_t)ROPE_TOKENS * kd * 2 + ROPE_TOKENS * sizeof(int);
+    if (dtype == HFA_BF16 && splits == 0 && n_tokens >= 4 * ROPE_TOKENS && rot_dim > 0 && rot_dim % 16 == 0 &&
+        head_dim % 8 == 0 && ld % 8 == 0 && ((uintptr_t)qkv & 15) == 0 && ((uintptr_t)k_cache & 15) == 0 &&
+        ((uintptr_t)v_cache & 15) == 0 && rows_lds <= 48 * 1024) {
+        rope_store_rows_kernel<<<(n_tokens + ROPE_TOKENS - 1) / ROPE_TOKENS, 256, rows_lds, stream>>>(
+            (uint16_t*)qkv, ld, positions, inv_freq, rot_dim, n_heads, n_kv_heads, head_dim, (uint16_t*)k_cache,
+            (uint16_t*)v_cache, slot_map, page_tokens, n_tokens);
+        HFA_LAUNCH_CHECK("rope_store");
+        return 0;
+    }
     const dim3 grid(n_tokens, n_heads + 2 * n_kv_heads);
     const int threads = head_dim >= 128 ? 128 : 64;
     if (dtype == HFA_F32)

@@ -465,6 +465,58 @@ def test_rope_store(ops32, dtype, H, G, D, rot):
     assert float(cache.k[unused].abs().max()) == 0.0
 
 
+@pytest.mark.parametrize("H,G,D,rot,page,T", [(4, 2, 16, 16, 8, 67), (28, 4, 128, 128, 16, 200), (5, 5, 48, 32, 8, 41),
+                                              (3, 1, 64, 64, 4, 40), (2, 2, 32, 32, 16, 64)])
+def test_rope_store_for_prompt_portions(ops16, H, G, D, rot, page, T):
+    """bf16 with many tokens takes a kernel of its own (8 tokens per block, 16 bytes per lane,
+    values through LDS): the result must be, bit for bit, what the kernel for few tokens gives:
+    token runs that fill cache rows in order (aligned to 8 and not), scattered rows, a last
+    block of fewer than 8 tokens, a part of the head that is not rotated, without a cache."""
+    rng = np.random.default_rng(T + D)
+    dtype = torch.bfloat16
+    qkv = rng.standard_normal((T, (H + 2 * G) * D)).astype(np.float32)
+    positions = [int(p) for p in np.concatenate([np.arange(100, 100 + T - 9), rng.integers(0, 30000, 9)])]
+    n_rows = (T + 40) // page * page + page
+    rows = list(range(16, 16 + 24)) + list(range(43, 43 + 11))          # a run aligned to 8, then one that is not
+    rest = [r for r in rng.permutation(n_rows) if r not in rows]
+    slot_map = (rows + [int(r) for r in rest])[:T]
+    i = np.arange(rot // 2, dtype=np.float64)
+    inv_freq = dev((1e4 ** (-2.0 * i / rot)).astype(np.float32))
+
+    def run(tokens):
+        t_qkv = dev(qkv[tokens], dtype)
+        cache = FakeCache(group=0, k=torch.zeros((n_rows, G * D), dtype=dtype, device="cuda"),
+                          v=torch.zeros((n_rows, G * D), dtype=dtype, device="cuda"), page_tokens=page)
+        ops16.rope_store(t_qkv, ints([positions[t] for t in tokens]), inv_freq, rot, H, G, D, cache,
+                         ints([slot_map[t] for t in tokens]))
+        return t_qkv, cache
+    all_q, all_c = run(list(range(T)))
+    few_q = torch.empty_like(all_q)
+    few_c = FakeCache(k=torch.zeros_like(all_c.k), v=torch.zeros_like(all_c.v))
+    for a in range(0, T, 7):                                            # 7 tokens at a time: the other kernel
+        toks = list(range(a, min(a + 7, T)))
+        q, c = run(toks)
+        few_q[toks] = q
+        for t in toks:
+            r = slot_map[t]
+            few_c.k[r] = c.k[r]
+        pages = sorted({slot_map[t] // page for t in toks})
+        for pg in pages:
+            blk = slice(pg * page, (pg + 1) * page)
+            few_c.v[blk] = torch.where(c.v[blk] != 0, c.v[blk], few_c.v[blk])
+    assert torch.equal(all_q, few_q) and torch.equal(all_c.k, few_c.k) and torch.equal(all_c.v, few_c.v)
+    src = rounded(qkv, dtype)                                           # and both are right
+    k_want = plain.rope(src[:, H * D:(H + G) * D].reshape(T, G, D), positions, rot, 1e4).reshape(T, G * D)
+    assert np.max(np.abs(all_c.k.float().cpu().numpy()[slot_map] - k_want)) <= 0.03
+    vc = from_value_layout(all_c.v.float().cpu().numpy(), page)
+    assert np.array_equal(vc[slot_map], src[:, (H + G) * D:].astype(np.float32))
+    no_cache = dev(qkv, dtype)                                          # without a cache: keys are rotated in place
+    ops16.rope_store(no_cache, ints(positions), inv_freq, rot, H, G, D, FakeCache(group=0, k=None, v=None, page_tokens=page), None)
+    assert torch.equal(no_cache[:, :H * D], all_q[:, :H * D])
+    assert np.max(np.abs(no_cache[:, H * D:(H + G) * D].float().cpu().numpy() - k_want)) <= 0.03
+    assert torch.equal(no_cache[:, (H + G) * D:], dev(qkv, dtype)[:, (H + G) * D:])
+
+
 def test_rope_relative_position(ops32):
     """<rope(q, p + s), rope(k, p' + s)> does not depend on the shift s: only distances count.
     A wrong sign or a wrong pairing breaks this."""

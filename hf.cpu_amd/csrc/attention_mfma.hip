@@ -49,9 +49,10 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
     const uint16_t* __restrict__ q, int ldq, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc, int kvw,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ token_slot,
     const int* __restrict__ positions, const int* __restrict__ q_start, int n_seqs, uint16_t* __restrict__ out,
-    int ldo, float* __restrict__ partial, int H, int P, int window, float scale_log2e, int tpt, int cpt,
+    int ldo, float* __restrict__ partial, int H, int psh, int window, float scale_log2e, int tpt, int cpt,
     int chunk_keys, int n_chunks, int one_tile_each) {
     constexpr int D = NDB * 32, KS = D / 16;
+    const int P = 1 << psh;                                // tokens per page, a power of two
     const int lane = threadIdx.x, col = lane & 31, half = lane >> 5;
     const int g = blockIdx.y, chunk = blockIdx.z;
 
@@ -115,13 +116,13 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
     // PG_MAX pages are fetched at once (pw0 = first page of the window), outside the steady loop.
     __shared__ int pg_s[PG_MAX];
     int pw0 = 0;
-    auto page_of = [&](int key) { return pg_s[key / P - pw0]; };
+    auto page_of = [&](int key) { return pg_s[(key >> psh) - pw0]; };
 
     auto load_k = [&](int key0, Frag (&kf)[KS]) {
         int key = key0 + col;                              // this lane's row of the key block
         key = key < hi ? key : hi;                         // rows past the end repeat the last key; they are masked
         const int page = page_of(key);
-        const unsigned off = (unsigned)(page * P + key % P) * (unsigned)kvw + (unsigned)(g * D + half * 8);
+        const unsigned off = __umul24((unsigned)((page << psh) + (key & (P - 1))), (unsigned)kvw) + (unsigned)(g * D + half * 8);
 #pragma unroll
         for (int ks = 0; ks < KS; ks++) kf[ks].u = *reinterpret_cast<const uint4*>(kc + (off + (unsigned)(ks * 16)));
     };
@@ -137,10 +138,10 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
                 ka = ka < (hi & ~3) ? ka : (hi & ~3);       // runs past the end are masked; read a valid one
                 const int page = page_of(ka);
                 // element offsets fit 32 bits (checked on the host), so one base serves every load
-                const unsigned off = (unsigned)page * (unsigned)(P * kvw) + (unsigned)((g * D + col) * P + ka % P);
+                const unsigned off = __umul24((unsigned)(page << psh), (unsigned)kvw) + (unsigned)(((g * D + col) << psh) + (ka & (P - 1)));
 #pragma unroll
                 for (int db = 0; db < NDB; db++)
-                    vf[db][kk].h[run] = *reinterpret_cast<const uint2*>(vc + (off + (unsigned)(db * 32 * P)));
+                    vf[db][kk].h[run] = *reinterpret_cast<const uint2*>(vc + (off + (unsigned)((db * 32) << psh)));
             }
         }
     };
@@ -214,14 +215,14 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
     const int first = (k_begin / KB) * KB;
     const int nb = first <= k_end ? (k_end - first) / KB + 1 : 0;
     const int k_top = first + nb * KB - 1 < hi ? first + nb * KB - 1 : hi;       // last key any load touches
-    const int win_blocks = PG_MAX * P / KB;                                       // key blocks a window of pages covers
+    const int win_blocks = (PG_MAX << psh) / KB;                                  // key blocks a window of pages covers
     for (int wb = 0; wb < nb; wb += win_blocks) {
         const int we = wb + win_blocks < nb ? wb + win_blocks : nb;               // blocks [wb, we)
         __syncthreads();                                                          // the old window is no longer read
-        pw0 = (first + wb * KB) / P;
+        pw0 = (first + wb * KB) >> psh;
         {
             const int top = first + we * KB - 1 < k_top ? first + we * KB - 1 : k_top;
-            const int n_pg = top / P - pw0 + 1;
+            const int n_pg = (top >> psh) - pw0 + 1;
             for (int i = lane; i < n_pg; i += WAVE) pg_s[i] = bt[pw0 + i];
         }
         __syncthreads();
@@ -292,8 +293,9 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
     const uint16_t* __restrict__ q, int ldq, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc, int kvw,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ token_slot,
     const int* __restrict__ positions, const int* __restrict__ q_start, int n_seqs, uint16_t* __restrict__ out,
-    int ldo, int P, int window, float scale_log2e, int tpt, int cpt) {
+    int ldo, int psh, int window, float scale_log2e, int tpt, int cpt) {
     constexpr int D = NDB * 32, KS = D / 16, KROW = D + 8;
+    const int P = 1 << psh;                                // tokens per page, a power of two
     __shared__ __attribute__((aligned(16))) uint16_t k_s[2][KB * KROW];
     __shared__ __attribute__((aligned(16))) uint16_t v_s[2][D * PVS];
     const int tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
@@ -347,7 +349,7 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
     // page ids in LDS, a window of PG_MAX pages at a time (see the kernel above)
     __shared__ int pg_s[PG_MAX];
     int pw0 = 0;
-    auto page_of = [&](int key) { return pg_s[key / P - pw0]; };
+    auto page_of = [&](int key) { return pg_s[(key >> psh) - pw0]; };
 
     // global -> registers -> LDS. Keys: 32 rows of D elements = 4 D chunks of 16 bytes.
     // Values: D rows of 32 keys = 4 D chunks of 8 keys. Each thread takes up to NCH of both.
@@ -363,14 +365,14 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
                 int key = key0 + c / (D / 8);
                 key = key < hi ? key : hi;
                 const int page = page_of(key);
-                const unsigned off = (unsigned)(page * P + key % P) * (unsigned)kvw + (unsigned)(g * D + (c % (D / 8)) * 8);
+                const unsigned off = __umul24((unsigned)((page << psh) + (key & (P - 1))), (unsigned)kvw) + (unsigned)(g * D + (c % (D / 8)) * 8);
                 rk[i] = *reinterpret_cast<const u32x4*>(kc + off);
             }
             {   // value chunk: dimension c / 4, keys key0 + 8 (c % 4) .. + 7
                 int ka = key0 + 8 * (c % 4);
                 ka = ka < (hi & ~7) ? ka : (hi & ~7);
                 const int page = page_of(ka);
-                const unsigned off = (unsigned)page * (unsigned)(P * kvw) + (unsigned)((g * D + c / 4) * P + ka % P);
+                const unsigned off = __umul24((unsigned)(page << psh), (unsigned)kvw) + (unsigned)(((g * D + c / 4) << psh) + (ka & (P - 1)));
                 const uint4 v = *reinterpret_cast<const uint4*>(vc + off);
                 rv[i][0] = make_uint2(v.x, v.y);
                 rv[i][1] = make_uint2(v.z, v.w);
@@ -391,14 +393,14 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
 
     const int first = (k_begin / KB) * KB;
     const int nb = (hi - first) / KB + 1;
-    const int win_blocks = PG_MAX * P / KB;
+    const int win_blocks = (PG_MAX << psh) / KB;
     for (int wb = 0; wb < nb; wb += win_blocks) {
         const int we = wb + win_blocks < nb ? wb + win_blocks : nb;               // blocks [wb, we)
         __syncthreads();                                                          // old window and stages are no longer read
-        pw0 = (first + wb * KB) / P;
+        pw0 = (first + wb * KB) >> psh;
         {
             const int top = first + we * KB - 1 < hi ? first + we * KB - 1 : hi;
-            const int n_pg = top / P - pw0 + 1;
+            const int n_pg = (top >> psh) - pw0 + 1;
             for (int i = tid; i < n_pg; i += 4 * WAVE) pg_s[i] = bt[pw0 + i];
         }
         __syncthreads();
@@ -424,23 +426,41 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
                     qf.u = q_s[wave][ks * WAVE + lane];
                     st = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf.v, qf.v, st, 0, 0, 0);
                 }
-                float mx = NEG_BIG;
+                // Most blocks lie wholly inside what every column of the wave may see (unused columns
+                // aside, whose results are dropped): no key of them needs the visibility test.
+                const bool inside = __all(!col_ok || (key0 >= vlo && key0 + KB - 1 <= vhi)) != 0;
+                float mx = NEG_BIG, mn, corr, psum = 0.f;
+                if (inside) {
 #pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const int kr = key0 + 8 * (r / 4) + 4 * half + (r % 4);
-                    const bool vis = kr >= vlo && kr <= vhi;
-                    st[r] = vis ? st[r] * scale_log2e : NEG_BIG;
-                    mx = fmaxf(mx, st[r]);
-                }
-                mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
-                const float mn = fmaxf(m, mx);
-                const float corr = fast_exp2(m - mn);
-                float psum = 0.f;
+                    for (int r = 0; r < 16; r++) {
+                        st[r] *= scale_log2e;
+                        mx = fmaxf(mx, st[r]);
+                    }
+                    mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+                    mn = fmaxf(m, mx);
+                    corr = fast_exp2(m - mn);
 #pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const float p = st[r] > 0.5f * NEG_BIG ? fast_exp2(st[r] - mn) : 0.f;
-                    st[r] = p;
-                    psum += p;
+                    for (int r = 0; r < 16; r++) {
+                        st[r] = fast_exp2(st[r] - mn);
+                        psum += st[r];
+                    }
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        const int kr = key0 + 8 * (r / 4) + 4 * half + (r % 4);
+                        const bool vis = kr >= vlo && kr <= vhi;
+                        st[r] = vis ? st[r] * scale_log2e : NEG_BIG;
+                        mx = fmaxf(mx, st[r]);
+                    }
+                    mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+                    mn = fmaxf(m, mx);
+                    corr = fast_exp2(m - mn);
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        const float p = st[r] > 0.5f * NEG_BIG ? fast_exp2(st[r] - mn) : 0.f;
+                        st[r] = p;
+                        psum += p;
+                    }
                 }
                 psum += __shfl_xor(psum, 32, WAVE);
                 l = l * corr + psum;
@@ -517,9 +537,16 @@ __global__ __launch_bounds__(WAVE) void attn_merge_kernel(const float* __restric
     }
 }
 
+// log2 of the page size, or -1 if it is not a power of two (the kernels shift and mask by it).
+static int page_shift(int page_tokens) {
+    int s = 0;
+    while ((1 << s) < page_tokens) s++;
+    return (1 << s) == page_tokens ? s : -1;
+}
+
 bool attn_mfma_supports(const AttnArgs& a) {
     const int group = a.n_heads / a.n_kv_heads;
-    return a.head_dim % 32 == 0 && a.head_dim <= 128 && a.page_tokens % 4 == 0 && group <= 32 && a.q_start != nullptr &&
+    return a.head_dim % 32 == 0 && a.head_dim <= 128 && a.page_tokens >= 4 && page_shift(a.page_tokens) >= 0 && group <= 32 && a.q_start != nullptr &&
            a.ldq % 8 == 0 && a.ldo % 4 == 0 && a.kv_width % 8 == 0 && a.kv_width * a.page_tokens < (1 << 20) &&
            ((uintptr_t)a.q & 15) == 0 &&
            ((uintptr_t)a.out & 7) == 0 && ((uintptr_t)a.k_cache & 15) == 0 && ((uintptr_t)a.v_cache & 15) == 0;
@@ -533,13 +560,13 @@ static int launch_ndb(const AttnArgs& a, int tiles, int tpt, int cpt, int chunk_
         attn_mfma_kernel<NDB, true><<<grid, WAVE, 0, a.stream>>>(
             (const uint16_t*)a.q, a.ldq, (const uint16_t*)a.k_cache, (const uint16_t*)a.v_cache, a.kv_width,
             a.block_table, a.max_blocks, a.token_slot, a.positions, a.q_start, a.n_seqs, (uint16_t*)a.out, a.ldo,
-            (float*)a.workspace, a.n_heads, a.page_tokens, a.window, sl, tpt, cpt, chunk_keys, n_chunks,
+            (float*)a.workspace, a.n_heads, page_shift(a.page_tokens), a.window, sl, tpt, cpt, chunk_keys, n_chunks,
             a.max_q_len <= tpt);
     else
         attn_mfma_kernel<NDB, false><<<grid, WAVE, 0, a.stream>>>(
             (const uint16_t*)a.q, a.ldq, (const uint16_t*)a.k_cache, (const uint16_t*)a.v_cache, a.kv_width,
             a.block_table, a.max_blocks, a.token_slot, a.positions, a.q_start, a.n_seqs, (uint16_t*)a.out, a.ldo,
-            nullptr, a.n_heads, a.page_tokens, a.window, sl, tpt, cpt, chunk_keys, n_chunks, a.max_q_len <= tpt);
+            nullptr, a.n_heads, page_shift(a.page_tokens), a.window, sl, tpt, cpt, chunk_keys, n_chunks, a.max_q_len <= tpt);
     HFA_LAUNCH_CHECK("attn_mfma");
     return 0;
 }
@@ -550,8 +577,8 @@ static int launch_prefill(const AttnArgs& a, int tpt, int cpt) {
     dim3 grid((a.n_tokens + tile_tokens - 1) / tile_tokens + a.n_seqs, a.n_kv_heads);
     attn_prefill_kernel<NDB><<<grid, 4 * WAVE, 0, a.stream>>>(
         (const uint16_t*)a.q, a.ldq, (const uint16_t*)a.k_cache, (const uint16_t*)a.v_cache, a.kv_width, a.block_table,
-        a.max_blocks, a.token_slot, a.positions, a.q_start, a.n_seqs, (uint16_t*)a.out, a.ldo, a.page_tokens,
-        a.window, a.scale * 1.4426950408889634f, tpt, cpt);
+        a.max_blocks, a.token_slot, a.positions, a.q_start, a.n_seqs, (uint16_t*)a.out, a.ldo,
+        page_shift(a.page_tokens), a.window, a.scale * 1.4426950408889634f, tpt, cpt);
     HFA_LAUNCH_CHECK("attn_prefill");
     return 0;
 }

@@ -279,7 +279,9 @@ class Ops:
             step.max_q_len, step.max_seq_len, out.data_ptr(), ldo, T, n_heads, n_kv_heads, head_dim,
             cache.page_tokens, int(window), float(scale), self.attn_workspace.data_ptr(),
             self.attn_workspace.numel(),
-            1 if self.force_plain_attention else 0, self._stream()))
+            # the matrix-core kernels address the cache with 32-bit element offsets and 24-bit row numbers
+            1 if self.force_plain_attention or cache.k.numel() >= 1 << 32 or cache.k.shape[0] >= 1 << 24 else 0,
+            self._stream()))
 
     def swiglu(self, gate_up, out):
         self.settle()

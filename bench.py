@@ -2,6 +2,7 @@
 """Throughput of the engine on the Qwen2.5-7B shape with random weights, one GPU.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L] [--no-points]
+    python bench.py --workload 0.5b | 32b      (the baseline's other workloads, through the scheduler)
 
 A step is one decode step of ``--batch`` sequences (default 8) whose prompts of 2,048
 random ids were prefilled before; W steps are run untimed, then exactly K steps are timed
@@ -23,6 +24,21 @@ SHAPE_7B = dict(architectures=["Qwen2ForCausalLM"], model_type="qwen2", num_hidd
                 num_attention_heads=28, num_key_value_heads=4, head_dim=128, intermediate_size=18944,
                 vocab_size=152064, rope_theta=1000000.0, rms_norm_eps=1e-6, tie_word_embeddings=False,
                 use_sliding_window=False, max_position_embeddings=32768, hidden_act="silu")
+# The other two workloads of the baseline: many requests of mixed lengths through the scheduler.
+WORKLOADS = {
+    "0.5b": dict(shape=dict(architectures=["Qwen2ForCausalLM"], model_type="qwen2", num_hidden_layers=24, hidden_size=896,
+                            num_attention_heads=14, num_key_value_heads=2, head_dim=64, intermediate_size=4864,
+                            vocab_size=151936, rope_theta=1000000.0, rms_norm_eps=1e-6, tie_word_embeddings=True,
+                            use_sliding_window=False, max_position_embeddings=32768, hidden_act="silu"),
+                 name="Qwen2.5-0.5B shape, random weights", requests=64, prompt_lo=16, prompt_hi=4096, new_tokens=128,
+                 ctx=32768, budget=2048),
+    "32b": dict(shape=dict(architectures=["Qwen2ForCausalLM"], model_type="qwen2", num_hidden_layers=64, hidden_size=5120,
+                           num_attention_heads=40, num_key_value_heads=8, head_dim=128, intermediate_size=27648,
+                           vocab_size=152064, rope_theta=1000000.0, rms_norm_eps=1e-5, tie_word_embeddings=False,
+                           use_sliding_window=False, max_position_embeddings=8192, hidden_act="silu"),
+                name="Qwen2.5-32B shape, random weights", requests=16, prompt_lo=4096, prompt_hi=4096, new_tokens=128,
+                ctx=8192, budget=1024),
+}
 PROMPT, NEW, PAGE = 2048, 256, 16
 HBM_PEAK = 8.0e12
 FLOP_PEAK = {"bf16": 2.5e15, "fp32": 157.3e12}
@@ -53,6 +69,50 @@ def prefill_flops(c, T):
     return 2.0 * T * L * per_layer + L * 4.0 * D * H * T * (T + 1) / 2 + 2.0 * head
 
 
+def serve_workload(which, dtype):
+    """``--workload 0.5b | 32b``: all requests are submitted at once and served by the scheduler
+    (prompt portions under the token budget beside decoded tokens, greedy); the second of two
+    runs is timed. One JSON line: prompt and generated tokens per second of wall time."""
+    import numpy as np
+    import torch
+    import hf_cpu_amd
+    import hf_cpu_amd.session as S
+    w = WORKLOADS[which]
+    cfg = hf_cpu_amd.config_from_dict(w["shape"])
+    t0 = time.perf_counter()
+    s = S.Session(cfg, dtype=dtype, ctx_max=w["ctx"], batch=w["budget"], page_size=PAGE, max_seqs=64,
+                  kv_tokens=w["requests"] * (w["prompt_hi"] + w["new_tokens"] + PAGE), seed=0)
+    torch.cuda.synchronize()
+    print(f"[bench] weights and cache ready in {time.perf_counter() - t0:.1f} s", file=sys.stderr, flush=True)
+    rng = np.random.default_rng(0)
+    prompts = [[int(t) for t in rng.integers(0, cfg.vocab_size, int(rng.integers(w["prompt_lo"], w["prompt_hi"] + 1)))]
+               for _ in range(w["requests"])]
+    for rep in range(2):
+        steps0 = s.engine.steps_run
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        gens = s.generate(prompts, temp=0.0, max_tokens=w["new_tokens"])
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        steps = s.engine.steps_run - steps0
+        n_prompt, n_gen = sum(len(p) for p in prompts), sum(len(g.tokens) for g in gens)
+        print(f"[bench] run {rep}: {n_prompt} prompt + {n_gen} generated tokens in {dt:.2f} s, {steps} steps, "
+              f"{sum(g.preemptions for g in gens)} preemptions", file=sys.stderr, flush=True)
+    sh = w["shape"]
+    short = "bf16" if dtype == "bfloat16" else "fp32"
+    print(json.dumps({
+        "metric": f"tokens served per second, prompts and generated ({w['name']})", "value": round((n_prompt + n_gen) / dt, 1),
+        "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": 1, "ms_per_step": round(dt / steps * 1e3, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": short, "data": "synthetic",
+        "config": {"model": w["name"], "num_hidden_layers": sh["num_hidden_layers"], "hidden_size": sh["hidden_size"],
+                   "num_attention_heads": sh["num_attention_heads"], "num_key_value_heads": sh["num_key_value_heads"],
+                   "head_dim": sh["head_dim"], "intermediate_size": sh["intermediate_size"], "vocab_size": sh["vocab_size"],
+                   "requests": w["requests"], "prompt_tokens": n_prompt, "generated_tokens": n_gen,
+                   "token_budget": w["budget"], "ctx": w["ctx"], "page_size": PAGE, "parallelism": "none"},
+        "generated_tok_per_s": round(n_gen / dt, 1)}))
+    return 0
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -65,10 +125,14 @@ def main():
     ap.add_argument("--prefill-reps", type=int, default=3)
     ap.add_argument("--only", choices=["prefill", "decode"], default=None,
                     help="run one phase only and print a short line (for profiling a phase by itself)")
+    ap.add_argument("--workload", choices=["7b", "0.5b", "32b"], default="7b",
+                    help="7b: the default measurement; 0.5b, 32b: the baseline's other workloads, served by the scheduler")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this engine runs on one GPU; --gpus must be 1")
         return 2
+    if args.workload != "7b":
+        return serve_workload(args.workload, args.dtype)
     if args.steps + args.warmup > NEW:
         print(f"bench.py: --steps + --warmup must not exceed the {NEW} new tokens of the workload")
         return 2

@@ -2,8 +2,11 @@
 
 ``load_engine(model_dir, dtype=...)`` reads a model folder (config.json +
 model.safetensors) and returns an Engine whose ``step`` runs batches of prompt
-portions and decoded tokens from a paged cache; ``generate`` and the command line
-sit on top of it. See DESIGN.md at the repository root for what each part owns.
+portions and decoded tokens from a paged cache; ``session.Session.generate`` and the
+command line (``cli``) sit on top of it. Configuration in ``config``, tensors in
+``weights``, layer parts in ``parts``, the cache's books and memory in ``cache``, the step
+function and the scheduler in ``engine``, sampling in ``sampling``, the HIP sources in
+``csrc`` and their Python face in ``kernels``.
 """
 from . import parts, models           # noqa: F401  (registration of parts and architectures)
 from .config import Qwen2Config, config_from_dict, read_config

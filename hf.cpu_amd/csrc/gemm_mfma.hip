@@ -15,6 +15,8 @@
 // Small M (decode) is bandwidth-bound and has few output tiles: K is split over blockIdx.z,
 // partial sums go to a workspace and a second kernel adds them in a fixed order and applies
 // bias and the output mode. Nothing is accumulated with atomics: results are reproducible.
+#include <type_traits>
+
 #include "common.h"
 #include "gemm_internal.h"
 
@@ -359,12 +361,13 @@ __global__ __launch_bounds__(WM* WN* WAVE) void gemm_dma_kernel(
     constexpr int SPREAD = STAGES == 3 ? (PRODUCTS / 2 > C::LOADS ? PRODUCTS / 2 : C::LOADS) : PRODUCTS;
     static_assert(SPREAD >= C::LOADS && SPREAD <= PRODUCTS && C::STEPS % 2 == 0, "at most one request after a matrix instruction");
     int stage = 0;
-    for (int t = 0; t < nk; t++) {
-        if (t + STAGES - 2 < nk)
+    // `steady`: tile t + AHEAD exists, so the step has no condition in it (all but the last steps).
+    auto step = [&](int t, auto steady) {
+        constexpr bool STEADY = decltype(steady)::value;
+        if (STEADY || t + STAGES - 2 < nk)
             asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(C::LOADS * (STAGES - 3)) : "memory");
         else
             asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
-        const bool more = t + AHEAD < nk;
         const int into = stage + AHEAD < STAGES ? stage + AHEAD : stage + AHEAD - STAGES;
         const int next = stage + 1 < STAGES ? stage + 1 : 0;
         int done = 0;
@@ -372,20 +375,24 @@ __global__ __launch_bounds__(WM* WN* WAVE) void gemm_dma_kernel(
         for (int j = 0; j < C::STEPS; j++) {
             if (j + 1 < C::STEPS)
                 fragments(stage, j + 1, fa[(j + 1) & 1], fw[(j + 1) & 1]);
-            else if (t + 1 < nk)
+            else if (STEADY || t + 1 < nk)
                 fragments(next, 0, fa[0], fw[0]);
+            __builtin_amdgcn_sched_barrier(0);               // the reads are issued before the products that hide them
 #pragma unroll
             for (int i = 0; i < C::FM; i++)
 #pragma unroll
                 for (int jj = 0; jj < C::FN; jj++) {
                     acc[i][jj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[j & 1][i], fw[j & 1][jj], acc[i][jj], 0, 0, 0);
                     done++;                                  // requests are dealt evenly among the first products
-                    if (done <= SPREAD && done * C::LOADS / SPREAD != (done - 1) * C::LOADS / SPREAD && more)
+                    if (STEADY && done <= SPREAD && done * C::LOADS / SPREAD != (done - 1) * C::LOADS / SPREAD)
                         request(done * C::LOADS / SPREAD - 1, into, t + AHEAD);
                 }
         }
         stage = next;
-    }
+    };
+    int t = 0;
+    for (; t + AHEAD < nk; t++) step(t, std::true_type());
+    for (; t < nk; t++) step(t, std::false_type());
     if constexpr (MODE == OUT_BF16 || MODE == OUT_SWIGLU) {
         // 16-bit results leave through LDS: a lane holds single columns, and a store of 2 bytes per
         // lane costs the memory path as much as one of 16. The block's tile is put together in

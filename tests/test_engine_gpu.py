@@ -12,6 +12,7 @@ pytestmark = pytest.mark.gpu
 # fp32: rounding of a few hundred fused multiply-adds per value (measured: about 1e-6).
 # bf16: activations and cache rounded to 8 bits of mantissa at every part (measured: 0.8e-2).
 TOL = {"float32": 5e-6, "bfloat16": 2e-2}
+KERNELS_AGREE = 2e-2     # bf16: another order of summation flips roundings of activations, which spread like any rounding
 LENGTHS = {"A": [7, 19, 33, 70, 101], "B": [1, 40, 77, 100, 130]}
 
 
@@ -197,3 +198,50 @@ def test_graph_replay_equals_eager(gpu, tiny, dtype):
         assert err <= (1e-6 if dtype == "float32" else 1e-2), f"decode step {i}: graph and eager differ by {err:.3e}"
     got = {("r4", len(reqs["r4"]) - 25 + i): runs[True][i][2] for i in range(25)}
     helpers.compare(got, want, TOL[dtype], "graph replay")
+
+
+@pytest.mark.parametrize("seed", range(20))
+def test_random_configurations(gpu, tmp_path, seed):
+    """Configurations drawn at random within what config.json allows (head sizes in steps of
+    16, any number of heads and groups, widths and vocabularies that are no power of two and not
+    even multiples of 8, windows, page sizes), each through a mixed trace with few pages, in
+    both precisions against the plain implementation: the kernels either take a size or hand
+    it to a kernel that does; they never give a wrong result."""
+    import hf_cpu_amd
+    rng = np.random.default_rng(100 + seed)
+    D = int(rng.choice([16, 32, 48, 64, 80, 96, 128]))
+    G = int(rng.choice([1, 2, 3, 4]))
+    group = int(rng.choice([1, 2, 3, 4, 7]))
+    window = int(rng.choice([0, 0, 7, 20, 33]))
+    layers = int(rng.integers(1, 4))
+    cfg = dict(architectures=["Qwen2ForCausalLM"], model_type="qwen2", num_hidden_layers=layers,
+               hidden_size=int(rng.choice([40, 56, 72, 100, 136, 150])), num_attention_heads=G * group,
+               num_key_value_heads=G, head_dim=D, intermediate_size=int(rng.choice([64, 100, 192, 200, 330])),
+               vocab_size=int(rng.integers(50, 1200)), rope_theta=float(rng.choice([1e4, 5e5, 1e6])),
+               rms_norm_eps=float(rng.choice([1e-6, 1e-5, 3e-5])), tie_word_embeddings=bool(rng.integers(0, 2)),
+               use_sliding_window=window > 0, sliding_window=window or 4096,
+               max_window_layers=int(rng.integers(0, layers + 1)), max_position_embeddings=256, hidden_act="silu")
+    page = int(rng.choice([4, 8, 16, 32]))
+    d = helpers.make_model_dir(str(tmp_path / "m"), cfg, seed=seed)
+    reqs = helpers.random_requests(cfg, [int(n) for n in rng.integers(1, 90, 5)], seed=seed)
+    steps = helpers.trace_mixed(reqs, seed=seed, max_live=3)
+    def run(dtype, plain_kernels=False):
+        engine = hf_cpu_amd.load_engine(d, dtype=dtype, page_tokens=page,
+                                        max_tokens=helpers.max_live_tokens(steps, round_to=max(64, page)), max_seqs=3)
+        engine.ops.force_plain_gemm = engine.ops.force_plain_attention = plain_kernels
+        got = helpers.run_trace_in_engine(engine, steps)
+        assert not engine.manager.held
+        engine.manager.check()
+        return got
+    helpers.compare(run("float32"), helpers.plain_logits(d, reqs), TOL["float32"], f"random configuration {seed} fp32 {cfg}")
+    # bf16 rounds activations at the same places whichever kernels run. Against float64 (weights
+    # rounded alike) widths as small as 40 average less of that rounding away than the two fixed
+    # configurations do: the bound is 3e-2 here. A kernel's fault shows between the kernels:
+    # the matrix-core kernels against the plain ones, on the same roundings.
+    want = helpers.plain_logits(d, reqs, round_weights_bf16=True)
+    got, got_plain = run("bfloat16"), run("bfloat16", plain_kernels=True)
+    helpers.compare(got, want, 3e-2, f"random configuration {seed} bf16 {cfg}")
+    helpers.compare(got_plain, want, 3e-2, f"random configuration {seed} bf16 with plain kernels {cfg}")
+    worst = max(float(np.max(np.abs(got[k] - got_plain[k]))) / float(np.max(np.abs(want[k[0]]))) for k in got)
+    assert worst <= KERNELS_AGREE, f"random configuration {seed}: kernels differ by {worst:.2e} {cfg}"
+    print(f"random configuration {seed}: matrix-core and plain kernels differ by {worst:.2e}")

@@ -15,6 +15,14 @@
 // Small M (decode) is bandwidth-bound and has few output tiles: K is split over blockIdx.z,
 // partial sums go to a workspace and a second kernel adds them in a fixed order and applies
 // bias and the output mode. Nothing is accumulated with atomics: results are reproducible.
+//
+// Which kernel takes which shape (gemm_mfma_launch, at the end of this file):
+//   M <= 32          gemm_mfma_kernel, tiles of 32 x 128, K split, two register sets of loads in flight
+//   M in 33 .. 64    gemm_stream_kernel (gemm_stream.hip) if N is a multiple of 128 and K of 64 and the
+//                    output has fewer than 512 tiles; else gemm_mfma_kernel with tiles of 64 x 128
+//   M > 64           gemm_dma_kernel (below) with tiles of 256 rows, if M wastes few of them and the
+//                    output has 128 tiles of 256 x 256 (or 64, then with K cut in two, or with tiles
+//                    of 256 x 128); else gemm_mfma_kernel with tiles of 128 x 128
 #include <type_traits>
 
 #include "common.h"

@@ -107,11 +107,57 @@ __device__ __forceinline__ void gemm_epilogue(floatx16 (&acc)[C::FM][C::FN], con
     }
 }
 
+// The block's tile of 16-bit results in LDS: rows of WIDTH columns, 16 bytes of padding.
+template <int BN, int MODE>
+struct DmaOut {
+    static constexpr int PAIR = MODE == OUT_SWIGLU ? 2 : 1;      // 32 gate and 32 up columns give 32 results
+    static constexpr int WIDTH = BN / PAIR, STRIDE = WIDTH + 8;
+    static constexpr int bytes(int bm) { return (MODE == OUT_BF16 || MODE == OUT_SWIGLU) ? bm * STRIDE * 2 : 0; }
+};
+
+// 16-bit results leave through LDS: a lane holds single columns, and a store of 2 bytes per lane
+// costs the memory path as much as one of 16. The block's tile is put together in LDS (the operand
+// stages are free by now), then written out 16 bytes per lane, whole rows. Needs 16-byte aligned
+// output rows and a multiple of 8 output columns (the launchers check).
+template <class C, int BM, int BN, int MODE>
+__device__ __forceinline__ void gemm_epilogue_rows(floatx16 (&acc)[C::FM][C::FN], const float* __restrict__ bias,
+                                                   void* __restrict__ out, int ldo, int M, int N, int m0, int n0,
+                                                   int wm, int wn, int lane, int tid, uint16_t* smem) {
+    using O = DmaOut<BN, MODE>;
+    static_assert(MODE != OUT_SWIGLU || C::FN % 2 == 0, "gate and up blocks must meet in one wave");
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < C::FM; i++) {
+#pragma unroll
+        for (int j = 0; j < C::FN; j += O::PAIR) {
+            const int col = (wn * C::TN + j * 32) / O::PAIR + (lane & 31);      // within the block's tile
+            const int gcol = n0 + wn * C::TN + j * 32 + (lane & 31);            // column of N (the gate's, if paired)
+            const float b = (MODE == OUT_BF16 && bias && gcol < N) ? bias[gcol] : 0.f;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int row = wm * C::TM + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
+                float v = acc[i][j][r] + b;
+                if constexpr (MODE == OUT_SWIGLU) v = (v / (1.0f + expf(-v))) * acc[i][j + 1][r];
+                smem[row * O::STRIDE + col] = bf16_bits(v);
+            }
+        }
+    }
+    __syncthreads();
+    const int out0 = n0 / O::PAIR, n_out = N / O::PAIR;
+    uint16_t* o16 = reinterpret_cast<uint16_t*>(out);
+    for (int c = tid; c < BM * (O::WIDTH / 8); c += C::NT) {
+        const int row = c / (O::WIDTH / 8), piece = c % (O::WIDTH / 8);
+        if (m0 + row < M && out0 + piece * 8 < n_out)
+            *reinterpret_cast<uint4*>(o16 + (size_t)(m0 + row) * ldo + out0 + piece * 8) =
+                *reinterpret_cast<const uint4*>(smem + row * O::STRIDE + piece * 8);
+    }
+}
+
 template <int BM, int BN, int BK, int WM, int WN, int MODE, int PF>
 __global__ __launch_bounds__(WM* WN* WAVE) void gemm_mfma_kernel(
     const uint16_t* __restrict__ A, int lda, const uint16_t* __restrict__ W, int ldw,
     const float* __restrict__ bias, void* __restrict__ out, int ldo, int M, int N, int K, int k_per_split,
-    int tiles_m, int tiles_n) {
+    int tiles_m, int tiles_n, int rows_out) {
     using C = MfmaCfg<BM, BN, BK, WM, WN>;
     extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
     const int tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
@@ -222,6 +268,13 @@ __global__ __launch_bounds__(WM* WN* WAVE) void gemm_mfma_kernel(
         __syncthreads();
     }
 
+    if constexpr (MODE == OUT_BF16 || MODE == OUT_SWIGLU) {
+        static_assert(DmaOut<BN, MODE>::bytes(BM) <= C::SMEM, "the tile of results fits the operand stages");
+        if (rows_out) {                                      // uniform: the output allows 16-byte stores
+            gemm_epilogue_rows<C, BM, BN, MODE>(acc, bias, out, ldo, M, N, m0, n0, wm, wn, lane, tid, smem);
+            return;
+        }
+    }
     gemm_epilogue<C, MODE>(acc, bias, out, ldo, M, N, m0, n0, wm, wn, lane);
 }
 
@@ -259,14 +312,6 @@ struct DmaCfg {
     static_assert(TM % 32 == 0 && TN % 32 == 0, "wave tiles are made of 32x32x16 products");
     static_assert(FM * FN * STEPS >= LOADS, "at most one request after a matrix instruction");
     __device__ static constexpr int swizzle(int row) { return BK == 64 ? (row & 7) : ((row >> 1) & 3); }
-};
-
-// The block's tile of 16-bit results in LDS: rows of WIDTH columns, 16 bytes of padding.
-template <int BN, int MODE>
-struct DmaOut {
-    static constexpr int PAIR = MODE == OUT_SWIGLU ? 2 : 1;      // 32 gate and 32 up columns give 32 results
-    static constexpr int WIDTH = BN / PAIR, STRIDE = WIDTH + 8;
-    static constexpr int bytes(int bm) { return (MODE == OUT_BF16 || MODE == OUT_SWIGLU) ? bm * STRIDE * 2 : 0; }
 };
 
 template <int BM, int BN, int BK, int WM, int WN, int STAGES, int MODE>
@@ -402,37 +447,7 @@ __global__ __launch_bounds__(WM* WN* WAVE) void gemm_dma_kernel(
     for (; t + AHEAD < nk; t++) step(t, std::true_type());
     for (; t < nk; t++) step(t, std::false_type());
     if constexpr (MODE == OUT_BF16 || MODE == OUT_SWIGLU) {
-        // 16-bit results leave through LDS: a lane holds single columns, and a store of 2 bytes per
-        // lane costs the memory path as much as one of 16. The block's tile is put together in
-        // LDS (the operand stages are free now), then written out 16 bytes per lane, whole rows.
-        using O = DmaOut<BN, MODE>;
-        static_assert(MODE != OUT_SWIGLU || C::FN % 2 == 0, "gate and up blocks must meet in one wave");
-        __syncthreads();
-#pragma unroll
-        for (int i = 0; i < C::FM; i++) {
-#pragma unroll
-            for (int j = 0; j < C::FN; j += O::PAIR) {
-                const int col = (wn * C::TN + j * 32) / O::PAIR + (lane & 31);      // within the block's tile
-                const int gcol = n0 + wn * C::TN + j * 32 + (lane & 31);            // column of N (the gate's, if paired)
-                const float b = (MODE == OUT_BF16 && bias && gcol < N) ? bias[gcol] : 0.f;
-#pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const int row = wm * C::TM + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
-                    float v = acc[i][j][r] + b;
-                    if constexpr (MODE == OUT_SWIGLU) v = (v / (1.0f + expf(-v))) * acc[i][j + 1][r];
-                    smem[row * O::STRIDE + col] = bf16_bits(v);
-                }
-            }
-        }
-        __syncthreads();
-        const int out0 = n0 / O::PAIR, n_out = N / O::PAIR;
-        uint16_t* o16 = reinterpret_cast<uint16_t*>(out);
-        for (int c = tid; c < BM * (O::WIDTH / 8); c += C::NT) {
-            const int row = c / (O::WIDTH / 8), piece = c % (O::WIDTH / 8);
-            if (m0 + row < M && out0 + piece * 8 < n_out)
-                *reinterpret_cast<uint4*>(o16 + (size_t)(m0 + row) * ldo + out0 + piece * 8) =
-                    *reinterpret_cast<const uint4*>(smem + row * O::STRIDE + piece * 8);
-        }
+        gemm_epilogue_rows<C, BM, BN, MODE>(acc, bias, out, ldo, M, N, m0, n0, wm, wn, lane, tid, smem);
     } else {
         gemm_epilogue<C, MODE>(acc, bias, out, ldo, M, N, m0, n0, wm, wn, lane);
     }
@@ -477,8 +492,10 @@ static int launch_cfg(const GemmArgs& g, void* out, int splits, int k_per_split)
     }
     const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
     dim3 grid(tiles_m * tiles_n, 1, splits);
+    const int n_out = MODE == OUT_SWIGLU ? g.N / 2 : g.N;
+    const int rows_out = (MODE == OUT_BF16 || MODE == OUT_SWIGLU) && g.ldo % 8 == 0 && n_out % 8 == 0 && ((uintptr_t)out & 15) == 0;
     kernel<<<grid, C::NT, C::SMEM, g.stream>>>((const uint16_t*)g.a, g.lda, (const uint16_t*)g.w, g.ldw, g.bias, out,
-                                              g.ldo, g.M, g.N, g.K, k_per_split, tiles_m, tiles_n);
+                                              g.ldo, g.M, g.N, g.K, k_per_split, tiles_m, tiles_n, rows_out);
     HFA_LAUNCH_CHECK("gemm_mfma");
     return 0;
 }
@@ -579,11 +596,13 @@ int gemm_mfma_launch(const GemmArgs& g, void* workspace, size_t workspace_bytes,
     const int BM = g.M > 64 ? 128 : (g.M > 32 ? 64 : 32), BN = 128;
     const int tiles = ((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN);
     const int k_tiles = (g.K + BK - 1) / BK;
-    // Few tiles and a long K: split K so that the machine is full; every split keeps at least 4 steps.
+    // Few tiles and a long K: split K so that the machine is full (two blocks a CU for the small tiles
+    // of decode, one for tiles of 128 rows); every split keeps at least 4 steps (8 for the large tiles).
     int splits = 1;
-    if (g.M <= 64 && tiles < 512) {
-        splits = (512 + tiles - 1) / tiles;
-        const int most = k_tiles / 4 > 0 ? k_tiles / 4 : 1;
+    const int want_blocks = g.M <= 64 ? 512 : 256, least_steps = g.M <= 64 ? 4 : 8;
+    if (tiles < want_blocks) {
+        splits = (want_blocks + tiles - 1) / tiles;
+        const int most = k_tiles / least_steps > 0 ? k_tiles / least_steps : 1;
         if (splits > most) splits = most;
         const size_t per_split = (size_t)g.M * g.N * sizeof(float);
         if (workspace == nullptr || per_split == 0) splits = 1;

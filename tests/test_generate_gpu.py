@@ -245,6 +245,45 @@ def test_generation_survives_a_cache_that_is_too_small(gpu, models):
     assert not tiny.engine.manager.held
 
 
+@pytest.mark.parametrize("seed", range(6))
+def test_serving_at_random_with_forks_a_window_and_a_tight_cache(gpu, models, seed):
+    """Configuration B (windowed layers, pages of 8) under a random load: prompts of 1 to 120
+    tokens, 3 to 30 new tokens, some with two or three continuations that fork from the
+    prompt's cache and sample with their own seeds, a token budget of 24 and a cache of 320
+    tokens, so that portions shrink, requests are preempted and recomputed, and shared pages
+    come and go. Every continuation ends with the tokens it gets when it runs alone in a
+    roomy cache, and the books balance."""
+    import hf_cpu_amd.session as S
+    from hf_cpu_amd.engine.scheduler import Request
+    from hf_cpu_amd.sampling import SamplerParams
+    cfg = helpers.CONFIG_B
+    rng = np.random.default_rng(40 + seed)
+    roomy = S.Session(models["B"], dtype="float32", ctx_max=256, batch=64, page_size=8, max_seqs=8)
+    tight = S.Session(models["B"], dtype="float32", ctx_max=256, batch=24, page_size=8, max_seqs=6, kv_tokens=320)
+    jobs = []
+    for j in range(10):
+        prompt = [int(t) for t in rng.integers(0, cfg["vocab_size"], int(rng.integers(1, 121)))]
+        n = int(rng.choice([1, 1, 2, 3]))
+        temp = float(rng.choice([0.0, 0.9]))
+        jobs.append((prompt, n, temp, int(rng.integers(3, 31)), 100 * j))
+    sched = tight.scheduler()
+    families = []
+    for j, (prompt, n, temp, new, seed0) in enumerate(jobs):
+        fam = [Request((j, i), list(prompt), SamplerParams(temp, 40, 0.95, 0.05), new, seed0 + i) for i in range(n)]
+        families.append(fam)
+        sched.submit(fam[0], forks=fam[1:])
+    sched.run()
+    mgr = tight.engine.manager
+    mgr.check()
+    assert not mgr.held and all(p.n_held == 0 for p in mgr.pools)
+    assert sum(r.preemptions for fam in families for r in fam) > 0, "the cache was meant to run out"
+    for (prompt, n, temp, new, seed0), fam in zip(jobs, families):
+        for i, r in enumerate(fam):
+            assert r.error is None and r.stop == "length", (r.req_id, r.error)
+            alone = roomy.generate(prompt, n=1, temp=temp, seed=seed0 + i, max_tokens=new)[0].tokens
+            assert r.generated == alone, f"request {r.req_id}: preempted {r.preemptions} times"
+
+
 def test_real_layer_sizes_in_both_precisions(gpu, tmp_path):
     """One layer with the sizes of the 7B shape (hidden 3584, 28 query heads on 4 key/value heads of
     128, feed-forward 18944; the vocabulary cut to 4096 to keep the plain implementation quick):

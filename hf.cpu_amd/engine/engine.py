@@ -9,7 +9,7 @@ Reference: ``forward_impl`` (src/model.c:545-640) with its two batch shapes
 import numpy as np
 import torch
 
-from ..cache import CacheManager, CacheStorage, OutOfPages
+from ..cache import CacheManager, CacheStorage
 from ..status import EINVAL, fail
 from .batch import Entry, GroupInputs, IntStaging, StepInputs, as_i32
 

@@ -12,7 +12,6 @@ from dataclasses import dataclass, field
 
 import torch
 
-from .config import read_config
 from .engine import Engine
 from .engine.scheduler import Request, Scheduler
 from .kernels import Ops

@@ -1,6 +1,4 @@
 """Configuration reading and the architecture registry (no GPU)."""
-import json
-
 import pytest
 
 import helpers

@@ -3,7 +3,6 @@ import numpy as np
 import pytest
 
 import helpers
-import plain
 
 pytestmark = pytest.mark.gpu
 

@@ -300,10 +300,14 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
     __shared__ __attribute__((aligned(16))) uint16_t v_s[2][D * PVS];
     const int tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
     const int col = lane & 31, half = lane >> 5;
-    const int g = blockIdx.y;
+    const int g = blockIdx.x;
     const int tile_tokens = 4 * tpt;
 
-    int tile = blockIdx.x, t0 = -1, t_end = 0;
+    // Tiles late in a prompt see many keys, early ones few. Blocks are numbered with the key/value
+    // head fastest and the tiles from the longest down, so that the long tiles of all heads start
+    // first and the short ones fill in beside them (with the head slowest, a CU got two blocks of
+    // the same length, and the CUs with the longest tiles set the kernel's time).
+    int tile = blockIdx.y, t0 = -1, t_end = 0;
     for (int s = 0; s < n_seqs; s++) {
         const int a = q_start[s], b = q_start[s + 1];
         const int nt = (b - a + tile_tokens - 1) / tile_tokens;
@@ -574,7 +578,7 @@ static int launch_ndb(const AttnArgs& a, int tiles, int tpt, int cpt, int chunk_
 template <int NDB>
 static int launch_prefill(const AttnArgs& a, int tpt, int cpt) {
     const int tile_tokens = 4 * tpt;
-    dim3 grid((a.n_tokens + tile_tokens - 1) / tile_tokens + a.n_seqs, a.n_kv_heads);
+    dim3 grid(a.n_kv_heads, (a.n_tokens + tile_tokens - 1) / tile_tokens + a.n_seqs);
     attn_prefill_kernel<NDB><<<grid, 4 * WAVE, 0, a.stream>>>(
         (const uint16_t*)a.q, a.ldq, (const uint16_t*)a.k_cache, (const uint16_t*)a.v_cache, a.kv_width, a.block_table,
         a.max_blocks, a.token_slot, a.positions, a.q_start, a.n_seqs, (uint16_t*)a.out, a.ldo,
@@ -587,7 +591,7 @@ int attn_mfma_launch(const AttnArgs& a) {
     const int cpt = a.n_heads / a.n_kv_heads;              // columns per token: the heads of a group
     const int tpt = 32 / cpt;                              // tokens per tile
     // Steps with prompt portions: the kernel that shares keys and values between four waves.
-    if (a.max_q_len >= 16 && a.page_tokens % 8 == 0) {
+    if (a.max_q_len >= 16 && a.page_tokens % 8 == 0 && (a.n_tokens + 4 * tpt - 1) / (4 * tpt) + a.n_seqs <= 65535) {
         switch (a.head_dim / 32) {
             case 1: return launch_prefill<1>(a, tpt, cpt);
             case 2: return launch_prefill<2>(a, tpt, cpt);

@@ -208,6 +208,7 @@ __global__ __launch_bounds__(128) void rope_store_kernel(
 // rows of one page, every value column is written with one 16-byte store instead of eight
 // 2-byte stores 2 * page_tokens bytes apart.
 #define ROPE_TOKENS 8
+#define ROPE_ROWS_FROM 512      // fewer tokens make too few blocks of 8: the kernel above spreads them better
 __global__ __launch_bounds__(256) void rope_store_rows_kernel(
     uint16_t* __restrict__ qkv, int ld, const int* __restrict__ positions, const float* __restrict__ inv_freq,
     int rot_dim, int H, int G, int D, uint16_t* __restrict__ k_cache, uint16_t* __restrict__ v_cache,
@@ -298,7 +299,7 @@ extern "C" int hfa_rope_store(void* qkv, int dtype, int ld, const int* positions
     HFA_REQUIRE(n_heads + 2 * n_kv_heads <= 65535, "rope_store: too many heads for the grid");
     const int kd = n_kv_heads * head_dim;
     const size_t rows_lds = (size_t)ROPE_TOKENS * rot_dim * sizeof(float) + (size_t)ROPE_TOKENS * kd * 2 + ROPE_TOKENS * sizeof(int);
-    if (dtype == HFA_BF16 && splits == 0 && n_tokens >= 4 * ROPE_TOKENS && rot_dim > 0 && rot_dim % 16 == 0 &&
+    if (dtype == HFA_BF16 && splits == 0 && n_tokens >= ROPE_ROWS_FROM && rot_dim > 0 && rot_dim % 16 == 0 &&
         head_dim % 8 == 0 && ld % 8 == 0 && ((uintptr_t)qkv & 15) == 0 && ((uintptr_t)k_cache & 15) == 0 &&
         ((uintptr_t)v_cache & 15) == 0 && rows_lds <= 48 * 1024) {
         rope_store_rows_kernel<<<(n_tokens + ROPE_TOKENS - 1) / ROPE_TOKENS, 256, rows_lds, stream>>>(

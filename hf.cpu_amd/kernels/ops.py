@@ -239,7 +239,7 @@ class Ops:
         if pend is not None and not pend.accumulate and pend.out.data_ptr() == qkv.data_ptr() \
                 and pend.out.shape == qkv.shape and qkv.shape[1] == (n_heads + 2 * n_kv_heads) * head_dim:
             self._pending = None
-            if qkv.dtype == torch.bfloat16 and qkv.shape[0] >= 32 and rot_dim > 0:
+            if qkv.dtype == torch.bfloat16 and qkv.shape[0] >= 512 and rot_dim > 0:
                 # A prompt portion: the kernel for many tokens does not add up partial sums; finishing
                 # the product first and then taking that kernel is the quicker way.
                 self._pending = pend

@@ -33,9 +33,12 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 // never subnormal results that matter), and the bf16 bits of a probability in [0, 1]: round to
 // nearest even without the NaN case.
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
-__device__ __forceinline__ uint32_t prob_bits(float p) {
-    const uint32_t u = __float_as_uint(p);
-    return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+// Two probabilities as a pair of bf16, round to nearest even: one v_cvt_pk_bf16_f32 on gfx950.
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t prob_pair(float lo, float hi) {
+    const floatx2 f = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
 }
 
 union Frag {
@@ -194,7 +197,7 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
             uint32_t w[4];
 #pragma unroll
             for (int e = 0; e < 4; e++)
-                w[e] = prob_bits(st[8 * kk + 2 * e]) | (prob_bits(st[8 * kk + 2 * e + 1]) << 16);
+                w[e] = prob_pair(st[8 * kk + 2 * e], st[8 * kk + 2 * e + 1]);
             pf[kk].u = make_uint4(w[0], w[1], w[2], w[3]);
         }
     };
@@ -293,21 +296,33 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
     const uint16_t* __restrict__ q, int ldq, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc, int kvw,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ token_slot,
     const int* __restrict__ positions, const int* __restrict__ q_start, int n_seqs, uint16_t* __restrict__ out,
-    int ldo, int psh, int window, float scale_log2e, int tpt, int cpt) {
+    int ldo, int psh, int window, float scale_log2e, int tpt, int cpt, int n_tiles, int pair_from) {
     constexpr int D = NDB * 32, KS = D / 16, KROW = D + 8;
     const int P = 1 << psh;                                // tokens per page, a power of two
     __shared__ __attribute__((aligned(16))) uint16_t k_s[2][KB * KROW];
     __shared__ __attribute__((aligned(16))) uint16_t v_s[2][D * PVS];
     const int tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
     const int col = lane & 31, half = lane >> 5;
-    const int g = blockIdx.x;
+    int g = blockIdx.x, tile = blockIdx.y;
     const int tile_tokens = 4 * tpt;
 
     // Tiles late in a prompt see many keys, early ones few. Blocks are numbered with the key/value
     // head fastest and the tiles from the longest down, so that the long tiles of all heads start
     // first and the short ones fill in beside them (with the head slowest, a CU got two blocks of
     // the same length, and the CUs with the longest tiles set the kernel's time).
-    int tile = blockIdx.y, t0 = -1, t_end = 0;
+    //
+    // When all blocks are resident at once, two to a CU, the second block of a CU (id pair_from + j,
+    // beside block j) takes the tiles from the shortest up, so that every CU has the same sum of keys.
+    if (pair_from > 0) {
+        const int id = blockIdx.y * gridDim.x + blockIdx.x;
+        if (id >= pair_from) {
+            const int j = id - pair_from;
+            if (j >= n_tiles * (int)gridDim.x - pair_from) return;
+            tile = n_tiles - 1 - j / (int)gridDim.x;
+            g = j % (int)gridDim.x;
+        }
+    }
+    int t0 = -1, t_end = 0;
     for (int s = 0; s < n_seqs; s++) {
         const int a = q_start[s], b = q_start[s + 1];
         const int nt = (b - a + tile_tokens - 1) / tile_tokens;
@@ -358,9 +373,9 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
     // global -> registers -> LDS. Keys: 32 rows of D elements = 4 D chunks of 16 bytes.
     // Values: D rows of 32 keys = 4 D chunks of 8 keys. Each thread takes up to NCH of both.
     constexpr int TOT = 4 * D, NCH = (TOT + 255) / 256;
-    u32x4 rk[NCH];
-    uint2 rv[NCH][2];
-    auto gload = [&](int key0) {
+    u32x4 rk0[NCH], rk1[NCH];
+    uint2 rv0[NCH][2], rv1[NCH][2];
+    auto gload = [&](int key0, u32x4 (&rk)[NCH], uint2 (&rv)[NCH][2]) {
 #pragma unroll
         for (int i = 0; i < NCH; i++) {
             const int c = tid + i * 256;
@@ -383,7 +398,7 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
             }
         }
     };
-    auto sstore = [&](int stage) {
+    auto sstore = [&](int stage, const u32x4 (&rk)[NCH], const uint2 (&rv)[NCH][2]) {
 #pragma unroll
         for (int i = 0; i < NCH; i++) {
             const int c = tid + i * 256;
@@ -409,12 +424,16 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
         }
         __syncthreads();
         const int last = first + (we - 1) * KB;
-        gload(first + wb * KB);
-        sstore(wb & 1);
+        auto at = [&](int b) { const int k = first + b * KB; return k < last ? k : last; };
+        gload(at(wb), rk0, rv0);
+        sstore(wb & 1, rk0, rv0);
+        gload(at(wb + 1), rk0, rv0);                          // unconditional: past the end the last block is fetched again
+        gload(at(wb + 2), rk1, rv1);
         __syncthreads();
-        for (int b = wb; b < we; b++) {
+        // Two register sets in rotation: the block after the next one is on its way while the next one
+        // goes into LDS, so a load has two blocks' worth of products and softmax to arrive.
+        auto one_block = [&](int b) {
             const int key0 = first + b * KB, stage = b & 1;
-            gload(key0 + KB < last ? key0 + KB : last);       // unconditional: the last block is fetched twice
             // A wave whose columns all end before this block skips the math. The test is made by all
             // lanes together: the matrix products need every lane, also those of unused columns.
             const bool wave_sees = __any(key0 <= vhi) != 0;
@@ -434,18 +453,15 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
                 // aside, whose results are dropped): no key of them needs the visibility test.
                 const bool inside = __all(!col_ok || (key0 >= vlo && key0 + KB - 1 <= vhi)) != 0;
                 float mx = NEG_BIG, mn, corr, psum = 0.f;
-                if (inside) {
+                if (inside) {                                   // the scale (positive) moves into the exponent's fma
 #pragma unroll
-                    for (int r = 0; r < 16; r++) {
-                        st[r] *= scale_log2e;
-                        mx = fmaxf(mx, st[r]);
-                    }
-                    mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+                    for (int r = 0; r < 16; r++) mx = fmaxf(mx, st[r]);
+                    mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE)) * scale_log2e;
                     mn = fmaxf(m, mx);
                     corr = fast_exp2(m - mn);
 #pragma unroll
                     for (int r = 0; r < 16; r++) {
-                        st[r] = fast_exp2(st[r] - mn);
+                        st[r] = fast_exp2(fmaf(st[r], scale_log2e, -mn));
                         psum += st[r];
                     }
                 } else {
@@ -481,7 +497,7 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
                     uint32_t w[4];
 #pragma unroll
                     for (int e = 0; e < 4; e++)
-                        w[e] = prob_bits(st[8 * kk + 2 * e]) | (prob_bits(st[8 * kk + 2 * e + 1]) << 16);
+                        w[e] = prob_pair(st[8 * kk + 2 * e], st[8 * kk + 2 * e + 1]);
                     pf[kk].u = make_uint4(w[0], w[1], w[2], w[3]);
                 }
 #pragma unroll
@@ -495,7 +511,16 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
                         o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf.v, pf[kk].v, o[db], 0, 0, 0);
                     }
             }
-            sstore(stage ^ 1);
+        };
+        for (int b = wb; b < we; b += 2) {
+            one_block(b);
+            sstore((b & 1) ^ 1, rk0, rv0);                    // block b + 1
+            gload(at(b + 3), rk0, rv0);
+            __syncthreads();
+            if (b + 1 >= we) break;
+            one_block(b + 1);
+            sstore(b & 1, rk1, rv1);                          // block b + 2
+            gload(at(b + 4), rk1, rv1);
             __syncthreads();
         }
     }
@@ -550,7 +575,8 @@ static int page_shift(int page_tokens) {
 
 bool attn_mfma_supports(const AttnArgs& a) {
     const int group = a.n_heads / a.n_kv_heads;
-    return a.head_dim % 32 == 0 && a.head_dim <= 128 && a.page_tokens >= 4 && page_shift(a.page_tokens) >= 0 && group <= 32 && a.q_start != nullptr &&
+    // a scale that is not positive goes to the plain kernel: the prompt kernel takes the maximum before scaling
+    return a.scale > 0.f && a.head_dim % 32 == 0 && a.head_dim <= 128 && a.page_tokens >= 4 && page_shift(a.page_tokens) >= 0 && group <= 32 && a.q_start != nullptr &&
            a.ldq % 8 == 0 && a.ldo % 4 == 0 && a.kv_width % 8 == 0 && a.kv_width * a.page_tokens < (1 << 20) &&
            ((uintptr_t)a.q & 15) == 0 &&
            ((uintptr_t)a.out & 7) == 0 && ((uintptr_t)a.k_cache & 15) == 0 && ((uintptr_t)a.v_cache & 15) == 0;
@@ -575,14 +601,28 @@ static int launch_ndb(const AttnArgs& a, int tiles, int tpt, int cpt, int chunk_
     return 0;
 }
 
+static int attn_cu_count() {
+    static int n = 0;
+    if (n == 0) {
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+            n = 256;
+    }
+    return n;
+}
+
 template <int NDB>
 static int launch_prefill(const AttnArgs& a, int tpt, int cpt) {
     const int tile_tokens = 4 * tpt;
     dim3 grid(a.n_kv_heads, (a.n_tokens + tile_tokens - 1) / tile_tokens + a.n_seqs);
+    // One request: the number of tiles is known here, and with it whether all blocks are resident at once.
+    const int n_tiles = a.n_seqs == 1 ? (a.n_tokens + tile_tokens - 1) / tile_tokens : 0;
+    const int cus = attn_cu_count();
+    const int pair_from = n_tiles * a.n_kv_heads > cus && n_tiles * a.n_kv_heads <= 2 * cus ? cus : 0;
     attn_prefill_kernel<NDB><<<grid, 4 * WAVE, 0, a.stream>>>(
         (const uint16_t*)a.q, a.ldq, (const uint16_t*)a.k_cache, (const uint16_t*)a.v_cache, a.kv_width, a.block_table,
         a.max_blocks, a.token_slot, a.positions, a.q_start, a.n_seqs, (uint16_t*)a.out, a.ldo,
-        page_shift(a.page_tokens), a.window, a.scale * 1.4426950408889634f, tpt, cpt);
+        page_shift(a.page_tokens), a.window, a.scale * 1.4426950408889634f, tpt, cpt, n_tiles, pair_from);
     HFA_LAUNCH_CHECK("attn_prefill");
     return 0;
 }

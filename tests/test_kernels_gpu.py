@@ -327,6 +327,8 @@ def test_paged_attention(ops32, dtype, H, G, D, page, window):
     (28, 4, 128, 16, 0, [700, 90, 333, 64], [100, 90, 17, 1]),           # portions of several prompts beside a decoded token
     (12, 4, 64, 8, 50, [400, 130], [130, 130]),                          # portions longer than the window
     (6, 2, 96, 32, 0, [300], [37]),                                      # pages of 32 tokens
+    (28, 4, 128, 16, 0, [1200], [1200]),                                 # one prompt whose 300 blocks are all resident: long tiles beside short ones
+    (28, 4, 128, 16, 0, [1100], [1000]),                                 # the same for a portion late in a prompt
 ])
 def test_paged_attention_on_matrix_cores(ops16, H, G, D, page, window, lengths, q_lens):
     """bf16 with head_dim a multiple of 32: long contexts (many key blocks, split into chunks when

@@ -21,8 +21,9 @@
 //   M in 33 .. 64    gemm_stream_kernel (gemm_stream.hip) if N is a multiple of 128 and K of 64 and the
 //                    output has fewer than 512 tiles; else gemm_mfma_kernel with tiles of 64 x 128
 //   M > 64           gemm_dma_kernel (below) with tiles of 256 rows, if M wastes few of them and the
-//                    output has 128 tiles of 256 x 256 (or 64, then with K cut in two, or with tiles
-//                    of 256 x 128); else gemm_mfma_kernel with tiles of 128 x 128
+//                    output has 128 tiles of 256 x 256 (tiles of 256 x 192 where those need fewer rounds
+//                    over the CUs; with 64 tiles K is cut in two, or the tiles are 256 x 128); else
+//                    gemm_mfma_kernel with tiles of 128 x 128
 #include <type_traits>
 
 #include "common.h"
@@ -303,12 +304,13 @@ struct DmaCfg {
     static constexpr int PIECES = BK / 8;                    // 16-byte pieces per row
     static constexpr int ROWS_PER_LOAD = WAVE / PIECES;
     static constexpr int STAGE_BYTES = ROWS * BK * 2;
-    static constexpr int LOADS = ROWS / ROWS_PER_LOAD / NW;  // per wave and stage
+    static constexpr int REQUESTS = ROWS / ROWS_PER_LOAD;    // per stage
+    static constexpr int LOADS = (REQUESTS + NW - 1) / NW;   // per wave and stage; past the last one a wave repeats it
     static constexpr int TM = BM / WM, TN = BN / WN;
     static constexpr int FM = TM / 32, FN = TN / 32;
     static constexpr int STEPS = BK / 16;
     static_assert(BK == 32 || BK == 64, "rows of 64 or 128 bytes");
-    static_assert(ROWS % (ROWS_PER_LOAD * NW) == 0 && BM % (ROWS_PER_LOAD * NW) == 0, "rows must spread evenly over the waves");
+    static_assert(ROWS % ROWS_PER_LOAD == 0 && BM % ROWS_PER_LOAD == 0, "a request fills whole rows of one operand");
     static_assert(TM % 32 == 0 && TN % 32 == 0, "wave tiles are made of 32x32x16 products");
     static_assert(FM * FN * STEPS >= LOADS, "at most one request after a matrix instruction");
     __device__ static constexpr int swizzle(int row) { return BK == 64 ? (row & 7) : ((row >> 1) & 3); }
@@ -353,12 +355,15 @@ __global__ __launch_bounds__(WM* WN* WAVE) void gemm_dma_kernel(
     const int kend = kbeg + k_per_split < K ? kbeg + k_per_split : K;
     const uint16_t* a_base = A + (size_t)m0 * lda + kbeg;
     const uint16_t* w_base = W + (size_t)n0 * ldw + kbeg;
+    // When the requests do not divide by the waves, the waves left over repeat the stage's last
+    // request (same bytes to the same place), so that every wave counts the same number of loads.
+    auto request_no = [&](int i) { return i * C::NW + wave < C::REQUESTS ? i * C::NW + wave : C::REQUESTS - 1; };
     uint32_t src[C::LOADS];
 #pragma unroll
     for (int i = 0; i < C::LOADS; i++) {
-        const int r = (i * C::NW + wave) * C::ROWS_PER_LOAD + lane / C::PIECES;
+        const int r = request_no(i) * C::ROWS_PER_LOAD + lane / C::PIECES;
         const int piece = (lane % C::PIECES) ^ C::swizzle(r);
-        if ((i * C::NW + wave) * C::ROWS_PER_LOAD < BM) {
+        if (request_no(i) * C::ROWS_PER_LOAD < BM) {
             const int last = M - 1 - m0;                     // rows past the edge repeat the last one
             src[i] = (uint32_t)(r < last ? r : last) * (uint32_t)lda * 2u + piece * 16;
         } else {
@@ -368,8 +373,8 @@ __global__ __launch_bounds__(WM* WN* WAVE) void gemm_dma_kernel(
     }
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint16_t*)smem;
     auto request = [&](int i, int stage, int t) {            // i is a constant after unrolling
-        const uint32_t dst = lds0 + stage * C::STAGE_BYTES + (i * C::NW + wave) * 1024;
-        const bool is_a = (i * C::NW + wave) * C::ROWS_PER_LOAD < BM;      // uniform over the wave
+        const uint32_t dst = lds0 + stage * C::STAGE_BYTES + request_no(i) * 1024;
+        const bool is_a = request_no(i) * C::ROWS_PER_LOAD < BM;           // uniform over the wave
         const uint16_t* base = (is_a ? a_base : w_base) + (size_t)t * BK;
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(src[i]), "s"(base) : "m0");
     };
@@ -529,7 +534,10 @@ static int launch_dma(const GemmArgs& g, int mode, void* out, int splits, int k_
         case OUT_F32: return launch_dma_cfg<BM, BN, BK, WM, WN, STAGES, OUT_F32>(g, out, splits, k_per_split);
         case OUT_ACC: return launch_dma_cfg<BM, BN, BK, WM, WN, STAGES, OUT_ACC>(g, out, splits, k_per_split);
         case OUT_PARTIAL: return launch_dma_cfg<BM, BN, BK, WM, WN, STAGES, OUT_PARTIAL>(g, out, splits, k_per_split);
-        default: return launch_dma_cfg<BM, BN, BK, WM, WN, STAGES, OUT_SWIGLU>(g, out, splits, k_per_split);
+        default:
+            if constexpr ((BN / WN) % 64 == 0) return launch_dma_cfg<BM, BN, BK, WM, WN, STAGES, OUT_SWIGLU>(g, out, splits, k_per_split);
+            hfa_set_error("gemm_dma: this tile shape cannot pair gate and up columns");
+            return 1;
     }
 }
 
@@ -626,7 +634,15 @@ int gemm_mfma_launch(const GemmArgs& g, void* workspace, size_t workspace_bytes,
     const bool halves = dma_ok && tiles256 < 128 && 2 * tiles256 >= 128 && g.K % 128 == 0 && g.K >= 2048 &&
                         mode != OUT_SWIGLU && workspace != nullptr &&
                         2 * (size_t)g.M * g.N * sizeof(float) <= workspace_bytes;
-    if (dma_ok && tiles256 >= 128)
+    // Tiles of 192 columns do three quarters of the work of 256 (a little less efficiently): they are
+    // taken when they need fewer rounds over the CUs by more than that.
+    const int cus = 256;
+    const int tiles192 = (rows256 / 256) * ((g.N + 191) / 192);
+    const bool narrow = dma_ok && tiles256 >= 128 && mode != OUT_SWIGLU &&
+                        ((tiles192 + cus - 1) / cus) * 80 < ((tiles256 + cus - 1) / cus) * 100;
+    if (narrow)
+        rc = launch_dma<256, 192, 32, 4, 2, 5>(g, kmode, kout, 1, g.K);
+    else if (dma_ok && tiles256 >= 128)
         rc = launch_dma<256, 256, 32, 2, 4, 4>(g, kmode, kout, 1, g.K);
     else if (halves) {
         rc = launch_dma<256, 256, 32, 2, 4, 4>(g, OUT_PARTIAL, workspace, 2, g.K / 2);

@@ -99,11 +99,11 @@ def test_gemm(ops32, adt, wdt, odt, M, N, K):
                                    (2048, 512, 3584), (2048, 4608, 1024), (1000, 8200, 512), (700, 5408, 640),
                                    (2048, 3584, 1024), (1024, 8192, 64), (2048, 3584, 64), (512, 4096, 128), (1800, 3600, 2176),
                                    (64, 4608, 3584), (48, 3584, 18944), (33, 37888, 256), (40, 1024, 8192),
-                                   (150, 4608, 3584), (300, 3584, 4736)])
+                                   (150, 4608, 3584), (300, 3584, 4736), (1900, 4624, 192)])
 def test_gemm_on_matrix_cores(ops16, M, N, K):
     """bf16 x bf16 with K a multiple of 8 runs on the matrix cores (K split for small M; tiles of
     256 rows loaded straight into LDS for long prompts and wide outputs, with edges in M and N
-    and as few as one or two steps of K, K cut in two where the output is narrow; for 33 to 64 rows one stream of tile-and-K units cut
+    and as few as one or two steps of K, K cut in two where the output is narrow, tiles of 192 columns where they fill the CUs better; for 33 to 64 rows one stream of tile-and-K units cut
     evenly over the CUs, with runs shorter and longer than a tile's K; K split also for prompt
     portions of a few hundred rows whose output has few tiles): against fp64 on the rounded operands, against the
     plain kernel on the same operands, in the three output modes, with operands that are views

@@ -99,7 +99,7 @@ def test_gemm(ops32, adt, wdt, odt, M, N, K):
                                    (2048, 512, 3584), (2048, 4608, 1024), (1000, 8200, 512), (700, 5408, 640),
                                    (2048, 3584, 1024), (1024, 8192, 64), (2048, 3584, 64), (512, 4096, 128), (1800, 3600, 2176),
                                    (64, 4608, 3584), (48, 3584, 18944), (33, 37888, 256), (40, 1024, 8192),
-                                   (150, 4608, 3584), (300, 3584, 4736), (1900, 4624, 192)])
+                                   (150, 4608, 3584), (300, 3584, 4736), (1900, 4624, 192), (50, 33024, 320), (64, 65536, 64)])
 def test_gemm_on_matrix_cores(ops16, M, N, K):
     """bf16 x bf16 with K a multiple of 8 runs on the matrix cores (K split for small M; tiles of
     256 rows loaded straight into LDS for long prompts and wide outputs, with edges in M and N
@@ -137,7 +137,7 @@ def test_gemm_on_matrix_cores(ops16, M, N, K):
 
 
 @pytest.mark.parametrize("M,E,F", [(1, 256, 352), (8, 256, 352), (64, 256, 352), (100, 256, 352), (300, 256, 352),
-                                   (1500, 192, 16416), (600, 320, 4512)])
+                                   (1500, 192, 16416), (600, 320, 4512), (48, 192, 16512), (64, 128, 18944)])
 def test_gemm_with_gate_up_epilogue(ops16, M, E, F):
     """Gate and up rows interleaved in blocks of 32; the product's last step forms silu(gate) * up:
     directly in the tile's epilogue (large M) or when the split K is added up (small M)."""

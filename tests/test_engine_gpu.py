@@ -65,6 +65,21 @@ def test_cuttings_agree_with_each_other(gpu, tiny, dtype):
             assert err <= tol, f"{name} {dtype}: {key}: cuttings differ by {err:.3e}"
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_the_same_trace_twice_gives_the_same_bits(gpu, tiny, dtype):
+    """No kernel adds with atomics or in an order that depends on timing: a mixed trace replayed
+    in a second engine gives the same logits bit for bit."""
+    name, cfg, d, reqs, _ = tiny
+    steps = helpers.trace_mixed(reqs, seed=11)
+    runs = []
+    for _ in range(2):
+        engine = engine_for(d, dtype, name, helpers.max_live_tokens(steps))
+        runs.append(helpers.run_trace_in_engine(engine, steps))
+    assert runs[0].keys() == runs[1].keys()
+    for key, row in runs[0].items():
+        assert np.array_equal(row, runs[1][key]), f"{name} {dtype}: {key} differs between two runs"
+
+
 def test_window_edge_shows(gpu, tmp_path):
     """Config B with one key made to stand out: a query far beyond the window must not see
     it in the windowed layers, one inside the window must. The plain implementation decides;

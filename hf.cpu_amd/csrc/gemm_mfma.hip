@@ -294,9 +294,11 @@ __global__ __launch_bounds__(WM* WN* WAVE) void gemm_mfma_kernel(
 //
 // LDS rows have no padding (the hardware places the 64 lanes' 16 bytes back to back); instead the
 // 16-byte pieces of a row are stored in swizzled order, which a lane arranges by which piece it
-// asks for: with rows of 128 bytes, piece p of row r lies at p ^ (r % 8); with rows of 64 bytes,
-// at p ^ ((r / 2) % 4). Eight lanes that read the same piece of eight consecutive rows then hit
-// eight different groups of banks.
+// asks for: with rows of 128 bytes, piece p of row r lies at p ^ ((r / 2) % 8); with rows of 64
+// bytes, at p ^ ((r / 4) % 4). A 16-byte read is served 16 lanes a cycle (all 64 banks): sixteen
+// lanes that read the same piece of sixteen consecutive rows then hit sixteen different groups
+// of four banks (with a swizzle that only tells eight rows apart, SQ_LDS_BANK_CONFLICT counts
+// four more cycles for every read).
 template <int BM, int BN, int BK, int WM, int WN>
 struct DmaCfg {
     static constexpr int NW = WM * WN, NT = NW * WAVE;
@@ -313,7 +315,7 @@ struct DmaCfg {
     static_assert(ROWS % ROWS_PER_LOAD == 0 && BM % ROWS_PER_LOAD == 0, "a request fills whole rows of one operand");
     static_assert(TM % 32 == 0 && TN % 32 == 0, "wave tiles are made of 32x32x16 products");
     static_assert(FM * FN * STEPS >= LOADS, "at most one request after a matrix instruction");
-    __device__ static constexpr int swizzle(int row) { return BK == 64 ? (row & 7) : ((row >> 1) & 3); }
+    __device__ static constexpr int swizzle(int row) { return BK == 64 ? ((row >> 1) & 7) : ((row >> 2) & 3); }
 };
 
 template <int BM, int BN, int BK, int WM, int WN, int STAGES, int MODE>

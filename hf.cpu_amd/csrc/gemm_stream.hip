@@ -67,12 +67,12 @@ __global__ __launch_bounds__(WM* WN* WAVE) void gemm_stream_kernel(
     // Request i of this wave fills rows (i * NW + wave) * 8 .. + 8 of a stage: rows 0 .. BM - 1 are
     // A's (rows past M repeat the last one), the others W's rows of the unit's column tile. This
     // lane supplies row lane / 8 of the eight, the 16-byte piece stored at lane % 8, which is
-    // piece (lane % 8) ^ (row % 8) of the row (see the swizzle in gemm_mfma.hip).
+    // piece (lane % 8) ^ ((row / 2) % 8) of the row (see the swizzle in gemm_mfma.hip).
     uint32_t src[C::LOADS];
 #pragma unroll
     for (int i = 0; i < C::LOADS; i++) {
         const int r = (i * C::NW + wave) * 8 + lane / 8;
-        const int piece = (lane % 8) ^ (r & 7);
+        const int piece = (lane % 8) ^ ((r >> 1) & 7);
         if ((i * C::NW + wave) * 8 < BM)
             src[i] = (uint32_t)(r < M - 1 ? r : M - 1) * (uint32_t)lda * 2u + piece * 16;
         else
@@ -91,7 +91,7 @@ __global__ __launch_bounds__(WM* WN* WAVE) void gemm_stream_kernel(
     };
     int piece_off[C::STEPS];
 #pragma unroll
-    for (int j = 0; j < C::STEPS; j++) piece_off[j] = ((2 * j + (lane >> 5)) ^ (lane & 7)) * 8;
+    for (int j = 0; j < C::STEPS; j++) piece_off[j] = ((2 * j + (lane >> 5)) ^ ((lane >> 1) & 7)) * 8;
     auto fragments = [&](int stage, int j, bf16x8 (&fa)[C::FM], bf16x8 (&fw)[C::FN]) {
         const uint16_t* sa = smem + stage * (C::STAGE_BYTES / 2) + (wm * C::TM + (lane & 31)) * C::BK + piece_off[j];
         const uint16_t* sw = smem + stage * (C::STAGE_BYTES / 2) + (BM + wn * C::TN + (lane & 31)) * C::BK + piece_off[j];

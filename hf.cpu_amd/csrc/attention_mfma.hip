@@ -33,6 +33,19 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 // never subnormal results that matter), and the bf16 bits of a probability in [0, 1]: round to
 // nearest even without the NaN case.
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+// A column's scores lie in lanes c and c + 32. v_permlane32_swap exchanges the upper half of one
+// register with the lower half of another; with the same value in both, every lane then holds
+// the lower lane's value in the first and the upper lane's in the second: maximum and sum of the
+// pair without a trip through LDS, and the same bits in both lanes.
+__device__ __forceinline__ float pair_max(float x) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float pair_sum(float x) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
 // Two probabilities as a pair of bf16, round to nearest even: one v_cvt_pk_bf16_f32 on gfx950.
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float floatx2 __attribute__((ext_vector_type(2)));
@@ -171,7 +184,7 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
             st[r] = vis ? st[r] * scale_log2e : NEG_BIG;
             mx = fmaxf(mx, st[r]);
         }
-        mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+        mx = pair_max(mx);
         const float mn = fmaxf(m, mx);
         const float corr = fast_exp2(m - mn);
         float psum = 0.f;
@@ -181,7 +194,7 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
             st[r] = p;
             psum += p;
         }
-        psum += __shfl_xor(psum, 32, WAVE);
+        psum = pair_sum(psum);
         l = l * corr + psum;
         m = mn;
         // the running maxima settle after a few blocks; the accumulators are rescaled only when
@@ -456,7 +469,7 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
                 if (inside) {                                   // the scale (positive) moves into the exponent's fma
 #pragma unroll
                     for (int r = 0; r < 16; r++) mx = fmaxf(mx, st[r]);
-                    mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE)) * scale_log2e;
+                    mx = pair_max(mx) * scale_log2e;
                     mn = fmaxf(m, mx);
                     corr = fast_exp2(m - mn);
 #pragma unroll
@@ -472,7 +485,7 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
                         st[r] = vis ? st[r] * scale_log2e : NEG_BIG;
                         mx = fmaxf(mx, st[r]);
                     }
-                    mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+                    mx = pair_max(mx);
                     mn = fmaxf(m, mx);
                     corr = fast_exp2(m - mn);
 #pragma unroll
@@ -482,7 +495,7 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
                         psum += p;
                     }
                 }
-                psum += __shfl_xor(psum, 32, WAVE);
+                psum = pair_sum(psum);
                 l = l * corr + psum;
                 m = mn;
                 if (__any(corr != 1.0f)) {                      // see above: only when a maximum moved

@@ -187,10 +187,11 @@ __global__ __launch_bounds__(WM* WN* WAVE) void gemm_mfma_kernel(
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
-    // PF = 2 (small M, bandwidth-bound): two register sets, so that while tile t is multiplied out
-    // of LDS, tiles t + 1 and t + 2 are on their way from memory, which doubles the bytes in flight
-    // of a block. PF = 1 (large M): one set, fewer registers, more blocks per CU.
-    uint4 ra0[C::A_CH], rw0[C::W_CH], ra1[PF == 2 ? C::A_CH : 1], rw1[PF == 2 ? C::W_CH : 1];
+    // PF register sets of loads: while tile t is multiplied out of LDS, tiles t + 1 .. t + PF are on
+    // their way from memory. PF = 1 (large M): few registers, more blocks per CU. PF = 2 (small M,
+    // bound by the weights' stream): twice the bytes in flight of a block; four sets stream no faster.
+    static_assert(PF == 1 || PF % 2 == 0, "the stage of a tile is known at compile time");
+    uint4 ra[PF][C::A_CH], rw[PF][C::W_CH];
     auto gload = [&](uint4* ra, uint4* rw, int k0) {
 #pragma unroll
         for (int i = 0; i < C::A_CH; i++) {
@@ -240,33 +241,32 @@ __global__ __launch_bounds__(WM* WN* WAVE) void gemm_mfma_kernel(
     };
 
     const int nk = (kend - kbeg + BK - 1) / BK;
-    gload(ra0, rw0, kbeg);
-    sstore(0, ra0, rw0);
-    if (nk > 1) gload(ra0, rw0, kbeg + BK);
-    if (PF == 2 && nk > 2) gload(ra1, rw1, kbeg + 2 * BK);
+    gload(ra[0], rw[0], kbeg);
+    sstore(0, ra[0], rw[0]);
+#pragma unroll
+    for (int p = 1; p <= PF; p++)                            // tile p waits in set p % PF
+        if (p < nk) gload(ra[p % PF], rw[p % PF], kbeg + p * BK);
     __syncthreads();
     if (PF == 1) {
         for (int t = 0; t < nk; t++) {
             compute(t & 1);
-            if (t + 1 < nk) sstore((t + 1) & 1, ra0, rw0);
-            if (t + 2 < nk) gload(ra0, rw0, kbeg + (t + 2) * BK);
+            if (t + 1 < nk) sstore((t + 1) & 1, ra[0], rw[0]);
+            if (t + 2 < nk) gload(ra[0], rw[0], kbeg + (t + 2) * BK);
             __syncthreads();
         }
     }
-    for (int t = 0; PF == 2 && t < nk; t += 2) {
-        compute(0);                                          // tile t
-        if (t + 1 < nk) {
-            sstore(1, ra0, rw0);                             // tile t + 1
-            if (t + 3 < nk) gload(ra0, rw0, kbeg + (t + 3) * BK);
+    for (int t0 = 0; PF > 1 && t0 < nk; t0 += PF) {
+#pragma unroll
+        for (int p = 0; p < PF; p++) {                       // tile t0 + p: its stage and the sets are constants here
+            const int t = t0 + p;
+            if (t >= nk) break;
+            compute(p & 1);
+            if (t + 1 < nk) {
+                sstore((p + 1) & 1, ra[(p + 1) % PF], rw[(p + 1) % PF]);
+                if (t + 1 + PF < nk) gload(ra[(p + 1) % PF], rw[(p + 1) % PF], kbeg + (t + 1 + PF) * BK);
+            }
+            __syncthreads();
         }
-        __syncthreads();
-        if (t + 1 >= nk) break;
-        compute(1);                                          // tile t + 1
-        if (t + 2 < nk) {
-            sstore(0, ra1, rw1);                             // tile t + 2
-            if (t + 4 < nk) gload(ra1, rw1, kbeg + (t + 4) * BK);
-        }
-        __syncthreads();
     }
 
     if constexpr (MODE == OUT_BF16 || MODE == OUT_SWIGLU) {

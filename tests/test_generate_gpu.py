@@ -222,6 +222,52 @@ def test_trace_run_program(gpu, models, tmp_path):
     assert bad.returncode == 1 and "ERANGE" in bad.stderr
 
 
+def test_trace_run_odd_but_legal_steps(gpu, models, tmp_path):
+    """Steps a trace may hold beyond the usual: a request of one token, wanted places out of order
+    and twice, a request that sits out several steps, a step that only ends requests, an id that
+    comes back as a new request after it ended, four requests that fill the pool to the last page."""
+    cfg = helpers.CONFIG_A
+    reqs = helpers.random_requests(cfg, [1, 64, 64, 63, 30], seed=21)
+    a, b, c, d, e = (reqs[f"r{i}"] for i in range(5))
+    st = helpers._step
+    steps = [
+        st(0, [("a", a, [0]), ("b", b[:40], [39, 0, 39])]),
+        st(1, [("c", c[:2], [1]), ("d", d[:61], [])]),
+        st(2, [("b", b[40:63], [22]), ("c", c[2:33], [30, 0])]),
+        st(3, [("d", d[61:], [1, 0])], ["a"]),
+        st(4, [], ["d"]),
+        st(5, [("a", e[:29], [28]), ("c", c[33:], range(31))]),         # the id "a" again: a new request
+        st(6, [("b", b[63:], [0]), ("a", e[29:], [0])], ["a", "b", "c"]),
+    ]
+    want = helpers.plain_logits(models["A"], reqs)
+    name_of = {0: {"a": "r0", "b": "r1", "c": "r2", "d": "r3"}, 5: {"a": "r4", "b": "r1", "c": "r2", "d": "r3"}}
+    for dtype, tol in (("float32", 5e-6), ("bfloat16", 2e-2)):
+        out = tmp_path / dtype
+        r = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", models["A"], "--dtype", dtype,
+                            "--out", str(out), "--max-tokens", "256"],
+                           input="".join(json.dumps(s) + "\n" for s in steps), text=True, capture_output=True, timeout=300)
+        assert r.returncode == 0, r.stderr
+        assert r.stdout.split() == [w for s in steps for w in ("done", str(s["step"]))]
+        assert not (out / "4.f32").exists()
+        at, names, got = {}, name_of[0], {}
+        for s in steps:
+            if s["step"] == 5:
+                names, at["a"] = name_of[5], 0
+            rows = []
+            for en in s["entries"]:
+                base = at.get(en["id"], 0)
+                rows += [(names[en["id"]], base + w) for w in en["want"]]
+                at[en["id"]] = base + len(en["tokens"])
+            if rows:
+                data = np.fromfile(out / f"{s['step']}.f32", dtype="<f4").reshape(len(rows), -1)
+                for key, row in zip(rows, data):
+                    scale = float(np.max(np.abs(want[key[0]])))
+                    err = float(np.max(np.abs(row - want[key[0]][key[1]])))
+                    assert err <= tol * scale, f"{dtype} step {s['step']} {key}: {err:.3e}"
+                    got[key] = True
+        assert ("r4", 29) in got and ("r1", 63) in got and ("r0", 0) in got
+
+
 def test_generation_survives_a_cache_that_is_too_small(gpu, models):
     """Six requests that together need about twice the pages there are: the scheduler shrinks
     prompt portions, preempts the newest running request when decoded tokens no longer fit, and

@@ -242,10 +242,11 @@ __global__ __launch_bounds__(WM* WN* WAVE) void gemm_mfma_kernel(
 
     const int nk = (kend - kbeg + BK - 1) / BK;
     gload(ra[0], rw[0], kbeg);
-    sstore(0, ra[0], rw[0]);
 #pragma unroll
-    for (int p = 1; p <= PF; p++)                            // tile p waits in set p % PF
-        if (p < nk) gload(ra[p % PF], rw[p % PF], kbeg + p * BK);
+    for (int p = 1; p < PF; p++)                             // tile p waits in set p % PF; all are asked for
+        if (p < nk) gload(ra[p], rw[p], kbeg + p * BK);      // before the first one is waited for
+    sstore(0, ra[0], rw[0]);
+    if (PF < nk) gload(ra[0], rw[0], kbeg + PF * BK);
     __syncthreads();
     if (PF == 1) {
         for (int t = 0; t < nk; t++) {

@@ -363,13 +363,13 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
     const int vhi = col_ok ? pos : -1;
     const int* bt = block_table + (size_t)token_slot[t0] * max_blocks;
 
-    // query fragments in LDS, each lane reading back what it wrote (ordered by the barrier below)
-    __shared__ uint4 q_s[4][KS * WAVE];
+    // query fragments stay in registers for the whole tile
+    Frag qf[KS];
     {
         const uint16_t* qp = q + (size_t)my_tok * ldq + my_head * D + half * 8;
 #pragma unroll
         for (int ks = 0; ks < KS; ks++)
-            q_s[wave][ks * WAVE + lane] = col_ok ? *reinterpret_cast<const uint4*>(qp + ks * 16) : make_uint4(0, 0, 0, 0);
+            qf[ks].u = col_ok ? *reinterpret_cast<const uint4*>(qp + ks * 16) : make_uint4(0, 0, 0, 0);
     }
     floatx16 o[NDB];
 #pragma unroll
@@ -455,13 +455,26 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
                 floatx16 st;
 #pragma unroll
                 for (int r = 0; r < 16; r++) st[r] = 0.f;
+                // All fragment reads of the block are asked for before the first product: left to itself
+                // the compiler reads one fragment, waits for it and multiplies, sixteen LDS round trips
+                // a block. The values' first half arrives while the softmax is computed.
+                Frag kf[KS], vf[2][NDB];
 #pragma unroll
-                for (int ks = 0; ks < KS; ks++) {
-                    Frag kf, qf;
-                    kf.u = *reinterpret_cast<const uint4*>(ks_ + ks * 16);
-                    qf.u = q_s[wave][ks * WAVE + lane];
-                    st = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf.v, qf.v, st, 0, 0, 0);
-                }
+                for (int ks = 0; ks < KS; ks++) kf[ks].u = *reinterpret_cast<const uint4*>(ks_ + ks * 16);
+                auto vread = [&](int kk) {
+#pragma unroll
+                    for (int db = 0; db < NDB; db++) {
+                        const uint16_t* vs_ = &v_s[stage][(32 * db + col) * PVS + 16 * kk + 4 * half];
+                        vf[kk][db].h[0] = *reinterpret_cast<const uint2*>(vs_);
+                        vf[kk][db].h[1] = *reinterpret_cast<const uint2*>(vs_ + 8);
+                    }
+                };
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int ks = 0; ks < KS; ks++)
+                    st = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ks].v, qf[ks].v, st, 0, 0, 0);
+                vread(0);
+                __builtin_amdgcn_sched_barrier(0);
                 // Most blocks lie wholly inside what every column of the wave may see (unused columns
                 // aside, whose results are dropped): no key of them needs the visibility test.
                 const bool inside = __all(!col_ok || (key0 >= vlo && key0 + KB - 1 <= vhi)) != 0;
@@ -513,16 +526,13 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
                         w[e] = prob_pair(st[8 * kk + 2 * e], st[8 * kk + 2 * e + 1]);
                     pf[kk].u = make_uint4(w[0], w[1], w[2], w[3]);
                 }
+                vread(1);
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int kk = 0; kk < 2; kk++)
 #pragma unroll
-                    for (int db = 0; db < NDB; db++) {
-                        const uint16_t* vs_ = &v_s[stage][(32 * db + col) * PVS + 16 * kk + 4 * half];
-                        Frag vf;
-                        vf.h[0] = *reinterpret_cast<const uint2*>(vs_);
-                        vf.h[1] = *reinterpret_cast<const uint2*>(vs_ + 8);
-                        o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf.v, pf[kk].v, o[db], 0, 0, 0);
-                    }
+                    for (int db = 0; db < NDB; db++)
+                        o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[kk][db].v, pf[kk].v, o[db], 0, 0, 0);
             }
         };
         for (int b = wb; b < we; b += 2) {

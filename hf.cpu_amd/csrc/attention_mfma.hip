@@ -301,6 +301,10 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
 // waves, so L2-to-CU traffic drops fourfold against the kernel above and several waves per SIMD
 // overlap their matrix products and softmax. Two LDS stages, one barrier per key block. Tiles
 // are numbered from the end of each request backwards, so the longest ones start first.
+// The running maximum of a column follows the scores only when they pass it by more than this (in
+// powers of two): probabilities then reach 2^MAX_SLACK at most, which bf16 and the fp32 sums hold
+// as exactly as values up to 1, and the accumulators are rescaled in few blocks instead of in most.
+#define MAX_SLACK 8.0f
 #define PKS 136      // LDS row of a key: 128 dims + 8 pad (elements)
 #define PVS 36       // LDS row of a value dimension: 32 keys + 4 pad (elements)
 
@@ -483,7 +487,7 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
 #pragma unroll
                     for (int r = 0; r < 16; r++) mx = fmaxf(mx, st[r]);
                     mx = pair_max(mx) * scale_log2e;
-                    mn = fmaxf(m, mx);
+                    mn = mx > m + MAX_SLACK ? mx : m;
                     corr = fast_exp2(m - mn);
 #pragma unroll
                     for (int r = 0; r < 16; r++) {
@@ -499,7 +503,7 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
                         mx = fmaxf(mx, st[r]);
                     }
                     mx = pair_max(mx);
-                    mn = fmaxf(m, mx);
+                    mn = mx > m + MAX_SLACK ? mx : m;
                     corr = fast_exp2(m - mn);
 #pragma unroll
                     for (int r = 0; r < 16; r++) {

@@ -207,12 +207,14 @@ class Engine:
     def _run(self, step, logits):
         """The forward pass of the step, eagerly or as a replay of the graph of its shape."""
         decode_only = step.max_q_len == 1 and step.n_tokens <= self.GRAPH_MAX_TOKENS
+        if decode_only:
+            # The kernels use max_seq_len only to choose how the key range is cut, so a graph
+            # captured for a length bucket serves every shorter length too. Steps that run eagerly
+            # take the same bucket: a replay and an eager run of a step give the same bits.
+            B = self.GRAPH_LEN_BUCKET
+            step.max_seq_len = min(-(-step.max_seq_len // B) * B, self.manager.max_context)
         if not (self.use_graphs and decode_only) or self.profile is not None:
             return self.model.forward(self.ops, step, self.storage.views, logits)
-        # The kernels use max_seq_len only to choose how the key range is cut, so a graph
-        # captured for a length bucket serves every shorter length too.
-        B = self.GRAPH_LEN_BUCKET
-        step.max_seq_len = min(-(-step.max_seq_len // B) * B, self.manager.max_context)
         key = (step.n_tokens, step.n_logit_rows, step.max_seq_len)
         stamp = (self.ops.scratch_generation, self.staging.generation)
         hit = self._graphs.get(key)

@@ -29,9 +29,13 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 #define PG_MAX 512
 #define NEG_BIG (-1.0e30f)
 
-// 2^x by the hardware instruction (arguments here are <= 0 or the -1e30 sentinel's difference,
-// never subnormal results that matter), and the bf16 bits of a probability in [0, 1]: round to
-// nearest even without the NaN case.
+// The running maximum of a column follows the scores only when they pass it by more than this (in
+// powers of two): probabilities then reach 2^MAX_SLACK at most, which bf16 and the fp32 sums hold
+// as exactly as values up to 1, and the accumulators are rescaled in few blocks instead of in most.
+#define MAX_SLACK 8.0f
+
+// 2^x by the hardware instruction (arguments here are at most MAX_SLACK or the -1e30 sentinel's
+// difference, never subnormal results that matter).
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 // A column's scores lie in lanes c and c + 32. v_permlane32_swap exchanges the upper half of one
 // register with the lower half of another; with the same value in both, every lane then holds
@@ -175,24 +179,40 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
             qf.u = q_s[ks * WAVE + lane];
             st = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ks].v, qf.v, st, 0, 0, 0);
         }
-        // element r of the lane: key key0 + 8 (r / 4) + 4 half + r % 4, this lane's column
-        float mx = NEG_BIG;
+        // element r of the lane: key key0 + 8 (r / 4) + 4 half + r % 4, this lane's column.
+        // Most blocks lie wholly inside what every column of the wave may see (unused columns
+        // aside, whose results are dropped): no key of them needs the visibility test, and the
+        // scale (positive) moves into the exponent's fma.
+        const bool inside = __all(!col_ok || (key0 >= vlo && key0 + KB - 1 <= vhi)) != 0;
+        float mx = NEG_BIG, mn, corr, psum = 0.f;
+        if (inside) {
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-            const int kr = key0 + 8 * (r / 4) + 4 * half + (r % 4);
-            const bool vis = kr >= vlo && kr <= vhi;
-            st[r] = vis ? st[r] * scale_log2e : NEG_BIG;
-            mx = fmaxf(mx, st[r]);
-        }
-        mx = pair_max(mx);
-        const float mn = fmaxf(m, mx);
-        const float corr = fast_exp2(m - mn);
-        float psum = 0.f;
+            for (int r = 0; r < 16; r++) mx = fmaxf(mx, st[r]);
+            mx = pair_max(mx) * scale_log2e;
+            mn = mx > m + MAX_SLACK ? mx : m;
+            corr = fast_exp2(m - mn);
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-            const float p = st[r] > 0.5f * NEG_BIG ? fast_exp2(st[r] - mn) : 0.f;
-            st[r] = p;
-            psum += p;
+            for (int r = 0; r < 16; r++) {
+                st[r] = fast_exp2(fmaf(st[r], scale_log2e, -mn));
+                psum += st[r];
+            }
+        } else {
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int kr = key0 + 8 * (r / 4) + 4 * half + (r % 4);
+                const bool vis = kr >= vlo && kr <= vhi;
+                st[r] = vis ? st[r] * scale_log2e : NEG_BIG;
+                mx = fmaxf(mx, st[r]);
+            }
+            mx = pair_max(mx);
+            mn = mx > m + MAX_SLACK ? mx : m;
+            corr = fast_exp2(m - mn);
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const float p = st[r] > 0.5f * NEG_BIG ? fast_exp2(st[r] - mn) : 0.f;
+                st[r] = p;
+                psum += p;
+            }
         }
         psum = pair_sum(psum);
         l = l * corr + psum;
@@ -301,10 +321,6 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
 // waves, so L2-to-CU traffic drops fourfold against the kernel above and several waves per SIMD
 // overlap their matrix products and softmax. Two LDS stages, one barrier per key block. Tiles
 // are numbered from the end of each request backwards, so the longest ones start first.
-// The running maximum of a column follows the scores only when they pass it by more than this (in
-// powers of two): probabilities then reach 2^MAX_SLACK at most, which bf16 and the fp32 sums hold
-// as exactly as values up to 1, and the accumulators are rescaled in few blocks instead of in most.
-#define MAX_SLACK 8.0f
 #define PKS 136      // LDS row of a key: 128 dims + 8 pad (elements)
 #define PVS 36       // LDS row of a value dimension: 32 keys + 4 pad (elements)
 

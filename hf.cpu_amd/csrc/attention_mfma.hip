@@ -113,16 +113,15 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
     int vhi = col_ok ? (pos < k_end ? pos : k_end) : -1;
     const int* bt = block_table + (size_t)token_slot[t0] * max_blocks;
 
-    // The query fragments live in LDS (each lane reads back what it wrote): registers are
-    // needed for the keys and values in flight.
-    __shared__ uint4 q_s[KS * WAVE];
+    // The query fragments stay in registers: read from LDS one by one before each product, they
+    // cost an LDS round trip a product that a single wave on its SIMD has nothing to hide behind.
+    Frag qf[KS];
     {
         const uint16_t* qp = q + (size_t)my_tok * ldq + my_head * D + half * 8;
 #pragma unroll
         for (int ks = 0; ks < KS; ks++)
-            q_s[ks * WAVE + lane] = col_ok ? *reinterpret_cast<const uint4*>(qp + ks * 16) : make_uint4(0, 0, 0, 0);
+            qf[ks].u = col_ok ? *reinterpret_cast<const uint4*>(qp + ks * 16) : make_uint4(0, 0, 0, 0);
     }
-    __syncthreads();
     floatx16 o[NDB];
 #pragma unroll
     for (int db = 0; db < NDB; db++)
@@ -174,11 +173,8 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
 #pragma unroll
         for (int r = 0; r < 16; r++) st[r] = 0.f;
 #pragma unroll
-        for (int ks = 0; ks < KS; ks++) {
-            Frag qf;
-            qf.u = q_s[ks * WAVE + lane];
-            st = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ks].v, qf.v, st, 0, 0, 0);
-        }
+        for (int ks = 0; ks < KS; ks++)
+            st = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ks].v, qf[ks].v, st, 0, 0, 0);
         // element r of the lane: key key0 + 8 (r / 4) + 4 half + r % 4, this lane's column.
         // Most blocks lie wholly inside what every column of the wave may see (unused columns
         // aside, whose results are dropped): no key of them needs the visibility test, and the

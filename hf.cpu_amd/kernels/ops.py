@@ -13,6 +13,7 @@ dtypes and layout on the host, hands raw pointers to the library on the current
 stream, and raises EngineError if the library refuses the call. Nothing here
 computes with a library routine or on the CPU.
 """
+import contextlib
 import ctypes
 from dataclasses import dataclass
 
@@ -24,6 +25,7 @@ from .lib import last_error, library
 F32, BF16 = 0, 1
 WORKSPACE_BYTES = 64 << 20           # partial sums of matrix products whose K is split
 _CODE = {torch.float32: F32, torch.bfloat16: BF16}
+_ELEMENT_BYTES = {torch.float32: 4, torch.bfloat16: 2, torch.float16: 2, torch.int32: 4, torch.int64: 8, torch.uint8: 1}
 
 
 def _code(t):
@@ -94,6 +96,8 @@ class Ops:
         self.act_dtype = act_dtype
         self.lib = library()
         self._scratch = {}
+        self._scratch_views = {}             # (name, shape, dtype) -> the view handed out last time
+        self._stream_handle = None
         self.scratch_generation = 0
         self.workspace = torch.empty(WORKSPACE_BYTES, dtype=torch.uint8, device=self.device)
         self.attn_workspace = torch.empty(WORKSPACE_BYTES, dtype=torch.uint8, device=self.device)
@@ -124,7 +128,19 @@ class Ops:
 
     # ---- plumbing ----------------------------------------------------------
     def _stream(self):
-        return torch.cuda.current_stream(self.device).cuda_stream
+        s = self._stream_handle
+        return s if s is not None else torch.cuda.current_stream(self.device).cuda_stream
+
+    @contextlib.contextmanager
+    def on_current_stream(self):
+        """Inside, every kernel goes to the stream that is current on entry: asked for once
+        instead of once per kernel (a forward pass enqueues hundreds)."""
+        before = self._stream_handle
+        self._stream_handle = torch.cuda.current_stream(self.device).cuda_stream
+        try:
+            yield self
+        finally:
+            self._stream_handle = before
 
     def _check(self, rc):
         if rc != 0:
@@ -133,10 +149,14 @@ class Ops:
     def scratch(self, name, shape, dtype):
         """A named work buffer that is reused from step to step; its contents are
         undefined on return. The same name always aliases the same memory."""
+        key = (name, tuple(shape), dtype)
+        view = self._scratch_views.get(key)
+        if view is not None:
+            return view
         n = 1
         for s in shape:
             n *= int(s)
-        nbytes = max(n, 1) * torch.empty((), dtype=dtype).element_size()
+        nbytes = max(n, 1) * _ELEMENT_BYTES[dtype]
         buf = self._scratch.get(name)
         if buf is None or buf.numel() < nbytes:
             if torch.cuda.is_current_stream_capturing():
@@ -144,7 +164,11 @@ class Ops:
             buf = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=self.device)
             self._scratch[name] = buf
             self.scratch_generation += 1          # captured graphs hold the old address
-        return buf[:nbytes].view(dtype).view(*shape)
+            self._scratch_views = {k: v for k, v in self._scratch_views.items() if k[0] != name}
+        view = buf[:nbytes].view(dtype).view(*shape)
+        if len(self._scratch_views) < 4096:
+            self._scratch_views[key] = view
+        return view
 
     # ---- kernels -----------------------------------------------------------
     def embed(self, table, tokens, out_x):

@@ -126,7 +126,7 @@ class Model:
         """Runs ``step``'s tokens through the schedule. ``caches[i]`` is the cache view
         of schedule entry ``i`` (None if it needs none). Writes fp32 logits for
         ``step.logit_rows`` into ``logits_out`` ([R, V]; R may be 0)."""
-        with ops.section("total"):
+        with ops.on_current_stream(), ops.section("total"):
             self._forward(ops, step, caches, logits_out)
 
     def _forward(self, ops, step, caches, logits_out):

@@ -578,31 +578,65 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
 }
 
 // out[t, h, :] = sum_c o_c 2^(m_c - M) / sum_c l_c 2^(m_c - M), chunks in ascending order.
-// Lanes first share the chunks (maximum, weights, sum), then the dimensions; the loads of the
-// second loop do not depend on one another.
+// One wave per (token, head). The kernel is a chain of memory round trips and little else, so it
+// is written to have few of them: the first MERGE_GROUP chunks' outputs are asked for before
+// anything else, a lane reads maximum and sum of "its" chunk as one pair, and the rest of the
+// outputs come MERGE_GROUP loads at a time. A lane owns two neighbouring dimensions (D <= 128).
 #define MERGE_MAX_CHUNKS 512
+#define MERGE_GROUP 16
 __global__ __launch_bounds__(WAVE) void attn_merge_kernel(const float* __restrict__ partial, uint16_t* __restrict__ out,
                                                           int ldo, int H, int D, int n_chunks) {
     __shared__ float w_s[MERGE_MAX_CHUNKS];
     const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-    const float* src = partial + (size_t)(t * H + h) * n_chunks * (D + 2);
-    float M = NEG_BIG;
-    for (int c = lane; c < n_chunks; c += WAVE) M = fmaxf(M, src[(size_t)c * (D + 2)]);
+    const size_t row = D + 2;
+    const float* src = partial + (size_t)(t * H + h) * n_chunks * row;
+    const bool has = 2 * lane < D;
+    const float* mine = src + 2 + 2 * lane;
+    float2 pre[MERGE_GROUP];
+#pragma unroll
+    for (int i = 0; i < MERGE_GROUP; i++)
+        pre[i] = has && i < n_chunks ? *reinterpret_cast<const float2*>(mine + i * row) : make_float2(0.f, 0.f);
+    const float2 ml0 = lane < n_chunks ? *reinterpret_cast<const float2*>(src + lane * row) : make_float2(NEG_BIG, 0.f);
+    float M = ml0.x;
+    for (int c = lane + WAVE; c < n_chunks; c += WAVE) M = fmaxf(M, src[c * row]);
     M = wave_max(M);
     float L = 0.f;
-    for (int c = lane; c < n_chunks; c += WAVE) {
-        const float w = exp2f(src[(size_t)c * (D + 2)] - M);
+    if (lane < n_chunks) {
+        const float w = exp2f(ml0.x - M);
+        w_s[lane] = w;
+        L = ml0.y * w;
+    }
+    for (int c = lane + WAVE; c < n_chunks; c += WAVE) {
+        const float2 ml = *reinterpret_cast<const float2*>(src + c * row);
+        const float w = exp2f(ml.x - M);
         w_s[c] = w;
-        L += src[(size_t)c * (D + 2) + 1] * w;
+        L += ml.y * w;
     }
     L = wave_sum(L);
     __syncthreads();
-    const float inv = 1.0f / L;
-    for (int d = lane; d < D; d += WAVE) {
-        float acc = 0.f;
-        for (int c = 0; c < n_chunks; c++) acc = fmaf(src[(size_t)c * (D + 2) + 2 + d], w_s[c], acc);
-        out[(size_t)t * ldo + h * D + d] = bf16_bits(acc * inv);
+    if (!has) return;
+    float ax = 0.f, ay = 0.f;
+#pragma unroll
+    for (int i = 0; i < MERGE_GROUP; i++)
+        if (i < n_chunks) {
+            ax = fmaf(pre[i].x, w_s[i], ax);
+            ay = fmaf(pre[i].y, w_s[i], ay);
+        }
+    for (int c0 = MERGE_GROUP; c0 < n_chunks; c0 += MERGE_GROUP) {
+        float2 v[MERGE_GROUP];
+#pragma unroll
+        for (int i = 0; i < MERGE_GROUP; i++)
+            v[i] = c0 + i < n_chunks ? *reinterpret_cast<const float2*>(mine + (c0 + i) * row) : make_float2(0.f, 0.f);
+#pragma unroll
+        for (int i = 0; i < MERGE_GROUP; i++)
+            if (c0 + i < n_chunks) {
+                ax = fmaf(v[i].x, w_s[c0 + i], ax);
+                ay = fmaf(v[i].y, w_s[c0 + i], ay);
+            }
     }
+    const float inv = 1.0f / L;
+    *reinterpret_cast<uint32_t*>(out + (size_t)t * ldo + h * D + 2 * lane) =
+        (uint32_t)bf16_bits(ax * inv) | ((uint32_t)bf16_bits(ay * inv) << 16);
 }
 
 // log2 of the page size, or -1 if it is not a power of two (the kernels shift and mask by it).

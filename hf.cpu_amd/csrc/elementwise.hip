@@ -60,6 +60,12 @@ __global__ __launch_bounds__(1024) void rmsnorm_kernel(float* __restrict__ x, co
     float* src = x + (size_t)xr * width;
     float ss = 0.f;
     const bool vec = (width & 3) == 0;
+    // Few rows (decode): a thread has four values only, which stay in registers for the second
+    // half; the scale's weights are asked for before the sum's barriers, and the four results
+    // leave in one store.
+    const bool one_pass = vec && (int)blockDim.x * 4 >= width;
+    float4 keep = make_float4(0.f, 0.f, 0.f, 0.f), g4 = keep;
+    if (one_pass && (int)threadIdx.x * 4 < width) g4 = *reinterpret_cast<const float4*>(w + threadIdx.x * 4);
     if (vec) {
         for (int i = threadIdx.x * 4; i < width; i += blockDim.x * 4) {
             float4 v = *reinterpret_cast<const float4*>(src + i);
@@ -82,6 +88,7 @@ __global__ __launch_bounds__(1024) void rmsnorm_kernel(float* __restrict__ x, co
                 *reinterpret_cast<float4*>(src + i) = v;
             }
             ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+            keep = v;
         }
     } else {
         for (int i = threadIdx.x; i < width; i += blockDim.x) {
@@ -97,7 +104,21 @@ __global__ __launch_bounds__(1024) void rmsnorm_kernel(float* __restrict__ x, co
     ss = block_sum(ss, red);            // its barriers also order the writes of x before the reads below
     const float scale = 1.0f / sqrtf(ss / (float)width + eps);
     TO* dst = out + (size_t)r * width;
-    if (vec) {
+    if (one_pass) {
+        const int i = threadIdx.x * 4;
+        if (i < width) {
+            const TO o0 = from_f32<TO>((keep.x * scale) * g4.x), o1 = from_f32<TO>((keep.y * scale) * g4.y);
+            const TO o2 = from_f32<TO>((keep.z * scale) * g4.z), o3 = from_f32<TO>((keep.w * scale) * g4.w);
+            if constexpr (sizeof(TO) == 2) {
+                uint2 pk;
+                pk.x = (uint32_t)o0.bits | ((uint32_t)o1.bits << 16);
+                pk.y = (uint32_t)o2.bits | ((uint32_t)o3.bits << 16);
+                *reinterpret_cast<uint2*>(dst + i) = pk;
+            } else {
+                dst[i] = o0; dst[i + 1] = o1; dst[i + 2] = o2; dst[i + 3] = o3;
+            }
+        }
+    } else if (vec) {
         for (int i = threadIdx.x * 4; i < width; i += blockDim.x * 4) {
             const float4 v = *reinterpret_cast<const float4*>(src + i);
             const float4 g = *reinterpret_cast<const float4*>(w + i);

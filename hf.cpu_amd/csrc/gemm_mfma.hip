@@ -485,6 +485,37 @@ __global__ void gemm_finish_kernel(const float* __restrict__ partial, int splits
         reinterpret_cast<float*>(out)[(size_t)row * ldo + col] += v;
 }
 
+// The gate/up case of the above, four results a thread: 16-byte loads of every plane asked for
+// together (in batches of eight planes), added in ascending order, one 8-byte store.
+__global__ void gemm_finish_swiglu4_kernel(const float* __restrict__ partial, int splits, uint16_t* __restrict__ out,
+                                           int ldo, int M, int N) {
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;      // (row, block of 64 columns, quad)
+    const int per_row = N / 8;
+    if (idx >= (size_t)M * per_row) return;
+    const int row = (int)(idx / per_row), in_row = (int)(idx % per_row);
+    const int blk = in_row / 8, quad = in_row % 8;
+    const size_t plane = (size_t)M * N;
+    const float* src = partial + (size_t)row * N + blk * 64 + quad * 4;
+    float4 g = make_float4(0.f, 0.f, 0.f, 0.f), u = g;
+    for (int s0 = 0; s0 < splits; s0 += 8) {
+        float4 pg[8], pu[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            pg[i] = s0 + i < splits ? *reinterpret_cast<const float4*>(src + (s0 + i) * plane) : make_float4(0.f, 0.f, 0.f, 0.f);
+            pu[i] = s0 + i < splits ? *reinterpret_cast<const float4*>(src + (s0 + i) * plane + 32) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            g.x += pg[i].x; g.y += pg[i].y; g.z += pg[i].z; g.w += pg[i].w;
+            u.x += pu[i].x; u.y += pu[i].y; u.z += pu[i].z; u.w += pu[i].w;
+        }
+    }
+    uint2 pk;
+    pk.x = (uint32_t)bf16_bits((g.x / (1.0f + expf(-g.x))) * u.x) | ((uint32_t)bf16_bits((g.y / (1.0f + expf(-g.y))) * u.y) << 16);
+    pk.y = (uint32_t)bf16_bits((g.z / (1.0f + expf(-g.z))) * u.z) | ((uint32_t)bf16_bits((g.w / (1.0f + expf(-g.w))) * u.w) << 16);
+    *reinterpret_cast<uint2*>(out + (size_t)row * ldo + blk * 32 + quad * 4) = pk;
+}
+
 template <int BM, int BN, int BK, int WM, int WN, int MODE, int PF>
 static int launch_cfg(const GemmArgs& g, void* out, int splits, int k_per_split) {
     using C = MfmaCfg<BM, BN, BK, WM, WN>;
@@ -571,6 +602,8 @@ int gemm_finish_launch(const float* partial, int splits, const float* bias, void
         gemm_finish_kernel<OUT_BF16><<<blocks, 256, 0, stream>>>(partial, splits, bias, out, ldo, M, N);
     else if (mode == OUT_F32)
         gemm_finish_kernel<OUT_F32><<<blocks, 256, 0, stream>>>(partial, splits, bias, out, ldo, M, N);
+    else if (mode == OUT_SWIGLU && !bias && N % 64 == 0 && ldo % 4 == 0 && ((uintptr_t)out & 7) == 0 && ((uintptr_t)partial & 15) == 0)
+        gemm_finish_swiglu4_kernel<<<(int)((total / 8 + 255) / 256), 256, 0, stream>>>(partial, splits, (uint16_t*)out, ldo, M, N);
     else if (mode == OUT_SWIGLU)
         gemm_finish_kernel<OUT_SWIGLU><<<blocks, 256, 0, stream>>>(partial, splits, bias, out, ldo, M, N);
     else

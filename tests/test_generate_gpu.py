@@ -378,3 +378,41 @@ def test_real_layer_sizes_at_the_batch_sizes_with_kernels_of_their_own(gpu, tmp_
     for _ in range(2):
         again = helpers.run_trace_in_engine(engine, steps)
         assert all(np.array_equal(again[key], row) for key, row in got.items())
+
+
+FAMILY = {   # one layer of other members of the family: sizes from their published config.json files
+    "0.5B": dict(hidden_size=896, num_attention_heads=14, num_key_value_heads=2, head_dim=64, intermediate_size=4864,
+                 tie_word_embeddings=True),
+    "1.5B": dict(hidden_size=1536, num_attention_heads=12, num_key_value_heads=2, head_dim=128, intermediate_size=8960,
+                 tie_word_embeddings=True),
+    "3B": dict(hidden_size=2048, num_attention_heads=16, num_key_value_heads=2, head_dim=128, intermediate_size=11008,
+               tie_word_embeddings=True),
+    "32B": dict(hidden_size=5120, num_attention_heads=40, num_key_value_heads=8, head_dim=128, intermediate_size=27648,
+                tie_word_embeddings=False, rms_norm_eps=1e-5),
+}
+
+
+@pytest.mark.parametrize("member", list(FAMILY))
+def test_layer_sizes_of_the_family(gpu, tmp_path, member):
+    """One layer with the sizes of other members of the family (widths that are not multiples of
+    the 256-column tiles, 7, 6, 8 and 5 query heads per key/value head, head_dim 64 and 128), in
+    bf16 against the plain implementation on weights rounded to bf16: a prompt of 600 tokens in one
+    step (tiles of 256 rows), a second prompt in portions beside decoded tokens, and both decoded
+    together."""
+    import hf_cpu_amd
+    cfg = dict(architectures=["Qwen2ForCausalLM"], num_hidden_layers=1, vocab_size=2048, rope_theta=1e6,
+               rms_norm_eps=1e-6, max_position_embeddings=1024)
+    cfg.update(FAMILY[member])
+    d = helpers.make_model_dir(str(tmp_path / "m"), cfg, seed=len(member))
+    reqs = helpers.random_requests(cfg, [600, 70], seed=5)
+    a, b = reqs["r0"], reqs["r1"]
+    steps = [helpers._step(0, [("r0", a[:-5], [0, 299, 594])]),
+             helpers._step(1, [("r0", [a[-5]], [0]), ("r1", b[:33], [32])]),
+             helpers._step(2, [("r0", [a[-4]], [0]), ("r1", b[33:-3], [0, len(b) - 37])])]
+    for j in range(3, 0, -1):
+        steps.append(helpers._step(len(steps), [("r0", [a[-j]], [0]), ("r1", [b[-j]], [0])], ["r0", "r1"] if j == 1 else []))
+    want = helpers.plain_logits(d, reqs, round_weights_bf16=True)
+    engine = hf_cpu_amd.load_engine(d, dtype="bfloat16", page_tokens=16, max_tokens=768, max_seqs=2)
+    worst = helpers.compare(helpers.run_trace_in_engine(engine, steps), want, 2e-2, f"{member} layer")
+    print(f"{member}-sized layer: worst relative difference {worst:.2e}")
+    assert not engine.manager.held

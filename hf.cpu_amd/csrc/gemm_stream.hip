@@ -213,7 +213,10 @@ int gemm_stream_slots(const GemmArgs& g, size_t workspace_bytes) {
     if (g.M <= 32 || g.M > 64 || g.K % BK != 0 || g.N % BN != 0 || g.lda >= (1 << 22) || g.ldw >= (1 << 22)) return 0;
     const long long nk = g.K / BK, tiles = g.N / BN, U = tiles * nk;
     const int G = cu_count();
-    if (tiles >= 2 * G || U < 4 * G) return 0;               // enough tiles for whole-tile kernels; or runs too short
+    // Enough tiles for whole-tile kernels; or runs so short (under 16 units a block) that filling and
+    // draining the stages outweighs the even cut: the split-K kernel is quicker there (q/k/v and o of
+    // the 7B shape: 12 us against 14).
+    if (tiles >= 2 * G || U < 16 * G) return 0;
     const long long per_block = U / G;                       // the shortest run
     const int slots = (int)((nk + per_block - 1) / per_block) + 1;
     if ((size_t)slots * g.M * g.N * sizeof(float) > workspace_bytes) return 0;

@@ -320,7 +320,7 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
 #define PKS 136      // LDS row of a key: 128 dims + 8 pad (elements)
 #define PVS 36       // LDS row of a value dimension: 32 keys + 4 pad (elements)
 
-template <int NDB>
+template <int NDB, bool SMALL_PAGES>
 __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) void attn_prefill_kernel(
     const uint16_t* __restrict__ q, int ldq, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc, int kvw,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ token_slot,
@@ -401,14 +401,46 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
 
     // global -> registers -> LDS. Keys: 32 rows of D elements = 4 D chunks of 16 bytes.
     // Values: D rows of 32 keys = 4 D chunks of 8 keys. Each thread takes up to NCH of both.
+    // With a whole number of chunks per thread (head_dim 64 and 128) no load or store stands under a
+    // condition: only then does the compiler count the loads in flight and wait for the older set alone.
     constexpr int TOT = 4 * D, NCH = (TOT + 255) / 256;
+    constexpr bool EVEN = TOT % 256 == 0;
     u32x4 rk0[NCH], rk1[NCH];
     uint2 rv0[NCH][2], rv1[NCH][2];
+    // Pages of up to 32 tokens divide a block of keys, whose first key is a multiple of 32: a
+    // thread's row then lies at the same place of the same page of every block, and its addresses
+    // are a page id times the page's size plus a constant. No key is clamped on this path: the
+    // window of page ids repeats the last valid page for pages past the end (see below), so what is
+    // read there is memory of that page, and it is masked like any key past a column's position.
+    constexpr bool small_pages = SMALL_PAGES;                  // the launcher's choice: pages of up to 32 tokens
+    const unsigned page_elems = (unsigned)kvw << psh;
+    int k_pg[NCH], v_pg[NCH];
+    unsigned k_at[NCH], v_at[NCH];
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+        const int c = tid + i * 256, row = c / (D / 8), k8 = 8 * (c % 4);
+        k_pg[i] = row >> psh;
+        k_at[i] = (unsigned)((row & (P - 1)) * kvw + g * D + (c % (D / 8)) * 8);
+        v_pg[i] = k8 >> psh;
+        v_at[i] = (unsigned)(((g * D + c / 4) << psh) + (k8 & (P - 1)));
+    }
     auto gload = [&](int key0, u32x4 (&rk)[NCH], uint2 (&rv)[NCH][2]) {
+        if constexpr (small_pages) {
+            const int pb = (key0 >> psh) - pw0;
+#pragma unroll
+            for (int i = 0; i < NCH; i++) {
+                if (!EVEN && tid + i * 256 >= TOT) break;
+                rk[i] = *reinterpret_cast<const u32x4*>(kc + (__umul24((unsigned)pg_s[pb + k_pg[i]], page_elems) + k_at[i]));
+                const uint4 v = *reinterpret_cast<const uint4*>(vc + (__umul24((unsigned)pg_s[pb + v_pg[i]], page_elems) + v_at[i]));
+                rv[i][0] = make_uint2(v.x, v.y);
+                rv[i][1] = make_uint2(v.z, v.w);
+            }
+            return;
+        }
 #pragma unroll
         for (int i = 0; i < NCH; i++) {
             const int c = tid + i * 256;
-            if (c >= TOT) break;
+            if (!EVEN && c >= TOT) break;
             {   // key chunk: row c / (D / 8), 16-byte piece c % (D / 8)
                 int key = key0 + c / (D / 8);
                 key = key < hi ? key : hi;
@@ -431,7 +463,7 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
 #pragma unroll
         for (int i = 0; i < NCH; i++) {
             const int c = tid + i * 256;
-            if (c >= TOT) break;
+            if (!EVEN && c >= TOT) break;
             *reinterpret_cast<u32x4*>(&k_s[stage][(c / (D / 8)) * KROW + (c % (D / 8)) * 8]) = rk[i];
             uint2* dst = reinterpret_cast<uint2*>(&v_s[stage][(c / 4) * PVS + 8 * (c % 4)]);
             dst[0] = rv[i][0];
@@ -449,7 +481,9 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
         {
             const int top = first + we * KB - 1 < hi ? first + we * KB - 1 : hi;
             const int n_pg = (top >> psh) - pw0 + 1;
-            for (int i = tid; i < n_pg; i += 4 * WAVE) pg_s[i] = bt[pw0 + i];
+            // pages past the last one that holds keys (the window's last block is loaded whole): its id again
+            const int n_all = small_pages ? ((first + we * KB - 1) >> psh) - pw0 + 1 : n_pg;
+            for (int i = tid; i < n_all; i += 4 * WAVE) pg_s[i] = bt[pw0 + (i < n_pg ? i : n_pg - 1)];
         }
         __syncthreads();
         const int last = first + (we - 1) * KB;
@@ -692,10 +726,16 @@ static int launch_prefill(const AttnArgs& a, int tpt, int cpt) {
     const int n_tiles = a.n_seqs == 1 ? (a.n_tokens + tile_tokens - 1) / tile_tokens : 0;
     const int cus = attn_cu_count();
     const int pair_from = n_tiles * a.n_kv_heads > cus && n_tiles * a.n_kv_heads <= 2 * cus ? cus : 0;
-    attn_prefill_kernel<NDB><<<grid, 4 * WAVE, 0, a.stream>>>(
-        (const uint16_t*)a.q, a.ldq, (const uint16_t*)a.k_cache, (const uint16_t*)a.v_cache, a.kv_width, a.block_table,
-        a.max_blocks, a.token_slot, a.positions, a.q_start, a.n_seqs, (uint16_t*)a.out, a.ldo,
-        page_shift(a.page_tokens), a.window, a.scale * 1.4426950408889634f, tpt, cpt, n_tiles, pair_from);
+    if (a.page_tokens <= 32)
+        attn_prefill_kernel<NDB, true><<<grid, 4 * WAVE, 0, a.stream>>>(
+            (const uint16_t*)a.q, a.ldq, (const uint16_t*)a.k_cache, (const uint16_t*)a.v_cache, a.kv_width, a.block_table,
+            a.max_blocks, a.token_slot, a.positions, a.q_start, a.n_seqs, (uint16_t*)a.out, a.ldo,
+            page_shift(a.page_tokens), a.window, a.scale * 1.4426950408889634f, tpt, cpt, n_tiles, pair_from);
+    else
+        attn_prefill_kernel<NDB, false><<<grid, 4 * WAVE, 0, a.stream>>>(
+            (const uint16_t*)a.q, a.ldq, (const uint16_t*)a.k_cache, (const uint16_t*)a.v_cache, a.kv_width, a.block_table,
+            a.max_blocks, a.token_slot, a.positions, a.q_start, a.n_seqs, (uint16_t*)a.out, a.ldo,
+            page_shift(a.page_tokens), a.window, a.scale * 1.4426950408889634f, tpt, cpt, n_tiles, pair_from);
     HFA_LAUNCH_CHECK("attn_prefill");
     return 0;
 }

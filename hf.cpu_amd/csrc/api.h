@@ -52,6 +52,10 @@ int hfa_rope_store(void* qkv, int dtype, int ld, const int* positions, const flo
                    const int* slot_map, int page_tokens, int n_tokens, const float* partial, int splits,
                    const float* partial_bias, hipStream_t stream);
 
+// `run` (a request's tokens in one call) from which hfa_paged_attention takes the kernel for prompt
+// portions for the whole call; see the launcher in attention_mfma.hip.
+int hfa_attention_prompt_rows(void);
+
 // Softmax attention of each token's query heads over its request's cached keys and values
 // (src/model.c:499-528). Key j of the request in slot s lies in cache row
 // block_table[s, j / page_tokens] * page_tokens + j % page_tokens. A key is visible to the

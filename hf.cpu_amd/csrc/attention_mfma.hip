@@ -740,11 +740,17 @@ static int launch_prefill(const AttnArgs& a, int tpt, int cpt) {
     return 0;
 }
 
+// A call in which some request brings this many tokens or more goes to the kernel for prompt portions,
+// whole: it walks each request's keys in one piece. A caller that has requests with single tokens and
+// long contexts beside prompt portions does better to make two calls, one below and one from this number up.
+#define PROMPT_ROWS 16
+extern "C" int hfa_attention_prompt_rows(void) { return PROMPT_ROWS; }
+
 int attn_mfma_launch(const AttnArgs& a) {
     const int cpt = a.n_heads / a.n_kv_heads;              // columns per token: the heads of a group
     const int tpt = 32 / cpt;                              // tokens per tile
     // Steps with prompt portions: the kernel that shares keys and values between four waves.
-    if (a.max_q_len >= 16 && a.page_tokens % 8 == 0 && (a.n_tokens + 4 * tpt - 1) / (4 * tpt) + a.n_seqs <= 65535) {
+    if (a.max_q_len >= PROMPT_ROWS && a.page_tokens % 8 == 0 && (a.n_tokens + 4 * tpt - 1) / (4 * tpt) + a.n_seqs <= 65535) {
         switch (a.head_dim / 32) {
             case 1: return launch_prefill<1>(a, tpt, cpt);
             case 2: return launch_prefill<2>(a, tpt, cpt);

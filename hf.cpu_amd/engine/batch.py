@@ -31,6 +31,11 @@ class StepInputs:
     tokens[T], positions[T], token_slot[T] (the state slot = block-table row of the
     token's request), q_start[S + 1] (token range of each request), seq_slot[S],
     seq_len[S] (the request's length after this step), logit_rows[R].
+
+    Requests that bring few tokens (fewer than ``Ops.prompt_rows``: decoded tokens, ends of prompts)
+    come first in a step: the first ``n_short_seqs`` requests with ``n_short_tokens`` tokens, none
+    of them more than ``max_short_q_len``. ``q_start_long`` is ``q_start`` of the remaining requests
+    counted from their first token, so that a kernel can be given either part as a step of its own.
     """
 
     def __init__(self, n_tokens, n_seqs, n_logit_rows):
@@ -40,6 +45,8 @@ class StepInputs:
         self.groups = []
         self.max_q_len = 0
         self.max_seq_len = 0
+        self.n_short_seqs = self.n_short_tokens = self.max_short_q_len = 0
+        self.q_start_long = None
         self.host = None          # dict of the numpy arrays the device views were copied from
 
     def group(self, index):

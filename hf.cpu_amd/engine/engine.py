@@ -187,10 +187,10 @@ class Engine:
             rows = np.arange(S, dtype=np.int32)
             q_start = np.arange(S + 1, dtype=np.int32)
             tokens = tokens.astype(np.int32)
-            arrays = [tokens, lengths, slots, q_start, slots, seq_len, rows] + slot_maps
+            arrays = [tokens, lengths, slots, q_start, slots, seq_len, rows, np.zeros(1, np.int32)] + slot_maps
             step = self._upload(arrays, S, S, S, 1, int(seq_len.max()),
                                 dict(tokens=tokens, positions=lengths, token_slot=slots, q_start=q_start,
-                                     seq_slot=slots, seq_len=seq_len, logit_rows=rows))
+                                     seq_slot=slots, seq_len=seq_len, logit_rows=rows), short=(S, S, 1))
             logits = self.ops.scratch("logits", (S, self.vocab_size), torch.float32)
             self._run(step, logits)
             if self.profile is not None:
@@ -244,35 +244,45 @@ class Engine:
         q_start = np.zeros(S + 1, np.int32)
         seq_slot = np.empty(S, np.int32)
         seq_len = np.empty(S, np.int32)
-        rows = []
+        rows_of = [None] * S
         slot_maps = [np.empty(T, np.int32) for _ in mgr.groups]
         at = 0
         max_q = max_len = 0
-        for s, e in enumerate(entries):
+        # Requests with few tokens first (see StepInputs); logits keep the order of the entries.
+        few = self.ops.prompt_rows
+        order = sorted(range(S), key=lambda i: len(entries[i].tokens) >= few)
+        n_short = n_short_tokens = max_short = 0
+        for s, i in enumerate(order):
+            e = entries[i]
             h = mgr.held[e.req_id]
             n = len(e.tokens)
+            if n < few:
+                n_short, n_short_tokens, max_short = n_short + 1, n_short_tokens + n, max(max_short, n)
             tokens[at:at + n] = e.tokens
             positions[at:at + n] = np.arange(h.length, h.length + n, dtype=np.int32)
             token_slot[at:at + n] = h.slot
             q_start[s + 1] = at + n
             seq_slot[s] = h.slot
             seq_len[s] = h.length + n
-            rows.extend(at + int(w) for w in e.want)
+            rows_of[i] = [at + int(w) for w in e.want]
             for g in range(len(mgr.groups)):
                 slot_maps[g][at:at + n] = mgr.slot_rows(e.req_id, g, h.length, n)
             max_q = max(max_q, n)
             max_len = max(max_len, h.length + n)
             at += n
-        rows = as_i32(rows)
-        arrays = [tokens, positions, token_slot, q_start, seq_slot, seq_len, rows] + slot_maps
+        rows = as_i32([r for per_entry in rows_of for r in per_entry])
+        q_start_long = q_start[n_short:] - n_short_tokens
+        arrays = [tokens, positions, token_slot, q_start, seq_slot, seq_len, rows, q_start_long] + slot_maps
         return self._upload(arrays, T, S, len(rows), max_q, max_len,
                             dict(tokens=tokens, positions=positions, token_slot=token_slot, q_start=q_start,
-                                 seq_slot=seq_slot, seq_len=seq_len, logit_rows=rows))
+                                 seq_slot=seq_slot, seq_len=seq_len, logit_rows=rows),
+                            short=(n_short, n_short_tokens, max_short))
 
-    def _upload(self, arrays, T, S, R, max_q, max_len, host):
+    def _upload(self, arrays, T, S, R, max_q, max_len, host, short):
         """Sends a step's arrays (tokens, positions, token_slot, q_start, seq_slot, seq_len,
-        logit_rows, then one slot map per group) and the block-table entries appended since the
-        last step; returns the StepInputs."""
+        logit_rows, q_start_long, then one slot map per group) and the block-table entries appended
+        since the last step; returns the StepInputs. ``short``: number of the leading requests with
+        few tokens, their tokens, and the most tokens one of them brings."""
         mgr = self.manager
         # Arrays whose sizes follow from (T, S, R) come first, so that their places in the
         # device buffer are the same for every step of one shape (a captured graph reads them there).
@@ -286,12 +296,13 @@ class Engine:
         views = self.staging.upload(arrays)
         step = StepInputs(T, S, R)
         (step.tokens, step.positions, step.token_slot, step.q_start, step.seq_slot, step.seq_len,
-         step.logit_rows) = views[:7]
+         step.logit_rows, step.q_start_long) = views[:8]
         step.max_q_len, step.max_seq_len = max_q, max_len
+        step.n_short_seqs, step.n_short_tokens, step.max_short_q_len = short
         step.host = host
         for g in range(G):
-            slot_map = views[7 + g]
-            idx, val = views[7 + G + 2 * g:9 + G + 2 * g]
+            slot_map = views[8 + g]
+            idx, val = views[8 + G + 2 * g:10 + G + 2 * g]
             table = self.storage.block_tables[g]
             if dirty[g]:
                 self.ops.scatter_i32(table.view(-1), idx, val)

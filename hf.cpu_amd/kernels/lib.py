@@ -39,6 +39,8 @@ def library():
             lib.hfa_last_error.restype = c_char_p
             lib.hfa_last_error.argtypes = []
             lib.hfa_version.restype = c_int
+            lib.hfa_attention_prompt_rows.restype = c_int
+            lib.hfa_attention_prompt_rows.argtypes = []
             for name, args in _SIGNATURES.items():
                 fn = getattr(lib, name)
                 fn.argtypes = args

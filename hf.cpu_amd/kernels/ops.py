@@ -95,6 +95,7 @@ class Ops:
         self.device = torch.device(device)
         self.act_dtype = act_dtype
         self.lib = library()
+        self.prompt_rows = int(self.lib.hfa_attention_prompt_rows())   # see StepInputs and paged_attention
         self._scratch = {}
         self._scratch_views = {}             # (name, shape, dtype) -> the view handed out last time
         self._stream_handle = None
@@ -302,16 +303,33 @@ class Ops:
             fail(EINVAL, "paged_attention: queries, cache and output must share a dtype")
         if cache.k.shape[1] != n_kv_heads * head_dim:
             fail(EINVAL, "paged_attention: the cache rows do not hold n_kv_heads * head_dim values")
-        self._check(self.lib.hfa_paged_attention(
-            q.data_ptr(), _code(q), ldq, cache.k.data_ptr(), cache.v.data_ptr(), cache.k.shape[1],
-            g.block_table.data_ptr(), g.block_table.shape[1], _ints(step.token_slot, "token_slot", T),
-            _ints(step.positions, "positions", T), _ints(step.q_start, "q_start", step.n_seqs + 1), step.n_seqs,
-            step.max_q_len, step.max_seq_len, out.data_ptr(), ldo, T, n_heads, n_kv_heads, head_dim,
-            cache.page_tokens, int(window), float(scale), self.attn_workspace.data_ptr(),
-            self.attn_workspace.numel(),
-            # the matrix-core kernels address the cache with 32-bit element offsets and 24-bit row numbers
-            1 if self.force_plain_attention or cache.k.numel() >= 1 << 32 or cache.k.shape[0] >= 1 << 24 else 0,
-            self._stream()))
+        _ints(step.token_slot, "token_slot", T)
+        _ints(step.positions, "positions", T)
+        _ints(step.q_start, "q_start", step.n_seqs + 1)
+        # the matrix-core kernels address the cache with 32-bit element offsets and 24-bit row numbers
+        plain = self.force_plain_attention or cache.k.numel() >= 1 << 32 or cache.k.shape[0] >= 1 << 24
+
+        def call(first, n_tokens, q_start, n_seqs, max_q_len):
+            self._check(self.lib.hfa_paged_attention(
+                q.data_ptr() + first * ldq * q.element_size(), _code(q), ldq, cache.k.data_ptr(), cache.v.data_ptr(),
+                cache.k.shape[1], g.block_table.data_ptr(), g.block_table.shape[1],
+                step.token_slot.data_ptr() + 4 * first, step.positions.data_ptr() + 4 * first, q_start.data_ptr(), n_seqs,
+                max_q_len, step.max_seq_len, out.data_ptr() + first * ldo * out.element_size(), ldo, n_tokens, n_heads,
+                n_kv_heads, head_dim, cache.page_tokens, int(window), float(scale), self.attn_workspace.data_ptr(),
+                self.attn_workspace.numel(), 1 if plain else 0, self._stream()))
+
+        # Decoded tokens beside prompt portions: one call would send all of them to the kernel for prompt
+        # portions, which walks a request's keys in one piece (a decoded token with a long context would
+        # take as long as thousands of prompt tokens). The step lays requests with few tokens first, so
+        # each part is a step of its own: the first goes to the kernel that cuts the keys into chunks.
+        n_short = getattr(step, "n_short_seqs", 0)
+        if not plain and q.dtype == torch.bfloat16 and step.max_q_len >= self.prompt_rows and 0 < n_short < step.n_seqs:
+            ts = step.n_short_tokens
+            _ints(step.q_start_long, "q_start_long", step.n_seqs - n_short + 1)
+            call(0, ts, step.q_start, n_short, step.max_short_q_len)
+            call(ts, T - ts, step.q_start_long, step.n_seqs - n_short, step.max_q_len)
+        else:
+            call(0, T, step.q_start, step.n_seqs, step.max_q_len)
 
     def swiglu(self, gate_up, out):
         self.settle()

@@ -258,3 +258,29 @@ def test_random_configurations(gpu, tmp_path, seed):
     worst = max(float(np.max(np.abs(got[k] - got_plain[k]))) / float(np.max(np.abs(want[k[0]]))) for k in got)
     assert worst <= KERNELS_AGREE, f"random configuration {seed}: kernels differ by {worst:.2e} {cfg}"
     print(f"random configuration {seed}: matrix-core and plain kernels differ by {worst:.2e}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decoded_tokens_between_prompt_portions_keep_their_places(gpu, tiny, dtype):
+    """A step whose entries alternate prompt portions of 16 tokens and more with single tokens: the
+    engine lays the short ones first (attention takes them as a step of their own), the logits still
+    come back in the order of the entries and of their wanted places."""
+    name, cfg, d, reqs, want = tiny
+    ids = [r for r in reqs if len(reqs[r]) >= 33][:3]
+    if len(ids) < 3:
+        pytest.skip("needs three requests of 33 tokens or more")
+    a, b, c = ids
+    engine = engine_for(d, dtype, name, max_tokens=512)
+    engine.step([(a, reqs[a][:20], []), (c, reqs[c][:5], [])])
+    entries = [(b, reqs[b][:30], [29, 0]), (a, [reqs[a][20]], [0]), (c, reqs[c][5:25], [3, 19]), (a + "x", reqs[a][:1], [0])]
+    rows = engine.step(entries).float().cpu().numpy()
+    places = [(b, 29), (b, 0), (a, 20), (c, 8), (c, 24), (a, 0)]
+    assert rows.shape[0] == len(places)
+    got = {((r, p) if i < 5 else ("first", 0)): row for i, ((r, p), row) in enumerate(zip(places, rows))}
+    first = got.pop(("first", 0))
+    helpers.compare(got, want, TOL[dtype], f"{name} {dtype} alternating entries")
+    scale = float(np.max(np.abs(want[a])))
+    assert float(np.max(np.abs(first - want[a][0]))) / scale <= TOL[dtype]
+    # and the requests go on from there
+    more = engine.step([(a, [reqs[a][21]], [0]), (b, reqs[b][30:33], [2])]).float().cpu().numpy()
+    helpers.compare({(a, 21): more[0], (b, 32): more[1]}, want, TOL[dtype], f"{name} {dtype} the step after")

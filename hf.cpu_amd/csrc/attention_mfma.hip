@@ -750,7 +750,13 @@ int attn_mfma_launch(const AttnArgs& a) {
     const int cpt = a.n_heads / a.n_kv_heads;              // columns per token: the heads of a group
     const int tpt = 32 / cpt;                              // tokens per tile
     // Steps with prompt portions: the kernel that shares keys and values between four waves.
-    if (a.max_q_len >= PROMPT_ROWS && a.page_tokens % 8 == 0 && (a.n_tokens + 4 * tpt - 1) / (4 * tpt) + a.n_seqs <= 65535) {
+    // That kernel has one block per 4 x tpt tokens and key/value head, and a block walks its request's
+    // keys in one piece. Few tokens with long contexts (a small token budget far into a long prompt)
+    // leave most CUs idle for a long walk: those go to the kernel below, which cuts the keys into chunks.
+    const long prompt_blocks = ((long)(a.n_tokens + 4 * tpt - 1) / (4 * tpt)) * a.n_kv_heads;
+    const bool few_long = 2 * prompt_blocks < attn_cu_count() && a.max_seq_len >= 1024 && a.workspace != nullptr;
+    if (a.max_q_len >= PROMPT_ROWS && !few_long && a.page_tokens % 8 == 0 &&
+        (a.n_tokens + 4 * tpt - 1) / (4 * tpt) + a.n_seqs <= 65535) {
         switch (a.head_dim / 32) {
             case 1: return launch_prefill<1>(a, tpt, cpt);
             case 2: return launch_prefill<2>(a, tpt, cpt);

@@ -22,7 +22,8 @@
 //                    output has fewer than 512 tiles; else gemm_mfma_kernel with tiles of 64 x 128
 //   M > 64           gemm_dma_kernel (below) with tiles of 256 rows, if M wastes few of them and the
 //                    output has 128 tiles of 256 x 256 (tiles of 256 x 192 where those need fewer rounds
-//                    over the CUs; with 64 tiles K is cut in two, or the tiles are 256 x 128); else
+//                    over the CUs; with fewer K is cut into parts that give every CU a block, or the tiles
+//                    are 256 x 128); else
 //                    gemm_mfma_kernel with tiles of 128 x 128
 #include <type_traits>
 
@@ -661,15 +662,25 @@ int gemm_mfma_launch(const GemmArgs& g, void* workspace, size_t workspace_bytes,
     // Long prompts: tiles of 256 rows fed by direct loads into LDS, if the rows they waste past M
     // cost less than they gain (they run about a quarter faster than the 128 x 128 tiles).
     const int rows256 = (g.M + 255) / 256 * 256, rows128 = (g.M + 127) / 128 * 128;
-    const bool dma_ok = BM == 128 && splits == 1 && g.K % 64 == 0 && g.lda < (1 << 22) && g.ldw < (1 << 22) &&
-                        (size_t)rows256 * 100 <= (size_t)rows128 * 128 &&
+    const bool rows_ok = BM == 128 && g.K % 64 == 0 && g.lda < (1 << 22) && g.ldw < (1 << 22) &&
+                         (size_t)rows256 * 100 <= (size_t)rows128 * 128;
+    const bool dma_ok = rows_ok && splits == 1 &&
                         (g.out_dtype != HFA_BF16 || (g.ldo % 8 == 0 && g.N % 16 == 0 && ((uintptr_t)g.out & 15) == 0));
     const int tiles256 = (rows256 / 256) * ((g.N + 255) / 256);
-    // A narrow output has too few 256 x 256 tiles for the CUs: K is cut in two and the halves' sums
-    // go to the workspace, if it holds them; otherwise tiles of 256 x 128.
-    const bool halves = dma_ok && tiles256 < 128 && 2 * tiles256 >= 128 && g.K % 128 == 0 && g.K >= 2048 &&
-                        mode != OUT_SWIGLU && workspace != nullptr &&
-                        2 * (size_t)g.M * g.N * sizeof(float) <= workspace_bytes;
+    // A narrow output has too few 256 x 256 tiles for the CUs: K is cut into as many parts as give
+    // every CU a block (at most one round of blocks, parts of 512 columns at least) and the parts' sums
+    // go to the workspace, if it holds them; otherwise tiles of 256 x 128 or the tiles of 128 rows.
+    int parts = 0, part_k = 0;
+    if (rows_ok && tiles256 < 128 && mode != OUT_SWIGLU && workspace != nullptr) {
+        parts = 256 / tiles256;
+        if (parts > g.K / 512) parts = g.K / 512;
+        while (parts > 1 && (size_t)parts * g.M * g.N * sizeof(float) > workspace_bytes) parts--;
+        if (parts >= 2) {
+            part_k = ((g.K / 32 + parts - 1) / parts) * 32;
+            parts = (g.K + part_k - 1) / part_k;
+        }
+    }
+    const bool halves = parts >= 2;
     // Tiles of 192 columns do three quarters of the work of 256 (a little less efficiently): they are
     // taken when they need fewer rounds over the CUs by more than that.
     const int cus = 256;
@@ -681,13 +692,13 @@ int gemm_mfma_launch(const GemmArgs& g, void* workspace, size_t workspace_bytes,
     else if (dma_ok && tiles256 >= 128)
         rc = launch_dma<256, 256, 32, 2, 4, 4>(g, kmode, kout, 1, g.K);
     else if (halves) {
-        rc = launch_dma<256, 256, 32, 2, 4, 4>(g, OUT_PARTIAL, workspace, 2, g.K / 2);
+        rc = launch_dma<256, 256, 32, 2, 4, 4>(g, OUT_PARTIAL, workspace, parts, part_k);
         if (rc) return rc;
         if (defer && pending_splits) {
-            *pending_splits = 2;
+            *pending_splits = parts;
             return 0;
         }
-        return gemm_finish_launch((const float*)workspace, 2, g.bias, g.out, mode, g.ldo, g.M, g.N, g.stream);
+        return gemm_finish_launch((const float*)workspace, parts, g.bias, g.out, mode, g.ldo, g.M, g.N, g.stream);
     } else if (dma_ok && 2 * tiles256 >= 128)
         rc = launch_dma<256, 128, 32, 4, 2, 6>(g, kmode, kout, 1, g.K);
     else if (BM == 128)

@@ -25,7 +25,7 @@ bool gemm_mfma_supports(const GemmArgs& g);
 int gemm_mfma_launch(const GemmArgs& g, void* workspace, size_t workspace_bytes, int defer, int* pending_splits);
 int gemm_mode_of(const GemmArgs& g);
 
-// bf16 x bf16 for 32 < M <= 64 as one stream of (column tile, 64 columns of K) units cut evenly over the
+// bf16 x bf16 for 32 < M <= 128 as one stream of (column tile, 64 columns of K) units cut evenly over the
 // CUs (N a multiple of 128, K of 64). gemm_stream_slots() says how many [M][N] fp32 planes of the
 // workspace the product will leave its partial sums in (0: not taken); their sum in ascending
 // order is the product.

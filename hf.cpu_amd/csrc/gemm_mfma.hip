@@ -18,8 +18,9 @@
 //
 // Which kernel takes which shape (gemm_mfma_launch, at the end of this file):
 //   M <= 32          gemm_mfma_kernel, tiles of 32 x 128, K split, two register sets of loads in flight
-//   M in 33 .. 64    gemm_stream_kernel (gemm_stream.hip) if N is a multiple of 128 and K of 64 and the
-//                    output has fewer than 512 tiles; else gemm_mfma_kernel with tiles of 64 x 128
+//   M in 33 .. 128   gemm_stream_kernel (gemm_stream.hip) if N is a multiple of 128 and K of 64, the output
+//                    has fewer than 512 tiles and a block gets 16 units or more; else gemm_mfma_kernel
+//                    with tiles of 64 x 128 or 128 x 128
 //   M > 64           gemm_dma_kernel (below) with tiles of 256 rows, if M wastes few of them and the
 //                    output has 128 tiles of 256 x 256 (tiles of 256 x 192 where those need fewer rounds
 //                    over the CUs; with fewer K is cut into parts that give every CU a block, or the tiles
@@ -625,7 +626,7 @@ int gemm_mfma_launch(const GemmArgs& g, void* workspace, size_t workspace_bytes,
         hfa_set_error("gemm: the gate/up epilogue needs N a multiple of 64, no bias and a bf16 output");
         return 1;
     }
-    if (g.M <= 64) {
+    if (g.M <= 128) {
         const int slots = gemm_stream_slots(g, workspace ? workspace_bytes : 0);
         if (slots > 0) {
             const int rc = gemm_stream_launch(g, workspace, slots);

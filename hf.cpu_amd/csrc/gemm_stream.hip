@@ -1,5 +1,6 @@
 // bf16 matrix product for few rows (decode), bound by the speed at which the weights stream in:
-// out[m, n] = sum_k a[m, k] * w[n, k] with 32 < M <= 64, left as partial sums in a workspace.
+// out[m, n] = sum_k a[m, k] * w[n, k] with 32 < M <= 128 (tiles of 64 or 128 rows), left as partial sums
+// in a workspace.
 //
 // The work is the list of (column tile, 64 columns of K) units in tile-major order, cut into
 // one contiguous run of units per block, one block per CU: no CU waits for a last, partly filled
@@ -210,7 +211,7 @@ static int launch_stream(const GemmArgs& g, float* partial, int blocks, int slot
 int gemm_stream_slots(const GemmArgs& g, size_t workspace_bytes) {
     const int BN = 128, BK = 64;
     // Up to 32 rows the tiles of gemm_mfma_kernel, several blocks to a CU, stream as fast.
-    if (g.M <= 32 || g.M > 64 || g.K % BK != 0 || g.N % BN != 0 || g.lda >= (1 << 22) || g.ldw >= (1 << 22)) return 0;
+    if (g.M <= 32 || g.M > 128 || g.K % BK != 0 || g.N % BN != 0 || g.lda >= (1 << 22) || g.ldw >= (1 << 22)) return 0;
     const long long nk = g.K / BK, tiles = g.N / BN, U = tiles * nk;
     const int G = cu_count();
     // Enough tiles for whole-tile kernels; or runs so short (under 16 units a block) that filling and
@@ -224,5 +225,6 @@ int gemm_stream_slots(const GemmArgs& g, size_t workspace_bytes) {
 }
 
 int gemm_stream_launch(const GemmArgs& g, void* workspace, int slots) {
+    if (g.M > 64) return launch_stream<128, 128, 2, 2, 4>(g, (float*)workspace, cu_count(), slots);
     return launch_stream<64, 128, 2, 2, 6>(g, (float*)workspace, cu_count(), slots);
 }

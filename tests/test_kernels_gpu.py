@@ -99,7 +99,9 @@ def test_gemm(ops32, adt, wdt, odt, M, N, K):
                                    (2048, 512, 3584), (2048, 4608, 1024), (1000, 8200, 512), (700, 5408, 640),
                                    (2048, 3584, 1024), (1024, 8192, 64), (2048, 3584, 64), (512, 4096, 128), (1800, 3600, 2176),
                                    (64, 4608, 3584), (48, 3584, 18944), (33, 37888, 256), (40, 1024, 8192),
-                                   (150, 4608, 3584), (300, 3584, 4736), (1900, 4624, 192), (50, 33024, 320), (64, 65536, 64)])
+                                   (150, 4608, 3584), (300, 3584, 4736), (1900, 4624, 192), (50, 33024, 320), (64, 65536, 64),
+                                   (100, 3584, 18944), (128, 4096, 8192), (65, 37888, 1024),      # the stream kernel's tiles of 128 rows
+                                   (400, 3584, 18944), (256, 4608, 3584), (700, 3584, 3584)])     # 256-row tiles, K cut into parts
 def test_gemm_on_matrix_cores(ops16, M, N, K):
     """bf16 x bf16 with K a multiple of 8 runs on the matrix cores (K split for small M; tiles of
     256 rows loaded straight into LDS for long prompts and wide outputs, with edges in M and N

@@ -325,7 +325,8 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
     const uint16_t* __restrict__ q, int ldq, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc, int kvw,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ token_slot,
     const int* __restrict__ positions, const int* __restrict__ q_start, int n_seqs, uint16_t* __restrict__ out,
-    int ldo, int psh, int window, float scale_log2e, int tpt, int cpt, int n_tiles, int pair_from) {
+    int ldo, int psh, int window, float scale_log2e, int tpt, int cpt, int n_tiles, int pair_from,
+    float* __restrict__ partial, int H, int chunk_keys, int n_chunks) {
     constexpr int D = NDB * 32, KS = D / 16, KROW = D + 8;
     const int P = 1 << psh;                                // tokens per page, a power of two
     __shared__ __attribute__((aligned(16))) uint16_t k_s[2][KB * KROW];
@@ -373,10 +374,19 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
     const int my_tok = col_ok ? w0 + col / cpt : t0;
     const int my_head = g * cpt + (col_ok ? col % cpt : 0);
     const int pos = positions[my_tok];
-    const int pos_first = positions[t0], hi = positions[t_end - 1];
-    const int k_begin = window > 0 && pos_first - window + 1 > 0 ? pos_first - window + 1 : 0;
+    const int pos_first = positions[t0];
+    int hi = positions[t_end - 1];
+    int k_begin = window > 0 && pos_first - window + 1 > 0 ? pos_first - window + 1 : 0;
+    // With n_chunks > 1 the block takes the keys of chunk blockIdx.z only (chunk_keys is a multiple
+    // of the key block) and leaves maximum, sum and unscaled output for attn_merge_kernel; a chunk
+    // that holds none of the tile's keys leaves an empty record.
+    if (n_chunks > 1) {
+        const int c_lo = blockIdx.z * chunk_keys, c_hi = c_lo + chunk_keys - 1;
+        k_begin = k_begin > c_lo ? k_begin : c_lo;
+        hi = hi < c_hi ? hi : c_hi;
+    }
     const int vlo = window > 0 && pos - window + 1 > k_begin ? pos - window + 1 : k_begin;
-    const int vhi = col_ok ? pos : -1;
+    const int vhi = col_ok ? (pos < hi ? pos : hi) : -1;
     const int* bt = block_table + (size_t)token_slot[t0] * max_blocks;
 
     // query fragments stay in registers for the whole tile
@@ -472,7 +482,7 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
     };
 
     const int first = (k_begin / KB) * KB;
-    const int nb = (hi - first) / KB + 1;
+    const int nb = hi >= k_begin ? (hi - first) / KB + 1 : 0;
     const int win_blocks = (PG_MAX << psh) / KB;
     for (int wb = 0; wb < nb; wb += win_blocks) {
         const int we = wb + win_blocks < nb ? wb + win_blocks : nb;               // blocks [wb, we)
@@ -598,6 +608,20 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
         }
     }
     if (!col_ok) return;
+    if (n_chunks > 1) {
+        float* dst = partial + ((size_t)(my_tok * H + my_head) * n_chunks + blockIdx.z) * (D + 2);
+        if (half == 0) {
+            dst[0] = m;
+            dst[1] = l;
+        }
+#pragma unroll
+        for (int db = 0; db < NDB; db++)
+#pragma unroll
+            for (int rg = 0; rg < 4; rg++)
+                *reinterpret_cast<float4*>(dst + 2 + 32 * db + 8 * rg + 4 * half) =
+                    make_float4(o[db][4 * rg], o[db][4 * rg + 1], o[db][4 * rg + 2], o[db][4 * rg + 3]);
+        return;
+    }
     const float inv = 1.0f / l;
     uint16_t* dst = out + (size_t)my_tok * ldo + my_head * D;
 #pragma unroll
@@ -725,18 +749,45 @@ static int launch_prefill(const AttnArgs& a, int tpt, int cpt) {
     // One request: the number of tiles is known here, and with it whether all blocks are resident at once.
     const int n_tiles = a.n_seqs == 1 ? (a.n_tokens + tile_tokens - 1) / tile_tokens : 0;
     const int cus = attn_cu_count();
-    const int pair_from = n_tiles * a.n_kv_heads > cus && n_tiles * a.n_kv_heads <= 2 * cus ? cus : 0;
+    int pair_from = n_tiles * a.n_kv_heads > cus && n_tiles * a.n_kv_heads <= 2 * cus ? cus : 0;
+    // Fewer blocks than two a CU, each with a long walk over its request's keys: the keys are cut into
+    // chunks of 256 or more over blockIdx.z until the machine is full, and attn_merge_kernel puts the
+    // chunks' results together (portions of a few hundred tokens far into a long prompt).
+    int n_chunks = 1, chunk_keys = a.max_seq_len;
+    const long blocks = (long)a.n_kv_heads * ((a.n_tokens + tile_tokens - 1) / tile_tokens);
+    if (blocks < 2 * cus && a.max_seq_len >= 512 && a.workspace != nullptr) {
+        long want = (2 * cus + blocks - 1) / blocks;
+        if (want > a.max_seq_len / 256) want = a.max_seq_len / 256;
+        if (want > MERGE_MAX_CHUNKS) want = MERGE_MAX_CHUNKS;
+        const size_t per_chunk = (size_t)a.n_tokens * a.n_heads * (a.head_dim + 2) * sizeof(float);
+        if ((size_t)want * per_chunk > a.workspace_bytes) want = (long)(a.workspace_bytes / per_chunk);
+        if (want > 1) {
+            chunk_keys = (int)((a.max_seq_len + want - 1) / want + 63) / 64 * 64;
+            n_chunks = (a.max_seq_len + chunk_keys - 1) / chunk_keys;
+        }
+    }
+    if (n_chunks > 1) {
+        pair_from = 0;
+        grid.z = n_chunks;
+    }
     if (a.page_tokens <= 32)
         attn_prefill_kernel<NDB, true><<<grid, 4 * WAVE, 0, a.stream>>>(
             (const uint16_t*)a.q, a.ldq, (const uint16_t*)a.k_cache, (const uint16_t*)a.v_cache, a.kv_width, a.block_table,
             a.max_blocks, a.token_slot, a.positions, a.q_start, a.n_seqs, (uint16_t*)a.out, a.ldo,
-            page_shift(a.page_tokens), a.window, a.scale * 1.4426950408889634f, tpt, cpt, n_tiles, pair_from);
+            page_shift(a.page_tokens), a.window, a.scale * 1.4426950408889634f, tpt, cpt, n_tiles, pair_from,
+            (float*)a.workspace, a.n_heads, chunk_keys, n_chunks);
     else
         attn_prefill_kernel<NDB, false><<<grid, 4 * WAVE, 0, a.stream>>>(
             (const uint16_t*)a.q, a.ldq, (const uint16_t*)a.k_cache, (const uint16_t*)a.v_cache, a.kv_width, a.block_table,
             a.max_blocks, a.token_slot, a.positions, a.q_start, a.n_seqs, (uint16_t*)a.out, a.ldo,
-            page_shift(a.page_tokens), a.window, a.scale * 1.4426950408889634f, tpt, cpt, n_tiles, pair_from);
+            page_shift(a.page_tokens), a.window, a.scale * 1.4426950408889634f, tpt, cpt, n_tiles, pair_from,
+            (float*)a.workspace, a.n_heads, chunk_keys, n_chunks);
     HFA_LAUNCH_CHECK("attn_prefill");
+    if (n_chunks > 1) {
+        attn_merge_kernel<<<dim3(a.n_tokens, a.n_heads), WAVE, 0, a.stream>>>((const float*)a.workspace, (uint16_t*)a.out, a.ldo,
+                                                                            a.n_heads, a.head_dim, n_chunks);
+        HFA_LAUNCH_CHECK("attn_merge");
+    }
     return 0;
 }
 
@@ -750,11 +801,11 @@ int attn_mfma_launch(const AttnArgs& a) {
     const int cpt = a.n_heads / a.n_kv_heads;              // columns per token: the heads of a group
     const int tpt = 32 / cpt;                              // tokens per tile
     // Steps with prompt portions: the kernel that shares keys and values between four waves.
-    // That kernel has one block per 4 x tpt tokens and key/value head, and a block walks its request's
-    // keys in one piece. Few tokens with long contexts (a small token budget far into a long prompt)
-    // leave most CUs idle for a long walk: those go to the kernel below, which cuts the keys into chunks.
+    // That kernel has one block per 4 x tpt tokens and key/value head (and chunk of keys, when it has
+    // few blocks). Very few tokens with long contexts (a token budget of 64 far into a long prompt)
+    // fill its tiles badly: those go to the kernel below, one wave per tile, which also cuts the keys.
     const long prompt_blocks = ((long)(a.n_tokens + 4 * tpt - 1) / (4 * tpt)) * a.n_kv_heads;
-    const bool few_long = 2 * prompt_blocks < attn_cu_count() && a.max_seq_len >= 1024 && a.workspace != nullptr;
+    const bool few_long = 8 * prompt_blocks < attn_cu_count() && a.max_seq_len >= 1024 && a.workspace != nullptr;
     if (a.max_q_len >= PROMPT_ROWS && !few_long && a.page_tokens % 8 == 0 &&
         (a.n_tokens + 4 * tpt - 1) / (4 * tpt) + a.n_seqs <= 65535) {
         switch (a.head_dim / 32) {

@@ -380,7 +380,8 @@ def tail_attention(q_tail, k, v, window):
 @pytest.mark.parametrize("H,G,D,page,window,lengths,q_lens", [
     (28, 4, 128, 16, 0, [40000, 9000, 17], [1, 1, 1]),       # more pages than one window of page ids holds
     (8, 2, 64, 16, 0, [20000], [200]),                         # a portion late in a long prompt: few blocks, keys in chunks
-    (8, 2, 64, 16, 0, [12000], [2100]),                        # the same with enough tokens for the kernel that shares keys through LDS
+    (8, 2, 64, 16, 0, [12000], [2100]),                        # the same with enough tokens for the kernel that shares keys through LDS (keys in chunks too)
+    (28, 4, 32, 16, 0, [12000], [2100]),                       # and with enough blocks that each walks all its keys, through several windows of page ids
     (4, 4, 32, 8, 5000, [30000, 4999, 5001], [3, 1, 2]),       # a window far into a long sequence
     (14, 2, 64, 16, 0, [100000], [1]),                         # more chunks of keys than one merge pass takes
 ])

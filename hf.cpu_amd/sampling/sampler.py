@@ -12,6 +12,7 @@ the row's log-sum-exp, kernels in csrc/sampling.hip); the few candidates left ar
 on the host in fp32 in exactly the order above. With ``top_k`` off (0) or beyond the
 kernel's 1024 the row is copied and ordered on the host.
 """
+from concurrent.futures import ThreadPoolExecutor
 from dataclasses import dataclass
 
 import numpy as np
@@ -81,7 +82,7 @@ def pick(ids, logits, params, rng):
 def order_on_host(row, top_k):
     """All candidates of a row in order, cut to top_k if it is on (src/sample.c:59-64, 81-98)."""
     row = np.asarray(row, dtype=f32)
-    order = np.lexsort((np.arange(len(row)), -row))
+    order = np.argsort(-row, kind="stable")                 # logit descending, ties by id ascending
     if 0 < top_k < len(order):
         order = order[:top_k]
     return order.astype(np.int64), row[order]
@@ -117,14 +118,29 @@ class Sampler:
             ids, vals, stats = (t.cpu().numpy() for t in self.ops.topk(logits, need_k))
         toks = [None] * R
         groups = {}                               # rows drawn from the device's candidates, by parameters
+        on_host = []                              # rows whose whole vocabulary is put in order on the host
         for i, (params, rng, n_lp) in enumerate(wants):
             if params.greedy:
                 toks[i] = int(arg[i])
             elif 0 < params.top_k <= TOPK_KERNEL_MAX and params.top_k < logits.shape[1]:
                 groups.setdefault(params, []).append(i)
             else:
-                cand, cl = order_on_host(logits[i].cpu().numpy(), params.top_k)
-                toks[i] = pick(cand, cl, params, rng)
+                on_host.append(i)
+        if on_host:
+            # One copy for all such rows; ordering a vocabulary takes milliseconds a row, and numpy's
+            # sort runs outside the interpreter's lock, so the rows are ordered side by side.
+            block = logits.cpu().numpy()
+
+            def draw(i):
+                cand, cl = order_on_host(block[i], wants[i][0].top_k)
+                return pick(cand, cl, wants[i][0], wants[i][1])
+
+            if len(on_host) == 1:
+                toks[on_host[0]] = draw(on_host[0])
+            else:
+                with ThreadPoolExecutor(max_workers=min(16, len(on_host))) as pool:
+                    for i, t in zip(on_host, pool.map(draw, on_host)):
+                        toks[i] = t
         for params, rows in groups.items():
             drawn = pick_rows(ids[rows, :params.top_k], vals[rows, :params.top_k], params, [wants[i][1] for i in rows])
             for i, t in zip(rows, drawn):

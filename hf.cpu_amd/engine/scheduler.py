@@ -28,6 +28,7 @@ when its last portion is done the other continuations are forked from the first 
 seed. A continuation for which no slot or page is free at that moment waits in the queue
 and computes the prompt itself.
 """
+import itertools
 import time
 from collections import deque
 from dataclasses import dataclass, field
@@ -173,7 +174,8 @@ class Scheduler:
         prefilling = [r for r in self.running if not (r.unfed == 1 and r.n_fed > 0)]
         live = len(self.running)
         free_slots = mgr.n_slots - len(mgr.held)
-        candidates = [(r, False) for r in prefilling] + [(r, True) for r in self.waiting]
+        # the loop leaves at the first request that has to wait: the queue is walked, never copied
+        candidates = itertools.chain(((r, False) for r in prefilling), ((r, True) for r in self.waiting))
         for r, is_new in candidates:
             if budget <= 0:
                 break
@@ -229,7 +231,12 @@ class Scheduler:
     def step(self):
         """Plans, runs and books one step. Returns the plan (None if there was nothing to do)."""
         now = self.clock()
-        for r in list(self.running) + list(self.waiting):                       # src/ops.c:790, 829
+        # Live requests are polled every step; a long queue is walked every 32nd step only (a request
+        # that waits has nothing that a cancellation could stop, it is only reported a little later).
+        polled = list(self.running)
+        if len(self.waiting) <= 256 or self.steps % 32 == 0:
+            polled += list(self.waiting)
+        for r in polled:                                                        # src/ops.c:790, 829
             expired = r.timeout > 0 and now - r.t_submit > r.timeout
             if r.cancel or expired:
                 if r.status == WAITING:

@@ -266,3 +266,17 @@ def test_continuations_end_with_a_prompt_that_fails():
     assert all(r.error is not None and r.error.code == "ERANGE" for r in fam)
     with pytest.raises(EngineError):
         s.submit(Request("x", [1, 2], greedy()), forks=[Request("y", [1, 3], greedy())])
+
+
+def test_a_cancellation_deep_in_a_long_queue_is_seen_within_32_steps():
+    """More than 256 requests waiting: the queue is polled every 32nd step only; a request cancelled
+    while it waits ends with ECANCEL before it is ever admitted."""
+    eng, s = make(budget=8, n_pages=64, slots=2)
+    rs = [s.submit(Request(i, [1, 2, 3], greedy(), max_tokens=40)) for i in range(400)]
+    s.step()
+    victim = rs[350]
+    victim.cancel = True
+    for _ in range(33):
+        s.step()
+    assert victim.error is not None and victim.error.code == "ECANCEL" and victim.admitted_at == -1
+    assert all(350 not in [r for r, _, _ in step] for step in eng.log)

@@ -83,6 +83,14 @@ int hfa_scatter_i32(int* dst, const int* idx, const int* val, int n, hipStream_t
 int hfa_argmax(const float* logits, int ld, int* out, int n_rows, int vocab, void* workspace,
                size_t workspace_bytes, hipStream_t stream);
 
+// All candidates of the chosen rows (rows[i], or row i if rows is null) in the order (logit
+// descending, id ascending), as the reference's sort leaves them when top-k is off
+// (src/sample.c:59-64, 93-98): ids and vals are [n_rows, vocab]. `scratch` needs
+// hfa_order_rows_scratch(n_rows, vocab) bytes, 8-byte aligned.
+size_t hfa_order_rows_scratch(int n_rows, int vocab);
+int hfa_order_rows(const float* logits, int ld, const int* rows, int* ids, float* vals, int n_rows, int vocab,
+                   void* scratch, size_t scratch_bytes, hipStream_t stream);
+
 // The k best of each row in the order (logit descending, id ascending) (src/sample.c:59-64),
 // and stats[r] = {max, log(sum(exp(l - max)))} (src/sample.c:25-33). k <= 1024.
 int hfa_topk(const float* logits, int ld, int* ids, float* vals, float* stats, int n_rows, int vocab, int k,

@@ -266,3 +266,119 @@ extern "C" int hfa_topk(const float* logits, int ld, int* ids, float* vals, floa
     HFA_LAUNCH_CHECK("topk");
     return 0;
 }
+
+// ---- a whole row in order --------------------------------------------------------------------
+// All candidates of a row in the order (logit descending, id ascending): what the reference's
+// qsort gives when top-k is off (src/sample.c:59-64, 93-98). One block of 1024 threads per chosen
+// row sorts the order-reversing integer image of its logits by least-significant-digit radix
+// sort, four passes of eight bits, each of them stable (so equal logits keep their ids' order):
+//  - a histogram of the digit over the row gives every digit its first place;
+//  - the row is then walked 1024 elements at a time in its present order. Inside a wave eight
+//    ballots tell each lane which lanes before it hold the same digit; the waves' counts per
+//    digit meet in LDS, and a prefix over the waves gives every element its place.
+// The passes go back and forth between two scratch rows of (key, id) pairs; the last pass writes
+// ids and logits. No atomics decide a place: the result is the same in every run.
+#define ORDER_THREADS 1024
+#define ORDER_WAVES (ORDER_THREADS / WAVE)
+
+__device__ __forceinline__ float key_float(uint32_t k) {     // inverse of float_key
+    return __uint_as_float((k & 0x80000000u) ? (k & 0x7fffffffu) : ~k);
+}
+
+__global__ __launch_bounds__(ORDER_THREADS) void order_rows_kernel(const float* __restrict__ logits, int ld,
+                                                                   const int* __restrict__ rows, int vocab,
+                                                                   uint2* __restrict__ scratch, int* __restrict__ ids,
+                                                                   float* __restrict__ vals) {
+    __shared__ uint32_t first[256];                           // next free place of each digit
+    __shared__ uint32_t wave_cnt[ORDER_WAVES][256];
+    const int tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
+    const int out_row = blockIdx.x;
+    const float* src_row = logits + (size_t)(rows ? rows[out_row] : out_row) * ld;
+    uint2* buf[2] = {scratch + (size_t)out_row * 2 * vocab, scratch + ((size_t)out_row * 2 + 1) * vocab};
+    int* ids_row = ids + (size_t)out_row * vocab;
+    float* vals_row = vals + (size_t)out_row * vocab;
+    const uint64_t below = lane == 0 ? 0ull : (~0ull >> (WAVE - lane));
+
+    for (int pass = 0; pass < 4; pass++) {
+        const int shift = 8 * pass;
+        const uint2* from = pass == 0 ? nullptr : buf[(pass - 1) & 1];
+        uint2* to = buf[pass & 1];
+        auto element = [&](int i) {                            // (key, id) number i of the present order
+            if (pass == 0) return make_uint2(~float_key(src_row[i] + 0.0f), (uint32_t)i);      // -0 counts as 0: a tie
+            return from[i];
+        };
+        // places of the digits
+        if (tid < 256) first[tid] = 0;
+        __syncthreads();
+        for (int i = tid; i < vocab; i += ORDER_THREADS) atomicAdd(&first[(element(i).x >> shift) & 255u], 1u);
+        __syncthreads();
+        if (tid < WAVE) {                                      // exclusive prefix over 256 counts by one wave
+            uint32_t c[4], s = 0;
+#pragma unroll
+            for (int j = 0; j < 4; j++) { c[j] = first[tid * 4 + j]; s += c[j]; }
+            uint32_t incl = s;
+#pragma unroll
+            for (int off = 1; off < WAVE; off <<= 1) {
+                const uint32_t up = __shfl_up(incl, off, WAVE);
+                if (lane >= off) incl += up;
+            }
+            uint32_t run = incl - s;
+#pragma unroll
+            for (int j = 0; j < 4; j++) { first[tid * 4 + j] = run; run += c[j]; }
+        }
+        __syncthreads();
+        // the stable scatter, 1024 elements of the present order at a time
+        for (int c0 = 0; c0 < vocab; c0 += ORDER_THREADS) {
+            for (int j = tid; j < ORDER_WAVES * 256; j += ORDER_THREADS) (&wave_cnt[0][0])[j] = 0;
+            __syncthreads();
+            const int i = c0 + tid;
+            const bool valid = i < vocab;
+            const uint2 e = valid ? element(i) : make_uint2(0, 0);
+            const uint32_t d = (e.x >> shift) & 255u;
+            uint64_t same = __ballot(valid);
+#pragma unroll
+            for (int b = 0; b < 8; b++) {
+                const uint64_t set = __ballot(valid && ((d >> b) & 1u));
+                same &= ((d >> b) & 1u) ? set : ~set;
+            }
+            const int rank = __popcll(same & below);
+            if (valid && rank == 0) wave_cnt[wave][d] = (uint32_t)__popcll(same);
+            __syncthreads();
+            if (tid < 256) {                                   // places of this chunk's waves, digit tid
+                uint32_t run = first[tid];
+#pragma unroll
+                for (int w = 0; w < ORDER_WAVES; w++) {
+                    const uint32_t c = wave_cnt[w][tid];
+                    wave_cnt[w][tid] = run;
+                    run += c;
+                }
+                first[tid] = run;
+            }
+            __syncthreads();
+            if (valid) {
+                const uint32_t at = wave_cnt[wave][d] + (uint32_t)rank;
+                if (pass < 3) {
+                    to[at] = e;
+                } else {
+                    ids_row[at] = (int)e.y;
+                    vals_row[at] = key_float(~e.x);
+                }
+            }
+            __syncthreads();
+        }
+        __threadfence_block();                                 // the next pass reads what this one wrote
+        __syncthreads();
+    }
+}
+
+extern "C" size_t hfa_order_rows_scratch(int n_rows, int vocab) { return (size_t)n_rows * 2 * vocab * sizeof(uint2); }
+
+extern "C" int hfa_order_rows(const float* logits, int ld, const int* rows, int* ids, float* vals, int n_rows, int vocab,
+                              void* scratch, size_t scratch_bytes, hipStream_t stream) {
+    HFA_REQUIRE(n_rows > 0 && vocab > 0 && ld >= vocab, "order_rows: bad sizes rows=%d vocab=%d ld=%d", n_rows, vocab, ld);
+    HFA_REQUIRE(scratch && scratch_bytes >= hfa_order_rows_scratch(n_rows, vocab) && ((uintptr_t)scratch & 7) == 0,
+                "order_rows: the scratch memory is smaller than two rows of (key, id) pairs for each of %d rows", n_rows);
+    order_rows_kernel<<<n_rows, ORDER_THREADS, 0, stream>>>(logits, ld, rows, vocab, (uint2*)scratch, ids, vals);
+    HFA_LAUNCH_CHECK("order_rows");
+    return 0;
+}

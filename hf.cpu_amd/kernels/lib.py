@@ -24,6 +24,7 @@ _SIGNATURES = {
     "hfa_scatter_i32": [P, P, P, I, P],
     "hfa_argmax": [P, I, P, I, I, P, c_size_t, P],
     "hfa_topk": [P, I, P, P, P, I, I, I, P],
+    "hfa_order_rows": [P, I, P, P, P, I, I, P, c_size_t, P],
 }
 
 
@@ -39,6 +40,8 @@ def library():
             lib.hfa_last_error.restype = c_char_p
             lib.hfa_last_error.argtypes = []
             lib.hfa_version.restype = c_int
+            lib.hfa_order_rows_scratch.restype = c_size_t
+            lib.hfa_order_rows_scratch.argtypes = [c_int, c_int]
             lib.hfa_attention_prompt_rows.restype = c_int
             lib.hfa_attention_prompt_rows.argtypes = []
             for name, args in _SIGNATURES.items():

@@ -356,6 +356,23 @@ class Ops:
                                         R, V, self.workspace.data_ptr(), self.workspace.numel(), self._stream()))
         return out
 
+    def order_rows(self, logits, rows=None):
+        """(ids [n, V] int32, values [n, V] fp32): every candidate of the chosen rows (all rows if
+        ``rows`` is None) in the order (logit descending, id ascending)."""
+        self.settle()
+        R, V = logits.shape
+        if logits.dtype != torch.float32:
+            fail(EINVAL, "order_rows: logits must be fp32")
+        n = R if rows is None else int(rows.numel())
+        ids = torch.empty((n, V), dtype=torch.int32, device=logits.device)
+        vals = torch.empty((n, V), dtype=torch.float32, device=logits.device)
+        need = int(self.lib.hfa_order_rows_scratch(n, V))
+        scratch = self.scratch("order_rows", (need,), torch.uint8)
+        self._check(self.lib.hfa_order_rows(logits.data_ptr(), _rows(logits, "order_rows logits"),
+                                            None if rows is None else _ints(rows, "order_rows rows", n), ids.data_ptr(),
+                                            vals.data_ptr(), n, V, scratch.data_ptr(), need, self._stream()))
+        return ids, vals
+
     def topk(self, logits, k, want_stats=True):
         """(ids [R, k] int32, values [R, k] fp32, stats [R, 2] fp32 = max and log-sum-exp
         above the max), candidates in the order (logit descending, id ascending)."""

@@ -16,6 +16,7 @@ from concurrent.futures import ThreadPoolExecutor
 from dataclasses import dataclass
 
 import numpy as np
+import torch
 
 from ..status import EINVAL, fail
 
@@ -80,7 +81,8 @@ def pick(ids, logits, params, rng):
 
 
 def order_on_host(row, top_k):
-    """All candidates of a row in order, cut to top_k if it is on (src/sample.c:59-64, 81-98)."""
+    """All candidates of a row in order, cut to top_k if it is on (src/sample.c:59-64, 81-98): the
+    order that the device's kernels give, written out in numpy for the tests of ``pick``."""
     row = np.asarray(row, dtype=f32)
     order = np.argsort(-row, kind="stable")                 # logit descending, ties by id ascending
     if 0 < top_k < len(order):
@@ -127,19 +129,22 @@ class Sampler:
             else:
                 on_host.append(i)
         if on_host:
-            # One copy for all such rows; ordering a vocabulary takes milliseconds a row, and numpy's
-            # sort runs outside the interpreter's lock, so the rows are ordered side by side.
-            block = logits.cpu().numpy()
+            # The device puts the whole vocabulary of these rows in order; the draw over so many
+            # candidates takes about a millisecond a row in numpy, outside the interpreter's lock,
+            # so the rows are drawn side by side.
+            chosen = None if len(on_host) == R else torch.tensor(on_host, dtype=torch.int32, device=logits.device)
+            all_ids, all_vals = (t.cpu().numpy() for t in self.ops.order_rows(logits, chosen))
 
-            def draw(i):
-                cand, cl = order_on_host(block[i], wants[i][0].top_k)
-                return pick(cand, cl, wants[i][0], wants[i][1])
+            def draw(j):
+                params, rng, _ = wants[on_host[j]]
+                k = params.top_k if 0 < params.top_k < all_ids.shape[1] else all_ids.shape[1]
+                return pick(all_ids[j, :k], all_vals[j, :k], params, rng)
 
             if len(on_host) == 1:
-                toks[on_host[0]] = draw(on_host[0])
+                toks[on_host[0]] = draw(0)
             else:
                 with ThreadPoolExecutor(max_workers=min(16, len(on_host))) as pool:
-                    for i, t in zip(on_host, pool.map(draw, on_host)):
+                    for i, t in zip(on_host, pool.map(draw, range(len(on_host)))):
                         toks[i] = t
         for params, rows in groups.items():
             drawn = pick_rows(ids[rows, :params.top_k], vals[rows, :params.top_k], params, [wants[i][1] for i in rows])

@@ -597,6 +597,27 @@ def test_argmax_and_topk(ops32):
     assert abs(float(stats[1, 1]) - np.log(np.sum(np.exp(small[1].astype(np.float64) - small[1].max())))) < 1e-5
 
 
+@pytest.mark.parametrize("V", [5, 1000, 1025, 4096, 152064])
+def test_order_rows(ops32, V):
+    """A whole row in order (logit descending, id ascending) against numpy's stable sort: random
+    logits with many ties (values drawn from a few hundred numbers), signed zeros, huge and tiny
+    values; all rows, and a choice of rows."""
+    rng = np.random.default_rng(V)
+    R = 5
+    pool = np.concatenate([rng.standard_normal(300).astype(np.float32) * 7, np.array([0.0, -0.0, 1e30, -1e30, 1e-40, -1e-40], np.float32)])
+    logits = pool[rng.integers(0, len(pool), (R, V))]
+    logits[1] = rng.standard_normal(V).astype(np.float32)            # a row without ties
+    logits[2] = 3.25                                                  # a row of equal values: ids in order
+    dev_logits = torch.from_numpy(logits).cuda()
+    for chosen in (None, [3, 0]):
+        rows = None if chosen is None else torch.tensor(chosen, dtype=torch.int32, device="cuda")
+        ids, vals = (t.cpu().numpy() for t in ops32.order_rows(dev_logits, rows))
+        for j, r in enumerate(range(R) if chosen is None else chosen):
+            want = np.argsort(-logits[r], kind="stable")            # 0.0 and -0.0 are a tie here as in the kernel
+            assert np.array_equal(ids[j], want), f"row {r}: first difference at {int(np.argmax(ids[j] != want))}"
+            assert np.array_equal(vals[j], logits[r][want])           # == : the kernel returns 0.0 for -0.0
+
+
 def test_kernels_refuse_what_they_cannot_do(ops32):
     from hf_cpu_amd.status import EngineError
     with pytest.raises(EngineError, match="head_dim"):

@@ -65,8 +65,104 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const TA* __restrict_
     }
 }
 
+// Few rows (decode): the product is bound by the stream of the weights, and 64 x 64 tiles leave most
+// CUs without a block. Here a block takes 32 output columns and all rows (up to 64), 256 threads each
+// own two columns of MR rows, and K goes through LDS in steps of 128 with the next step's values on
+// their way in registers. Every output is still one chain of fused multiply-adds in ascending k, so
+// the bits are those of the kernel above, whatever M is.
+#define SBN 32
+#define SBK 128
+
+template <typename TA, typename TW, typename TO, bool ACC, int MR>
+__global__ __launch_bounds__(256) void gemm_generic_rows_kernel(const TA* __restrict__ a, int lda,
+                                                                const TW* __restrict__ w, int ldw,
+                                                                const float* __restrict__ bias, TO* __restrict__ out,
+                                                                int ldo, int M, int N, int K) {
+    constexpr int ROWS = 16 * MR;
+    __shared__ __attribute__((aligned(16))) float As[ROWS][SBK + 4];
+    __shared__ __attribute__((aligned(16))) float Ws[SBN][SBK + 4];
+    const int tid = threadIdx.x;
+    const int n0 = blockIdx.x * SBN;
+    const int nc = tid % 16, mg = tid / 16;                   // columns nc and nc + 16; rows mg + 16 j
+    float acc[MR][2];
+#pragma unroll
+    for (int j = 0; j < MR; j++) acc[j][0] = acc[j][1] = 0.f;
+    // what a thread fetches of a step: element e of the tiles, row e / SBK, column e % SBK
+    constexpr int WN = SBN * SBK / 256, AN = ROWS * SBK / 256;
+    float rw[WN], ra[AN];
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < WN; i++) {
+            const int e = tid + i * 256, r = e / SBK, k = k0 + e % SBK, n = n0 + r;
+            rw[i] = (n < N && k < K) ? to_f32(w[(size_t)n * ldw + k]) : 0.f;
+        }
+#pragma unroll
+        for (int i = 0; i < AN; i++) {
+            const int e = tid + i * 256, r = e / SBK, k = k0 + e % SBK;
+            ra[i] = (r < M && k < K) ? to_f32(a[(size_t)r * lda + k]) : 0.f;
+        }
+    };
+    fetch(0);
+    for (int k0 = 0; k0 < K; k0 += SBK) {
+        __syncthreads();                                      // the step before is no longer read
+#pragma unroll
+        for (int i = 0; i < WN; i++) { const int e = tid + i * 256; Ws[e / SBK][e % SBK] = rw[i]; }
+#pragma unroll
+        for (int i = 0; i < AN; i++) { const int e = tid + i * 256; As[e / SBK][e % SBK] = ra[i]; }
+        __syncthreads();
+        if (k0 + SBK < K) fetch(k0 + SBK);
+#pragma unroll 4
+        for (int kk = 0; kk < SBK; kk += 4) {
+            const float4 w0 = *reinterpret_cast<const float4*>(&Ws[nc][kk]);
+            const float4 w1 = *reinterpret_cast<const float4*>(&Ws[nc + 16][kk]);
+#pragma unroll
+            for (int j = 0; j < MR; j++) {
+                const float4 av = *reinterpret_cast<const float4*>(&As[mg + 16 * j][kk]);
+                acc[j][0] = fmaf(av.x, w0.x, acc[j][0]); acc[j][1] = fmaf(av.x, w1.x, acc[j][1]);
+                acc[j][0] = fmaf(av.y, w0.y, acc[j][0]); acc[j][1] = fmaf(av.y, w1.y, acc[j][1]);
+                acc[j][0] = fmaf(av.z, w0.z, acc[j][0]); acc[j][1] = fmaf(av.z, w1.z, acc[j][1]);
+                acc[j][0] = fmaf(av.w, w0.w, acc[j][0]); acc[j][1] = fmaf(av.w, w1.w, acc[j][1]);
+            }
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < MR; j++) {
+        const int m = mg + 16 * j;
+        if (m >= M) continue;
+#pragma unroll
+        for (int c = 0; c < 2; c++) {
+            const int n = n0 + nc + 16 * c;
+            if (n >= N) continue;
+            float v = acc[j][c] + (bias ? bias[n] : 0.f);
+            TO* dst = out + (size_t)m * ldo + n;
+            if (ACC) v += to_f32(*dst);
+            *dst = from_f32<TO>(v);
+        }
+    }
+}
+
+template <typename TA, typename TW, int MR>
+static int launch_rows(const GemmArgs& g) {
+    const dim3 grid((g.N + SBN - 1) / SBN);
+    const TA* a = (const TA*)g.a;
+    const TW* w = (const TW*)g.w;
+    if (g.out_dtype == HFA_F32) {
+        if (g.accumulate)
+            gemm_generic_rows_kernel<TA, TW, float, true, MR><<<grid, 256, 0, g.stream>>>(a, g.lda, w, g.ldw, g.bias, (float*)g.out, g.ldo, g.M, g.N, g.K);
+        else
+            gemm_generic_rows_kernel<TA, TW, float, false, MR><<<grid, 256, 0, g.stream>>>(a, g.lda, w, g.ldw, g.bias, (float*)g.out, g.ldo, g.M, g.N, g.K);
+    } else {
+        gemm_generic_rows_kernel<TA, TW, bf16, false, MR><<<grid, 256, 0, g.stream>>>(a, g.lda, w, g.ldw, g.bias, (bf16*)g.out, g.ldo, g.M, g.N, g.K);
+    }
+    HFA_LAUNCH_CHECK("gemm_generic_rows");
+    return 0;
+}
+
 template <typename TA, typename TW>
 static int launch_out(const GemmArgs& g) {
+    if (g.M <= 16) return launch_rows<TA, TW, 1>(g);
+    if (g.M <= 32) return launch_rows<TA, TW, 2>(g);
+    if (g.M <= 64) return launch_rows<TA, TW, 4>(g);
     dim3 grid((g.N + GBN - 1) / GBN, (g.M + GBM - 1) / GBM);
     const TA* a = (const TA*)g.a;
     const TW* w = (const TW*)g.w;

@@ -94,6 +94,25 @@ def test_gemm(ops32, adt, wdt, odt, M, N, K):
         assert float(wide[:, N:].abs().max()) == 0.0
 
 
+@pytest.mark.parametrize("N,K", [(100, 333), (1000, 3584), (37, 18944)])
+def test_fp32_rows_do_not_depend_on_the_batch(ops32, N, K):
+    """The 32-bit product sums every output in ascending k whatever the number of rows (few rows
+    take a kernel of their own): a row gives the same bits alone, among 7, 20, 50 and 200 rows."""
+    rng = np.random.default_rng(N + K)
+    a = rng.standard_normal((200, K)).astype(np.float32)
+    w = (rng.standard_normal((N, K)) / math.sqrt(K)).astype(np.float32)
+    b = rng.standard_normal(N).astype(np.float32)
+    da, dw, db = dev(a), dev(w), dev(b)
+    whole = torch.empty((200, N), dtype=torch.float32, device="cuda")
+    ops32.gemm(da, dw, whole, bias=db)
+    want = a.astype(np.float64) @ w.astype(np.float64).T + b
+    assert np.max(np.abs(whole.cpu().numpy() - want)) <= 2e-5 * max(1.0, np.max(np.abs(want)))
+    for M in (1, 7, 20, 50, 64):
+        part = torch.empty((M, N), dtype=torch.float32, device="cuda")
+        ops32.gemm(da[:M], dw, part, bias=db)
+        assert torch.equal(part, whole[:M]), f"{M} rows differ from the same rows among 200"
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 256, 512), (8, 4608, 3584), (8, 3584, 18944), (33, 200, 1000),
                                    (64, 1000, 4096), (65, 129, 72), (200, 333, 264), (500, 1100, 1024),
                                    (2048, 512, 3584), (2048, 4608, 1024), (1000, 8200, 512), (700, 5408, 640),

@@ -1,7 +1,8 @@
 // The plain matrix product: out[m, n] (+)= sum_k a[m, k] * w[n, k] + bias[n] with fp32
 // fused multiply-add in ascending k for every output element, whatever M is. It serves the
 // 32-bit path (no reduced-precision matrix mode) and every shape the MFMA kernels refuse.
-// 64x64 output tile per 256-thread block, K in steps of 16 through LDS, 4x4 outputs a thread.
+// 64x64 or 128x128 output tile per 256-thread block, K in steps of 16 through LDS, 4x4 or 8x8 outputs a
+// thread; few rows have a kernel of their own further down.
 #include "common.h"
 #include "gemm_internal.h"
 
@@ -9,53 +10,74 @@
 #define GBN 64
 #define GBK 16
 
-template <typename TA, typename TW, typename TO, bool ACC>
+template <typename TA, typename TW, typename TO, bool ACC, int T>
 __global__ __launch_bounds__(256) void gemm_generic_kernel(const TA* __restrict__ a, int lda,
                                                            const TW* __restrict__ w, int ldw,
                                                            const float* __restrict__ bias, TO* __restrict__ out,
                                                            int ldo, int M, int N, int K) {
-    __shared__ float As[GBK][GBM + 4];
-    __shared__ float Ws[GBK][GBN + 4];
+    constexpr int BMN = 16 * T;                               // the tile's rows and columns: T x T outputs a thread
+    __shared__ __attribute__((aligned(16))) float As[GBK][BMN + 4];
+    __shared__ __attribute__((aligned(16))) float Ws[GBK][BMN + 4];
     const int tid = threadIdx.x;
-    const int m0 = blockIdx.y * GBM, n0 = blockIdx.x * GBN;
+    const int m0 = blockIdx.y * BMN, n0 = blockIdx.x * BMN;
     const int tx = tid % 16, ty = tid / 16;
     const int lr = tid / 4, lk = (tid % 4) * 4;
-    float acc[4][4];
+    float acc[T][T];
 #pragma unroll
-    for (int i = 0; i < 4; i++)
+    for (int i = 0; i < T; i++)
 #pragma unroll
-        for (int j = 0; j < 4; j++) acc[i][j] = 0.f;
+        for (int j = 0; j < T; j++) acc[i][j] = 0.f;
 
-    for (int k0 = 0; k0 < K; k0 += GBK) {
-        const int m = m0 + lr, n = n0 + lr;
+    // the next step's values travel in registers while this step is multiplied
+    constexpr int NL = BMN / 64 * 4;
+    float ra[NL], rw[NL];
+    auto fetch = [&](int k0) {
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int k = k0 + lk + i;
-            As[lk + i][lr] = (m < M && k < K) ? to_f32(a[(size_t)m * lda + k]) : 0.f;
-            Ws[lk + i][lr] = (n < N && k < K) ? to_f32(w[(size_t)n * ldw + k]) : 0.f;
+        for (int r0 = 0; r0 < BMN; r0 += 64) {
+            const int m = m0 + r0 + lr, n = n0 + r0 + lr;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int k = k0 + lk + i;
+                ra[r0 / 16 + i] = (m < M && k < K) ? to_f32(a[(size_t)m * lda + k]) : 0.f;
+                rw[r0 / 16 + i] = (n < N && k < K) ? to_f32(w[(size_t)n * ldw + k]) : 0.f;
+            }
         }
+    };
+    fetch(0);
+    for (int k0 = 0; k0 < K; k0 += GBK) {
+#pragma unroll
+        for (int r0 = 0; r0 < BMN; r0 += 64)
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                As[lk + i][r0 + lr] = ra[r0 / 16 + i];
+                Ws[lk + i][r0 + lr] = rw[r0 / 16 + i];
+            }
         __syncthreads();
+        if (k0 + GBK < K) fetch(k0 + GBK);
 #pragma unroll
         for (int kk = 0; kk < GBK; kk++) {
-            float av[4], wv[4];
+            float av[T], wv[T];
 #pragma unroll
-            for (int i = 0; i < 4; i++) av[i] = As[kk][ty * 4 + i];
+            for (int i = 0; i < T; i += 4) {
+                const float4 v = *reinterpret_cast<const float4*>(&As[kk][ty * T + i]);
+                av[i] = v.x; av[i + 1] = v.y; av[i + 2] = v.z; av[i + 3] = v.w;
+                const float4 u = *reinterpret_cast<const float4*>(&Ws[kk][tx * T + i]);
+                wv[i] = u.x; wv[i + 1] = u.y; wv[i + 2] = u.z; wv[i + 3] = u.w;
+            }
 #pragma unroll
-            for (int j = 0; j < 4; j++) wv[j] = Ws[kk][tx * 4 + j];
+            for (int i = 0; i < T; i++)
 #pragma unroll
-            for (int i = 0; i < 4; i++)
-#pragma unroll
-                for (int j = 0; j < 4; j++) acc[i][j] = fmaf(av[i], wv[j], acc[i][j]);
+                for (int j = 0; j < T; j++) acc[i][j] = fmaf(av[i], wv[j], acc[i][j]);
         }
         __syncthreads();
     }
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const int m = m0 + ty * 4 + i;
+    for (int i = 0; i < T; i++) {
+        const int m = m0 + ty * T + i;
         if (m >= M) continue;
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const int n = n0 + tx * 4 + j;
+        for (int j = 0; j < T; j++) {
+            const int n = n0 + tx * T + j;
             if (n >= N) continue;
             float v = acc[i][j] + (bias ? bias[n] : 0.f);
             TO* dst = out + (size_t)m * ldo + n;
@@ -158,27 +180,35 @@ static int launch_rows(const GemmArgs& g) {
     return 0;
 }
 
+template <typename TA, typename TW, int T>
+static int launch_tiles(const GemmArgs& g) {
+    dim3 grid((g.N + 16 * T - 1) / (16 * T), (g.M + 16 * T - 1) / (16 * T));
+    const TA* a = (const TA*)g.a;
+    const TW* w = (const TW*)g.w;
+    if (g.out_dtype == HFA_F32) {
+        if (g.accumulate)
+            gemm_generic_kernel<TA, TW, float, true, T><<<grid, 256, 0, g.stream>>>(a, g.lda, w, g.ldw, g.bias,
+                                                                                   (float*)g.out, g.ldo, g.M, g.N, g.K);
+        else
+            gemm_generic_kernel<TA, TW, float, false, T><<<grid, 256, 0, g.stream>>>(a, g.lda, w, g.ldw, g.bias,
+                                                                                    (float*)g.out, g.ldo, g.M, g.N, g.K);
+    } else {
+        gemm_generic_kernel<TA, TW, bf16, false, T><<<grid, 256, 0, g.stream>>>(a, g.lda, w, g.ldw, g.bias,
+                                                                               (bf16*)g.out, g.ldo, g.M, g.N, g.K);
+    }
+    HFA_LAUNCH_CHECK("gemm_generic");
+    return 0;
+}
+
 template <typename TA, typename TW>
 static int launch_out(const GemmArgs& g) {
     if (g.M <= 16) return launch_rows<TA, TW, 1>(g);
     if (g.M <= 32) return launch_rows<TA, TW, 2>(g);
     if (g.M <= 64) return launch_rows<TA, TW, 4>(g);
-    dim3 grid((g.N + GBN - 1) / GBN, (g.M + GBM - 1) / GBM);
-    const TA* a = (const TA*)g.a;
-    const TW* w = (const TW*)g.w;
-    if (g.out_dtype == HFA_F32) {
-        if (g.accumulate)
-            gemm_generic_kernel<TA, TW, float, true><<<grid, 256, 0, g.stream>>>(a, g.lda, w, g.ldw, g.bias,
-                                                                                (float*)g.out, g.ldo, g.M, g.N, g.K);
-        else
-            gemm_generic_kernel<TA, TW, float, false><<<grid, 256, 0, g.stream>>>(a, g.lda, w, g.ldw, g.bias,
-                                                                                 (float*)g.out, g.ldo, g.M, g.N, g.K);
-    } else {
-        gemm_generic_kernel<TA, TW, bf16, false><<<grid, 256, 0, g.stream>>>(a, g.lda, w, g.ldw, g.bias,
-                                                                            (bf16*)g.out, g.ldo, g.M, g.N, g.K);
-    }
-    HFA_LAUNCH_CHECK("gemm_generic");
-    return 0;
+    // Tiles of 128 x 128 (8 x 8 outputs a thread: half the LDS reads per multiply-add) where there are
+    // enough of them for the machine, else 64 x 64.
+    if ((long)((g.N + 127) / 128) * ((g.M + 127) / 128) >= 256) return launch_tiles<TA, TW, 8>(g);
+    return launch_tiles<TA, TW, 4>(g);
 }
 
 int gemm_generic_launch(const GemmArgs& g) {

@@ -19,6 +19,7 @@ import numpy as np
 import torch
 
 from ..status import EINVAL, fail
+from .mathx import hfc_expf
 
 TOPK_KERNEL_MAX = 1024
 f32 = np.float32
@@ -56,7 +57,7 @@ def pick_rows(ids, logits, params, rngs):
     ids = np.asarray(ids)
     R, k = logits.shape
     col = np.arange(k)[None, :]
-    p = np.exp((logits - logits[:, :1]) / f32(params.temp), dtype=f32)
+    p = hfc_expf((logits - logits[:, :1]) / f32(params.temp))               # src/sample.c:99, src/mathx.c:7-32
     p = (p / np.cumsum(p, axis=1, dtype=f32)[:, -1:]).astype(f32)
     kept = np.full(R, k)
     if params.min_p > 0:

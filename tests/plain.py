@@ -200,6 +200,31 @@ class Rng:
         return np.float32(((x * 0x2545f4914f6cdd1d) & MASK64) >> 40) / np.float32(16777216.0)
 
 
+def expf(x):
+    """The reference's own exponential, src/mathx.c:7-32, one fp32 operation at a time: exp(x) =
+    2^n exp(r), n = floor(x log2(e) + 1/2), r = x - n ln2 taken off in two parts, exp(r) by a
+    polynomial of degree 7. The sampler's probabilities come from this routine (src/sample.c:99),
+    and a draw can turn on their last bit."""
+    f = np.float32
+    x = f(x)
+    if x != x:
+        return x
+    if x > f(88.3762626647949):
+        x = f(88.3762626647949)
+    if x < f(-87.3365478515625):
+        return f(0.0)
+    fx = f(math.floor(f(f(x * f(1.44269504088896341)) + f(0.5))))
+    n = int(fx)
+    x = f(x - f(fx * f(0.693359375)))
+    x = f(x - f(fx * f(-2.12194440e-4)))
+    z = f(x * x)
+    y = f(1.9875691500e-4)
+    for c in (1.3981999507e-3, 8.3334519073e-3, 4.1665795894e-2, 1.6666665459e-1, 5.0000001201e-1):
+        y = f(f(y * x) + f(c))
+    y = f(f(f(y * z) + x) + f(1.0))
+    return f(y * f(math.ldexp(1.0, n)))
+
+
 def sample(logits, temp, top_k, top_p, min_p, rng):
     """src/sample.c:66-117: greedy when temp <= 0 (first index of the maximum); else sort by
     (logit descending, id ascending), keep top_k, p = exp((l - max)/temp) normalised in fp32,
@@ -212,7 +237,7 @@ def sample(logits, temp, top_k, top_p, min_p, rng):
         order = order[:top_k]
     f = np.float32
     mx = logits[order[0]]
-    p = [f(np.exp(f((logits[i] - mx) / f(temp)))) for i in order]
+    p = [expf(f(f(logits[i] - mx) / f(temp))) for i in order]
     total = f(0)
     for v in p:
         total = f(total + v)

@@ -149,3 +149,22 @@ def test_sampler_of_the_plain_implementation():
     assert all(plain.sample(logits, 1.0, 0, 0.6, 0.0, rng) in (0, 1) for _ in range(50))  # top-p 0.6
     assert all(plain.sample(logits, 1.0, 0, 1.0, 0.4, rng) in (0, 1) for _ in range(50))  # min-p 0.4
     assert abs(plain.logprob(logits, 1) - math.log(0.25)) < 1e-6
+
+
+def test_exponential_of_the_reference():
+    """The checks that the reference's own test holds for its exponential (tests/test_kern.c:21-32):
+    relative error below 4e-7 from -87 to 88 in steps of 0.0137, exp(0) = 1, exp(-100) = 0, a finite
+    value for 1000. The product's vectorised routine gives the same bits as the plain one."""
+    import math
+    from hf_cpu_amd.sampling.mathx import hfc_expf
+    xs = np.arange(-87.0, 88.0, 0.0137, dtype=np.float32)
+    got = np.array([plain.expf(x) for x in xs], dtype=np.float32)
+    ref = np.exp(xs.astype(np.float64))
+    assert np.max(np.abs(got.astype(np.float64) - ref) / ref) < 4e-7
+    assert plain.expf(0.0) == 1.0 and plain.expf(-100.0) == 0.0 and math.isfinite(plain.expf(1000.0))
+    assert np.array_equal(hfc_expf(xs), got)
+    edge = np.array([0.0, -0.0, -100.0, 1000.0, -87.3365478515625, -87.33655, 88.3762626647949, 1e-30, -1e-30], np.float32)
+    assert np.array_equal(hfc_expf(edge), np.array([plain.expf(x) for x in edge], dtype=np.float32))
+    rng = np.random.default_rng(0)
+    more = (rng.standard_normal(20000) * 20).astype(np.float32)
+    assert np.array_equal(hfc_expf(more), np.array([plain.expf(x) for x in more], dtype=np.float32))

@@ -91,6 +91,12 @@ size_t hfa_order_rows_scratch(int n_rows, int vocab);
 int hfa_order_rows(const float* logits, int ld, const int* rows, int* ids, float* vals, int n_rows, int vocab,
                    void* scratch, size_t scratch_bytes, hipStream_t stream);
 
+// The draw over ordered rows (src/sample.c:99-114): vals/ids [n_rows, vocab] as hfa_order_rows leaves them,
+// params[r] = {temp, top_p, min_p, u} with u the request's uniform number in [0, 1), cuts[r] = candidates
+// left by top-k (1..vocab). tokens[r] = the drawn id. vals is overwritten with the probabilities.
+int hfa_draw_rows(float* vals, const int* ids, int n_rows, int vocab, const float* params, const int* cuts,
+                  int* tokens, hipStream_t stream);
+
 // The k best of each row in the order (logit descending, id ascending) (src/sample.c:59-64),
 // and stats[r] = {max, log(sum(exp(l - max)))} (src/sample.c:25-33). k <= 1024.
 int hfa_topk(const float* logits, int ld, int* ids, float* vals, float* stats, int n_rows, int vocab, int k,

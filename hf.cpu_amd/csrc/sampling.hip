@@ -382,3 +382,115 @@ extern "C" int hfa_order_rows(const float* logits, int ld, const int* rows, int*
     HFA_LAUNCH_CHECK("order_rows");
     return 0;
 }
+
+// ---- the draw over a whole ordered row ---------------------------------------------------------
+// Steps 3 to 6 of the reference's sampler (src/sample.c:99-114) over candidates that are already
+// in order: p = exp((l - l_0) / temp) by the reference's own exponential (src/mathx.c:7-32, every
+// operation rounded to fp32, nothing fused), the sum of all p as one running fp32 sum in candidate
+// order, p / sum, the min-p and top-p cuts, r = u * (running sum of the kept), the first
+// candidate whose running sum exceeds r. The running sums are what the reference's loops compute,
+// so they are made by one thread, which reads the row from LDS in pieces that all threads fetch;
+// everything else is spread over the block. `vals` is overwritten with the probabilities.
+#define DRAW_THREADS 1024
+#define DRAW_PIECE 4096
+
+__device__ __forceinline__ float ref_expf(float x) {
+    if (x != x) return x;
+    if (x > 88.3762626647949f) x = 88.3762626647949f;
+    if (x < -87.3365478515625f) return 0.0f;
+    const float fx = floorf(__fadd_rn(__fmul_rn(x, 1.44269504088896341f), 0.5f));
+    const int n = (int)fx;
+    x = __fsub_rn(x, __fmul_rn(fx, 0.693359375f));
+    x = __fsub_rn(x, __fmul_rn(fx, -2.12194440e-4f));
+    const float z = __fmul_rn(x, x);
+    float y = 1.9875691500e-4f;
+    y = __fadd_rn(__fmul_rn(y, x), 1.3981999507e-3f);
+    y = __fadd_rn(__fmul_rn(y, x), 8.3334519073e-3f);
+    y = __fadd_rn(__fmul_rn(y, x), 4.1665795894e-2f);
+    y = __fadd_rn(__fmul_rn(y, x), 1.6666665459e-1f);
+    y = __fadd_rn(__fmul_rn(y, x), 5.0000001201e-1f);
+    y = __fadd_rn(__fadd_rn(__fmul_rn(y, z), x), 1.0f);
+    return __fmul_rn(y, __uint_as_float((uint32_t)(n + 127) << 23));
+}
+
+// One thread's running sum of p[0 .. n) in order, started from `start`; stops after the first element
+// at which `stop(sum)` holds (returns its index, else n). The pieces pass through `piece` (LDS).
+template <class Stop>
+__device__ int draw_running(const float* __restrict__ p, int n, float start, float* piece, float* shared2, Stop stop) {
+    int hit = n;
+    float sum = start;
+    for (int c0 = 0; c0 < n; c0 += DRAW_PIECE) {
+        const int len = n - c0 < DRAW_PIECE ? n - c0 : DRAW_PIECE;
+        __syncthreads();                                      // the piece before is summed
+        for (int i = threadIdx.x; i < len; i += DRAW_THREADS) piece[i] = p[c0 + i];
+        __syncthreads();
+        if (threadIdx.x == 0 && hit == n) {
+            for (int i = 0; i < len; i++) {
+                sum = __fadd_rn(sum, piece[i]);
+                if (stop(sum)) { hit = c0 + i; break; }
+            }
+            shared2[0] = sum;
+            shared2[1] = __int_as_float(hit);
+        }
+        __syncthreads();
+        hit = __float_as_int(shared2[1]);                     // every thread leaves the loop together
+        if (hit != n) break;
+    }
+    __syncthreads();
+    return hit;                                               // the sum is in shared2[0]
+}
+
+__global__ __launch_bounds__(DRAW_THREADS) void draw_rows_kernel(float* __restrict__ vals, const int* __restrict__ ids,
+                                                                 int vocab, const float* __restrict__ params,
+                                                                 const int* __restrict__ cuts, int* __restrict__ tokens) {
+    __shared__ float piece[DRAW_PIECE];
+    __shared__ float shared2[2];
+    __shared__ int first_below;
+    const int row = blockIdx.x, tid = threadIdx.x;
+    float* p = vals + (size_t)row * vocab;
+    const int* id = ids + (size_t)row * vocab;
+    const float temp = params[4 * row], top_p = params[4 * row + 1], min_p = params[4 * row + 2], u = params[4 * row + 3];
+    const int m = cuts[row];                                  // candidates after the top-k cut
+    const float l0 = p[0];
+    __syncthreads();                                          // p[0] is read by all before it is overwritten
+    for (int i = tid; i < m; i += DRAW_THREADS) p[i] = ref_expf(__fdiv_rn(__fsub_rn(p[i], l0), temp));
+    __threadfence_block();
+    draw_running(p, m, 0.0f, piece, shared2, [](float) { return false; });
+    const float total = shared2[0];
+    __syncthreads();
+    for (int i = tid; i < m; i += DRAW_THREADS) p[i] = __fdiv_rn(p[i], total);
+    if (tid == 0) first_below = m;
+    __threadfence_block();
+    __syncthreads();
+    int kept = m;
+    if (min_p > 0.0f) {                                       // the leading run with p >= min_p * p_0, at least one
+        const float least = __fmul_rn(min_p, p[0]);
+        int mine = m;
+        for (int i = tid; i < m; i += DRAW_THREADS)
+            if (p[i] < least) { mine = i; break; }            // a thread's indices ascend: its first is its least
+        if (mine < m) atomicMin(&first_below, mine);
+        __syncthreads();
+        kept = first_below > 0 ? first_below : 1;
+    }
+    float sum;
+    if (top_p > 0.0f && top_p < 1.0f) {
+        const int at = draw_running(p, kept, 0.0f, piece, shared2, [top_p](float s) { return s >= top_p; });
+        if (at < kept) kept = at + 1;
+        sum = shared2[0];                                     // the running sum over the kept, either way
+    } else {
+        draw_running(p, kept, 0.0f, piece, shared2, [](float) { return false; });
+        sum = shared2[0];
+    }
+    __syncthreads();
+    const float r = __fmul_rn(u, sum);
+    const int at = draw_running(p, kept, 0.0f, piece, shared2, [r](float s) { return r < s; });
+    if (tid == 0) tokens[row] = id[at < kept ? at : kept - 1];
+}
+
+extern "C" int hfa_draw_rows(float* vals, const int* ids, int n_rows, int vocab, const float* params, const int* cuts,
+                             int* tokens, hipStream_t stream) {
+    HFA_REQUIRE(n_rows > 0 && vocab > 0, "draw_rows: bad sizes rows=%d vocab=%d", n_rows, vocab);
+    draw_rows_kernel<<<n_rows, DRAW_THREADS, 0, stream>>>(vals, ids, vocab, params, cuts, tokens);
+    HFA_LAUNCH_CHECK("draw_rows");
+    return 0;
+}

@@ -373,6 +373,20 @@ class Ops:
                                             vals.data_ptr(), n, V, scratch.data_ptr(), need, self._stream()))
         return ids, vals
 
+    def draw_rows(self, ids, vals, params, cuts):
+        """tokens [n] int32 drawn from rows that ``order_rows`` put in order: ``params`` [n, 4] fp32 =
+        (temp, top_p, min_p, uniform number), ``cuts`` [n] int32 = candidates left by top-k. ``vals``
+        is overwritten with the probabilities."""
+        n, V = vals.shape
+        if vals.dtype != torch.float32 or not vals.is_contiguous() or ids.shape != vals.shape:
+            fail(EINVAL, "draw_rows: expected contiguous fp32 values and ids of one shape")
+        if params.dtype != torch.float32 or not params.is_contiguous() or tuple(params.shape) != (n, 4):
+            fail(EINVAL, f"draw_rows: expected [{n}, 4] fp32 parameters")
+        tokens = torch.empty((n,), dtype=torch.int32, device=vals.device)
+        self._check(self.lib.hfa_draw_rows(vals.data_ptr(), _ints(ids, "draw_rows ids", n * V), n, V, params.data_ptr(),
+                                           _ints(cuts, "draw_rows cuts", n), tokens.data_ptr(), self._stream()))
+        return tokens
+
     def topk(self, logits, k, want_stats=True):
         """(ids [R, k] int32, values [R, k] fp32, stats [R, 2] fp32 = max and log-sum-exp
         above the max), candidates in the order (logit descending, id ascending)."""

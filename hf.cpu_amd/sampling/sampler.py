@@ -10,9 +10,10 @@ one draw ``r = uniform * sum`` picks the first candidate whose running sum excee
 The GPU does the part that touches the whole vocabulary (argmax; the ordered best-k and
 the row's log-sum-exp, kernels in csrc/sampling.hip); the few candidates left are finished
 on the host in fp32 in exactly the order above. With ``top_k`` off (0) or beyond the
-kernel's 1024 the row is copied and ordered on the host.
+best-k kernel's 1024 the device orders the whole row and draws from it itself, by the same
+fp32 operations in the same order as ``pick_rows``, which stays the statement of the draw
+and what the tests compare the kernel with.
 """
-from concurrent.futures import ThreadPoolExecutor
 from dataclasses import dataclass
 
 import numpy as np
@@ -121,32 +122,31 @@ class Sampler:
             ids, vals, stats = (t.cpu().numpy() for t in self.ops.topk(logits, need_k))
         toks = [None] * R
         groups = {}                               # rows drawn from the device's candidates, by parameters
-        on_host = []                              # rows whose whole vocabulary is put in order on the host
+        whole = []                                # rows drawn from the whole vocabulary, in order, on the device
         for i, (params, rng, n_lp) in enumerate(wants):
             if params.greedy:
                 toks[i] = int(arg[i])
             elif 0 < params.top_k <= TOPK_KERNEL_MAX and params.top_k < logits.shape[1]:
                 groups.setdefault(params, []).append(i)
             else:
-                on_host.append(i)
-        if on_host:
-            # The device puts the whole vocabulary of these rows in order; the draw over so many
-            # candidates takes about a millisecond a row in numpy, outside the interpreter's lock,
-            # so the rows are drawn side by side.
-            chosen = None if len(on_host) == R else torch.tensor(on_host, dtype=torch.int32, device=logits.device)
-            all_ids, all_vals = (t.cpu().numpy() for t in self.ops.order_rows(logits, chosen))
-
-            def draw(j):
-                params, rng, _ = wants[on_host[j]]
-                k = params.top_k if 0 < params.top_k < all_ids.shape[1] else all_ids.shape[1]
-                return pick(all_ids[j, :k], all_vals[j, :k], params, rng)
-
-            if len(on_host) == 1:
-                toks[on_host[0]] = draw(0)
-            else:
-                with ThreadPoolExecutor(max_workers=min(16, len(on_host))) as pool:
-                    for i, t in zip(on_host, pool.map(draw, range(len(on_host)))):
-                        toks[i] = t
+                whole.append(i)
+        if whole:
+            # The device puts the whole vocabulary of these rows in order and draws from it
+            # (csrc/sampling.hip: the same fp32 operations in the same order as ``pick_rows``);
+            # the host gives each request's uniform number and reads back one token a row.
+            V = logits.shape[1]
+            chosen = None if len(whole) == R else torch.tensor(whole, dtype=torch.int32, device=logits.device)
+            all_ids, all_vals = self.ops.order_rows(logits, chosen)
+            numbers = np.empty((len(whole), 4), dtype=f32)
+            cuts = np.empty(len(whole), dtype=np.int32)
+            for j, i in enumerate(whole):
+                params, rng, _ = wants[i]
+                numbers[j] = (params.temp, params.top_p, params.min_p, rng.uniform())
+                cuts[j] = params.top_k if 0 < params.top_k < V else V
+            drawn = self.ops.draw_rows(all_ids, all_vals, torch.from_numpy(numbers).to(logits.device),
+                                       torch.from_numpy(cuts).to(logits.device)).cpu().numpy()
+            for i, t in zip(whole, drawn):
+                toks[i] = int(t)
         for params, rows in groups.items():
             drawn = pick_rows(ids[rows, :params.top_k], vals[rows, :params.top_k], params, [wants[i][1] for i in rows])
             for i, t in zip(rows, drawn):

@@ -86,6 +86,12 @@ def test_sampling_is_reproducible_and_follows_the_plain_sampler(gpu, models):
         top = sorted(range(len(row)), key=lambda j: (-row[j], j))[:3]
         assert [j for j, _ in a[0].top[i]] == top
         toks.append(t)
+    # top-k off: the device draws from the whole vocabulary in order; the plain sampler again
+    whole = s.generate(prompt, n=1, temp=1.1, top_k=0, top_p=0.9, min_p=0.01, seed=5, max_tokens=16)[0].tokens
+    rng, toks = plain.Rng(5), list(prompt)
+    for i, t in enumerate(whole):
+        assert plain.sample(plain.forward(pcfg, w, toks)[-1], 1.1, 0, 0.9, 0.01, rng) == t, f"top-k off, token {i}"
+        toks.append(t)
 
 
 @pytest.mark.parametrize("name,length", [("A", 21), ("B", 43), ("B", 150)])

@@ -637,6 +637,46 @@ def test_order_rows(ops32, V):
             assert np.array_equal(vals[j], logits[r][want])           # == : the kernel returns 0.0 for -0.0
 
 
+@pytest.mark.parametrize("V", [1, 7, 1000, 4097, 152064])
+def test_draw_rows(ops32, V):
+    """The device's draw over a whole ordered row against the sampler's written-out draw on the same
+    candidates with the same uniform numbers: the same token, row for row. The rows differ in
+    temperature, in each cut being on or off, and in how peaked they are (a peaked row ends the
+    top-p cut within a few candidates, a flat one takes it far into the row: past several of the
+    kernel's pieces); uniform numbers include 0 and the largest below 1."""
+    from hf_cpu_amd.sampling import SamplerParams, pick
+    rng = np.random.default_rng(V + 1)
+
+    class Fixed:
+        def __init__(self, u):
+            self.u = u
+
+        def uniform(self):
+            return self.u
+
+    cases = []
+    for temp in (0.05, 0.8, 1.0, 4.5):
+        for top_k in (0, 3, 2000):
+            for top_p in (0.0, 0.3, 0.95, 1.0):
+                for min_p in (0.0, 0.05, 0.9):
+                    cases.append((temp, top_k, top_p, min_p))
+    rng.shuffle(cases)
+    cases = cases[:96]
+    R = len(cases)
+    logits = rng.standard_normal((R, V)).astype(np.float32) * rng.choice([0.01, 1.0, 6.0], (R, 1)).astype(np.float32)
+    logits[::5] = np.round(logits[::5] * 2) / 2                          # rows with many ties
+    us = rng.integers(0, 1 << 24, R).astype(np.float32) / np.float32(1 << 24)
+    us[:4] = [0.0, (2.0 ** 24 - 1) / 2.0 ** 24, 0.5, 2.0 ** -24]
+    ids, vals = ops32.order_rows(torch.from_numpy(logits).cuda())
+    host_ids, host_vals = ids.cpu().numpy(), vals.cpu().numpy()
+    numbers = np.array([(t, tp, mp, u) for (t, _, tp, mp), u in zip(cases, us)], dtype=np.float32)
+    cuts = np.array([k if 0 < k < V else V for _, k, _, _ in cases], dtype=np.int32)
+    got = ops32.draw_rows(ids, vals, torch.from_numpy(numbers).cuda(), torch.from_numpy(cuts).cuda()).cpu().numpy()
+    for r, (temp, top_k, top_p, min_p) in enumerate(cases):
+        want = pick(host_ids[r, :cuts[r]], host_vals[r, :cuts[r]], SamplerParams(temp, top_k, top_p, min_p), Fixed(us[r]))
+        assert int(got[r]) == want, f"row {r}: temp {temp} top_k {top_k} top_p {top_p} min_p {min_p} u {us[r]}"
+
+
 def test_kernels_refuse_what_they_cannot_do(ops32):
     from hf_cpu_amd.status import EngineError
     with pytest.raises(EngineError, match="head_dim"):

@@ -677,6 +677,27 @@ def test_draw_rows(ops32, V):
         assert int(got[r]) == want, f"row {r}: temp {temp} top_k {top_k} top_p {top_p} min_p {min_p} u {us[r]}"
 
 
+def test_sampler_with_rows_of_every_kind_in_one_step(ops32):
+    """One call of the sampler for rows that take every one of its paths (greedy, the best-k
+    kernel, the whole vocabulary with top-k off, a top-k beyond the best-k kernel's 1024, greedy
+    with log-probabilities) gives each row what the plain sampler gives it alone, and moves each
+    request's generator on by one draw (two calls in a row are compared)."""
+    from hf_cpu_amd.sampling import Rng, Sampler, SamplerParams
+    rng = np.random.default_rng(77)
+    V = 3001
+    kinds = [(0.0, 40, 0.95, 0.05), (0.8, 40, 0.95, 0.05), (1.3, 0, 1.0, 0.0), (0.7, 2000, 0.9, 0.0), (0.0, 0, 1.0, 0.0),
+             (2.0, 0, 0.5, 0.02), (0.9, 1, 1.0, 0.0), (1.0, 1024, 1.0, 0.0), (1.0, 1025, 1.0, 0.0)]
+    wants = [(SamplerParams(*k), Rng(100 + i), 2 if i == 4 else 0) for i, k in enumerate(kinds)]
+    theirs = [plain.Rng(100 + i) for i in range(len(kinds))]
+    sampler = Sampler(ops32)
+    for call in range(2):
+        logits = (rng.standard_normal((len(kinds), V)) * 3).astype(np.float32)
+        got = sampler.sample(torch.from_numpy(logits).cuda(), wants)
+        for i, k in enumerate(kinds):
+            assert got[i].token == plain.sample(logits[i], *k, theirs[i]), f"call {call}, row {i}: {k}"
+        assert [t for t, _ in got[4].top] == [int(t) for t in np.argsort(-logits[4], kind="stable")[:2]]
+
+
 def test_kernels_refuse_what_they_cannot_do(ops32):
     from hf_cpu_amd.status import EngineError
     with pytest.raises(EngineError, match="head_dim"):

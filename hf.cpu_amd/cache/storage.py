@@ -26,23 +26,31 @@ class StateView:
 
 class CacheStorage:
     """Key/value rows for every schedule entry that stores, a block table per group
-    ([n_slots, max_blocks] int32, row = the request's slot), and the state rows."""
+    ([n_slots + 1, max_blocks] int32, row = the request's slot), and the state rows.
+
+    Beyond what the manager hands out there is one more page in every group (``pad_pages[g]``)
+    and one more slot (``pad_slot``) whose block tables begin with that page: rows that a step
+    adds to fill a batch up to a size it has a graph for live there, apart from every request."""
 
     def __init__(self, manager, dtype, device):
         self.manager = manager
         self.views = [None] * len(manager.entry_group)
         rows = None
         for g, pool in zip(manager.groups, manager.pools):
-            rows = pool.n_pages * manager.page_tokens
+            rows = (pool.n_pages + 1) * manager.page_tokens
             for e in g.entries:
                 self.views[e] = PagedView(g.index,
                                           torch.zeros((rows, g.k_width), dtype=dtype, device=device),
                                           torch.zeros((rows, g.v_width), dtype=dtype, device=device),
                                           manager.page_tokens, g.window)
         for e, n_floats in manager.state_entries.items():
-            self.views[e] = StateView(torch.zeros((manager.n_slots, n_floats), dtype=torch.float32, device=device))
-        self.block_tables = [torch.zeros((manager.n_slots, manager.max_blocks), dtype=torch.int32, device=device)
+            self.views[e] = StateView(torch.zeros((manager.n_slots + 1, n_floats), dtype=torch.float32, device=device))
+        self.block_tables = [torch.zeros((manager.n_slots + 1, manager.max_blocks), dtype=torch.int32, device=device)
                              for _ in manager.groups]
+        self.pad_slot = manager.n_slots
+        self.pad_pages = [pool.n_pages for pool in manager.pools]
+        for table, page in zip(self.block_tables, self.pad_pages):
+            table[self.pad_slot, 0] = page
 
     def clear_slot(self, slot):
         """State starts from zero for a newly admitted request."""

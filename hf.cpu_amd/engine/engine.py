@@ -17,6 +17,7 @@ from .batch import Entry, GroupInputs, IntStaging, StepInputs, as_i32
 class Engine:
     GRAPH_MAX_TOKENS = 256        # decode-only steps up to this many requests replay a captured graph
     GRAPH_LEN_BUCKET = 256        # a graph serves request lengths up to a multiple of this
+    BATCH_BUCKET = 8              # decode steps of more requests than this are filled up to a multiple of it
 
     def __init__(self, model, ops, page_tokens=16, n_pages=None, max_tokens=None, max_seqs=8,
                  max_context=None, graphs=True):
@@ -184,15 +185,33 @@ class Engine:
             for m in slot_maps:
                 assert m.min() >= 0, "a position about to be written has no page"
             seq_len = lengths + 1
-            rows = np.arange(S, dtype=np.int32)
-            q_start = np.arange(S + 1, dtype=np.int32)
             tokens = tokens.astype(np.int32)
+            # Requests come and go, so a serving loop sees every batch size; a graph per size would be
+            # captured and hardly ever replayed. Steps of more than BATCH_BUCKET requests are filled up
+            # to a multiple of it with rows that belong to no request: row i of them is position i of
+            # the storage's spare slot and spare page, which no request's block table names.
+            B = self.BATCH_BUCKET
+            pad = (-S) % B if S > B and not mgr.state_entries else 0
+            if pad > P or S + pad > self.GRAPH_MAX_TOKENS:
+                pad = 0
+            if pad:
+                extra = np.arange(pad, dtype=np.int32)
+                spare = np.full(pad, self.storage.pad_slot, np.int32)
+                tokens = np.concatenate([tokens, np.zeros(pad, np.int32)])
+                lengths = np.concatenate([lengths, extra])
+                slots = np.concatenate([slots, spare])
+                seq_len = np.concatenate([seq_len, extra + 1])
+                slot_maps = [np.concatenate([m, np.int32(page * P) + extra]) for m, page in zip(slot_maps, self.storage.pad_pages)]
+            N = S + pad
+            rows = np.arange(N, dtype=np.int32)
+            q_start = np.arange(N + 1, dtype=np.int32)
             arrays = [tokens, lengths, slots, q_start, slots, seq_len, rows, np.zeros(1, np.int32)] + slot_maps
-            step = self._upload(arrays, S, S, S, 1, int(seq_len.max()),
+            step = self._upload(arrays, N, N, N, 1, int(seq_len.max()),
                                 dict(tokens=tokens, positions=lengths, token_slot=slots, q_start=q_start,
-                                     seq_slot=slots, seq_len=seq_len, logit_rows=rows), short=(S, S, 1))
-            logits = self.ops.scratch("logits", (S, self.vocab_size), torch.float32)
+                                     seq_slot=slots, seq_len=seq_len, logit_rows=rows), short=(N, N, 1))
+            logits = self.ops.scratch("logits", (N, self.vocab_size), torch.float32)
             self._run(step, logits)
+            logits = logits[:S]
             if self.profile is not None:
                 self._book_times("decode")
         except BaseException:

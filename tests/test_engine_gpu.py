@@ -213,6 +213,46 @@ def test_graph_replay_equals_eager(gpu, tiny, dtype):
     helpers.compare(got, want, TOL[dtype], "graph replay")
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_batches_of_every_size_share_a_few_graphs(gpu, tmp_path, dtype):
+    """Nineteen requests decoded together that end one after another, so that every batch size
+    from 19 down to 1 occurs: every row against the plain implementation, and sizes above 8 are
+    filled up to a multiple of 8 with rows of no request (they live on a page and in a slot that
+    the manager never hands out), so that 24 and 16 are the only shapes captured for them. A
+    second pass over the same sizes replays, and gives the bits of the first."""
+    import hf_cpu_amd
+    cfg = helpers.CONFIG_B
+    d = helpers.make_model_dir(str(tmp_path / "m"), cfg, seed=3)
+    n_req = 19
+    lengths = [22 + (5 * i) % 13 + i for i in range(n_req)]               # request i ends after lengths[i] tokens
+    reqs = helpers.random_requests(cfg, lengths, seed=31)
+    want = helpers.plain_logits(d, reqs)
+    engine = hf_cpu_amd.load_engine(d, dtype=dtype, page_tokens=8, max_tokens=64 * n_req, max_seqs=n_req)
+    passes = []
+    for again in range(2):
+        got, sizes = {}, set()
+        for r, toks in reqs.items():
+            engine.step([(r, toks[:12], [])])
+        at = {r: 12 for r in reqs}
+        while at:
+            live = list(at)
+            logits = engine.step([(r, [reqs[r][at[r]]], [0]) for r in live]).float().cpu().numpy()
+            sizes.add(len(live))
+            for r, row in zip(live, logits):
+                got[(r, at[r])] = row.copy()
+                at[r] += 1
+                if at[r] == len(reqs[r]):
+                    del at[r]
+                    engine.release(r)
+        assert sizes == set(range(1, n_req + 1))
+        helpers.compare(got, want, TOL[dtype], "batches of every size")
+        passes.append(got)
+    assert all(np.array_equal(passes[0][k], passes[1][k]) for k in passes[0])
+    assert {key[0] for key in engine._graphs if key[0] > 8} <= {16, 24}
+    assert engine.graph_replays > 0
+    assert not engine.manager.held and all(p.n_held == 0 for p in engine.manager.pools)
+
+
 @pytest.mark.parametrize("seed", range(20))
 def test_random_configurations(gpu, tmp_path, seed):
     """Configurations drawn at random within what config.json allows (head sizes in steps of

@@ -82,11 +82,18 @@ extern "C" int hfa_argmax(const float* logits, int ld, int* out, int n_rows, int
     return 0;
 }
 
-// Ordered best-k of a row, one block of 1024 threads per row, in a fixed number of passes over
-// the row (which stays in L2) whatever k is:
+// Ordered best-k of a row, one block of 1024 threads per row.
+//
+// The short way, two passes over the row: the first finds every thread's own maximum (and from them
+// the row's); the k-th largest of these 1024 maxima cannot lie above the row's k-th largest value, so
+// the second pass, which also adds up exp(l - max) for the log-sum-exp, collects the values that
+// reach it: at least k, and for logits without heavy ties hardly more. If at most 1024 were
+// collected they are sorted in LDS by (logit descending, id ascending) and the first k are the answer.
+//
+// Otherwise (ties by the thousand, or a k near 1024) the long way, in a fixed number of passes
+// over the row (which stays in L2) whatever k is:
 //  1. the k-th largest value is found by three histogram passes over the order-preserving
-//     integer image of the floats (11 + 11 + 10 bits); pass 1 also finds the maximum, pass 2
-//     also adds up exp(l - max) for the log-sum-exp;
+//     integer image of the floats (11 + 11 + 10 bits);
 //  2. two sweeps collect the values above it and, of the values equal to it, those with the
 //     smallest ids until k are together: each wave owns a contiguous segment of the row and
 //     walks it 64 ids at a time, so ballots and counts give every candidate its place in id
@@ -131,6 +138,38 @@ __device__ int topk_find_bin(const uint32_t* hist, int n_bins, int& rank, int* p
     return pick[0];
 }
 
+// `found` candidates in LDS, sorted by (logit descending, id ascending) with a bitonic network over
+// n <= 1024 entries, one thread per entry; the first k go to the row's output. All threads call it.
+__device__ void topk_sort_and_store(float* cand_v, int* cand_i, int found, int k, int* __restrict__ ids,
+                                    float* __restrict__ vals) {
+    const int tid = threadIdx.x;
+    int n = 2;
+    while (n < found) n <<= 1;
+    for (int i = found + tid; i < n; i += TOPK_THREADS) {    // padding sorts to the end
+        cand_v[i] = -INFINITY;
+        cand_i[i] = 0x7fffffff;
+    }
+    for (int size = 2; size <= n; size <<= 1)
+        for (int stride = size >> 1; stride > 0; stride >>= 1) {
+            __syncthreads();
+            const int j = tid ^ stride;
+            if (tid < n && j > tid) {
+                const bool forward = (tid & size) == 0;      // this pair's better entry goes first
+                const float va = cand_v[tid], vb = cand_v[j];
+                const int ia = cand_i[tid], ib = cand_i[j];
+                if (better(vb, ib, va, ia) == forward) {
+                    cand_v[tid] = vb; cand_i[tid] = ib;
+                    cand_v[j] = va; cand_i[j] = ia;
+                }
+            }
+        }
+    __syncthreads();
+    for (int c = tid; c < k; c += TOPK_THREADS) {
+        ids[(size_t)blockIdx.x * k + c] = cand_i[c] == 0x7fffffff ? -1 : cand_i[c];
+        vals[(size_t)blockIdx.x * k + c] = cand_v[c];
+    }
+}
+
 __global__ __launch_bounds__(TOPK_THREADS) void topk_kernel(const float* __restrict__ logits, int ld,
                                                             int* __restrict__ ids, float* __restrict__ vals,
                                                             float* __restrict__ stats, int vocab, int k) {
@@ -144,29 +183,41 @@ __global__ __launch_bounds__(TOPK_THREADS) void topk_kernel(const float* __restr
     const int tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
     constexpr int NW = TOPK_THREADS / WAVE;
 
-    // ---- pass 1: top 11 bits, and the maximum ----
-    for (int i = tid; i < 2048; i += TOPK_THREADS) hist[i] = 0;
-    __syncthreads();
+    // ---- the row's maximum, and every thread's own ----
+    __shared__ int n_cand;
     float mx = -INFINITY;
-    for (int i = tid; i < vocab; i += TOPK_THREADS) {
-        const float v = row[i];
-        mx = fmaxf(mx, v);
-        if (k > 0) atomicAdd(&hist[float_key(v) >> 21], 1u);
-    }
+    for (int i = tid; i < vocab; i += TOPK_THREADS) mx = fmaxf(mx, row[i]);
+    const float own = mx;
     mx = block_max(mx, red);
-    uint32_t prefix = 0;
-    int rank = k;
-    if (k > 0) prefix = (uint32_t)topk_find_bin(hist, 2048, rank, pick);
+    float least = INFINITY;                                  // what a candidate of the short way has to reach
+    if (k > 0) {
+        cand_v[tid] = own;                                   // the 1024 maxima, largest first
+        for (int size = 2; size <= TOPK_THREADS; size <<= 1)
+            for (int stride = size >> 1; stride > 0; stride >>= 1) {
+                __syncthreads();
+                const int j = tid ^ stride;
+                if (j > tid) {
+                    const float va = cand_v[tid], vb = cand_v[j];
+                    if ((vb > va) == ((tid & size) == 0)) { cand_v[tid] = vb; cand_v[j] = va; }
+                }
+            }
+        __syncthreads();
+        least = cand_v[k - 1];
+        if (tid == 0) n_cand = 0;
+        __syncthreads();                                     // all have read it before the list is filled again
+    }
 
-    // ---- pass 2: the next 11 bits among the elements of that bin, and the sum of exp(l - max) ----
-    for (int i = tid; i < 2048; i += TOPK_THREADS) hist[i] = 0;
-    __syncthreads();
+    // ---- the sum of exp(l - max), and the candidates of the short way ----
     float sum = 0.f;
+    bool full = false;                                       // this thread met a full list: it stops offering
     for (int i = tid; i < vocab; i += TOPK_THREADS) {
         const float v = row[i];
         sum += expf(v - mx);
-        const uint32_t key = float_key(v);
-        if (k > 0 && (key >> 21) == prefix) atomicAdd(&hist[(key >> 10) & 0x7ffu], 1u);
+        if (!full && v >= least) {
+            const int at = atomicAdd(&n_cand, 1);
+            if (at < TOPK_MAX) { cand_v[at] = v; cand_i[at] = i; }
+            else full = true;
+        }
     }
     sum = block_sum(sum, red);
     if (stats && tid == 0) {
@@ -174,6 +225,28 @@ __global__ __launch_bounds__(TOPK_THREADS) void topk_kernel(const float* __restr
         stats[2 * blockIdx.x + 1] = logf(sum);
     }
     if (k == 0) return;
+    __syncthreads();
+    const int found = n_cand;
+    if (found >= k && found <= TOPK_MAX) {
+        topk_sort_and_store(cand_v, cand_i, found, k, ids, vals);
+        return;
+    }
+    __syncthreads();
+
+    // ---- the long way. Pass 1: top 11 bits ----
+    for (int i = tid; i < 2048; i += TOPK_THREADS) hist[i] = 0;
+    __syncthreads();
+    for (int i = tid; i < vocab; i += TOPK_THREADS) atomicAdd(&hist[float_key(row[i]) >> 21], 1u);
+    int rank = k;
+    uint32_t prefix = (uint32_t)topk_find_bin(hist, 2048, rank, pick);
+
+    // ---- pass 2: the next 11 bits among the elements of that bin ----
+    for (int i = tid; i < 2048; i += TOPK_THREADS) hist[i] = 0;
+    __syncthreads();
+    for (int i = tid; i < vocab; i += TOPK_THREADS) {
+        const uint32_t key = float_key(row[i]);
+        if ((key >> 21) == prefix) atomicAdd(&hist[(key >> 10) & 0x7ffu], 1u);
+    }
     prefix = (prefix << 11) | (uint32_t)topk_find_bin(hist, 2048, rank, pick);
 
     // ---- pass 3: the last 10 bits ----
@@ -228,33 +301,8 @@ __global__ __launch_bounds__(TOPK_THREADS) void topk_kernel(const float* __restr
         base_above += __popcll(ma);
         base_equal += __popcll(me);
     }
-    int n = 2;
-    while (n < k) n <<= 1;
-    for (int i = k + tid; i < n; i += TOPK_THREADS) {        // padding sorts to the end
-        cand_v[i] = -INFINITY;
-        cand_i[i] = 0x7fffffff;
-    }
-
-    // ---- sort: bitonic network over n <= 1024 entries, one thread per entry ----
-    for (int size = 2; size <= n; size <<= 1)
-        for (int stride = size >> 1; stride > 0; stride >>= 1) {
-            __syncthreads();
-            const int j = tid ^ stride;
-            if (tid < n && j > tid) {
-                const bool forward = (tid & size) == 0;      // this pair's better entry goes first
-                const float va = cand_v[tid], vb = cand_v[j];
-                const int ia = cand_i[tid], ib = cand_i[j];
-                if (better(vb, ib, va, ia) == forward) {
-                    cand_v[tid] = vb; cand_i[tid] = ib;
-                    cand_v[j] = va; cand_i[j] = ia;
-                }
-            }
-        }
     __syncthreads();
-    for (int c = tid; c < k; c += TOPK_THREADS) {
-        ids[(size_t)blockIdx.x * k + c] = cand_i[c] == 0x7fffffff ? -1 : cand_i[c];
-        vals[(size_t)blockIdx.x * k + c] = cand_v[c];
-    }
+    topk_sort_and_store(cand_v, cand_i, k, k, ids, vals);
 }
 
 extern "C" int hfa_topk(const float* logits, int ld, int* ids, float* vals, float* stats, int n_rows, int vocab,

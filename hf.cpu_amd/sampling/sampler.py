@@ -7,12 +7,12 @@ probabilities ``exp((l - max) / temp)`` normalised in fp32, cut by ``min_p`` (le
 with ``p >= min_p * p_max``), cut by ``top_p`` (shortest prefix whose sum reaches it), and
 one draw ``r = uniform * sum`` picks the first candidate whose running sum exceeds ``r``.
 
-The GPU does the part that touches the whole vocabulary (argmax; the ordered best-k and
-the row's log-sum-exp, kernels in csrc/sampling.hip); the few candidates left are finished
-on the host in fp32 in exactly the order above. With ``top_k`` off (0) or beyond the
-best-k kernel's 1024 the device orders the whole row and draws from it itself, by the same
-fp32 operations in the same order as ``pick_rows``, which stays the statement of the draw
-and what the tests compare the kernel with.
+The GPU does all of it (kernels in csrc/sampling.hip): argmax; the ordered best-k and the
+row's log-sum-exp, or, with ``top_k`` off (0) or beyond the best-k kernel's 1024, the whole
+row in order; and the draw from these candidates, by the same fp32 operations in the same
+order as ``pick_rows`` below, which stays the statement of the draw and what the tests
+compare the kernel with. The host gives each request's uniform number and reads one token
+a row.
 """
 from dataclasses import dataclass
 
@@ -105,6 +105,11 @@ class Sampler:
     def __init__(self, ops):
         self.ops = ops
 
+    def _draw(self, ids, vals, numbers, cuts):
+        device = vals.device
+        return self.ops.draw_rows(ids, vals, torch.from_numpy(numbers).to(device),
+                                  torch.from_numpy(cuts).to(device)).cpu().numpy()
+
     def sample(self, logits, wants):
         R = logits.shape[0]
         if R != len(wants):
@@ -115,26 +120,38 @@ class Sampler:
             if n_lp or (not params.greedy and 0 < params.top_k <= TOPK_KERNEL_MAX):
                 need_k = max(need_k, n_lp, 0 if params.greedy else min(params.top_k, TOPK_KERNEL_MAX))
         need_k = min(need_k, logits.shape[1])
+        V = logits.shape[1]
         greedy = [i for i, (p, _, _) in enumerate(wants) if p.greedy]
         arg = self.ops.argmax(logits).cpu().numpy() if greedy else None
-        ids = vals = stats = None
+        best = ids = vals = stats = None
         if need_k or any(n for _, _, n in wants):
-            ids, vals, stats = (t.cpu().numpy() for t in self.ops.topk(logits, need_k))
+            best = self.ops.topk(logits, need_k)
+            if any(n for _, _, n in wants):       # before the draw below turns the values into probabilities
+                ids, vals, stats = (t.cpu().numpy() for t in best)
         toks = [None] * R
-        groups = {}                               # rows drawn from the device's candidates, by parameters
-        whole = []                                # rows drawn from the whole vocabulary, in order, on the device
+        few = []                                  # rows drawn from the best-k kernel's candidates
+        whole = []                                # rows drawn from the whole vocabulary, in order
         for i, (params, rng, n_lp) in enumerate(wants):
             if params.greedy:
                 toks[i] = int(arg[i])
-            elif 0 < params.top_k <= TOPK_KERNEL_MAX and params.top_k < logits.shape[1]:
-                groups.setdefault(params, []).append(i)
+            elif 0 < params.top_k <= TOPK_KERNEL_MAX and params.top_k < V:
+                few.append(i)
             else:
                 whole.append(i)
+        # Either way the device draws (csrc/sampling.hip: the same fp32 operations in the same order
+        # as ``pick_rows``); the host gives each request's uniform number and reads back one token a row.
+        if few:
+            numbers = np.zeros((R, 4), dtype=f32)
+            numbers[:, :2] = 1                    # rows that are not drawn here: any harmless draw
+            cuts = np.ones(R, dtype=np.int32)
+            for i in few:
+                params, rng, _ = wants[i]
+                numbers[i] = (params.temp, params.top_p, params.min_p, rng.uniform())
+                cuts[i] = params.top_k
+            drawn = self._draw(best[0], best[1], numbers, cuts)
+            for i in few:
+                toks[i] = int(drawn[i])
         if whole:
-            # The device puts the whole vocabulary of these rows in order and draws from it
-            # (csrc/sampling.hip: the same fp32 operations in the same order as ``pick_rows``);
-            # the host gives each request's uniform number and reads back one token a row.
-            V = logits.shape[1]
             chosen = None if len(whole) == R else torch.tensor(whole, dtype=torch.int32, device=logits.device)
             all_ids, all_vals = self.ops.order_rows(logits, chosen)
             numbers = np.empty((len(whole), 4), dtype=f32)
@@ -143,14 +160,8 @@ class Sampler:
                 params, rng, _ = wants[i]
                 numbers[j] = (params.temp, params.top_p, params.min_p, rng.uniform())
                 cuts[j] = params.top_k if 0 < params.top_k < V else V
-            drawn = self.ops.draw_rows(all_ids, all_vals, torch.from_numpy(numbers).to(logits.device),
-                                       torch.from_numpy(cuts).to(logits.device)).cpu().numpy()
-            for i, t in zip(whole, drawn):
+            for i, t in zip(whole, self._draw(all_ids, all_vals, numbers, cuts)):
                 toks[i] = int(t)
-        for params, rows in groups.items():
-            drawn = pick_rows(ids[rows, :params.top_k], vals[rows, :params.top_k], params, [wants[i][1] for i in rows])
-            for i, t in zip(rows, drawn):
-                toks[i] = t
         for i, (params, rng, n_lp) in enumerate(wants):
             tok = toks[i]
             ch = Choice(tok)

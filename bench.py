@@ -69,10 +69,10 @@ def prefill_flops(c, T):
     return 2.0 * T * L * per_layer + L * 4.0 * D * H * T * (T + 1) / 2 + 2.0 * head
 
 
-def serve_workload(which, dtype):
+def serve_workload(which, dtype, temp=0.0):
     """``--workload 0.5b | 32b``: all requests are submitted at once and served by the scheduler
-    (prompt portions under the token budget beside decoded tokens, greedy); the second of two
-    runs is timed. One JSON line: prompt and generated tokens per second of wall time."""
+    (prompt portions under the token budget beside decoded tokens; greedy, or with ``--temp``
+    the reference's default sampling at that temperature); the second of two runs is timed. One JSON line: prompt and generated tokens per second of wall time."""
     import numpy as np
     import torch
     import hf_cpu_amd
@@ -91,7 +91,7 @@ def serve_workload(which, dtype):
         steps0 = s.engine.steps_run
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        gens = s.generate(prompts, temp=0.0, max_tokens=w["new_tokens"])
+        gens = s.generate(prompts, temp=temp, seed=1, max_tokens=w["new_tokens"])
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
         steps = s.engine.steps_run - steps0
@@ -108,7 +108,7 @@ def serve_workload(which, dtype):
                    "num_attention_heads": sh["num_attention_heads"], "num_key_value_heads": sh["num_key_value_heads"],
                    "head_dim": sh["head_dim"], "intermediate_size": sh["intermediate_size"], "vocab_size": sh["vocab_size"],
                    "requests": w["requests"], "prompt_tokens": n_prompt, "generated_tokens": n_gen,
-                   "token_budget": w["budget"], "ctx": w["ctx"], "page_size": PAGE, "parallelism": "none"},
+                   "token_budget": w["budget"], "ctx": w["ctx"], "page_size": PAGE, "temp": temp, "parallelism": "none"},
         "generated_tok_per_s": round(n_gen / dt, 1)}))
     return 0
 
@@ -127,12 +127,14 @@ def main():
                     help="run one phase only and print a short line (for profiling a phase by itself)")
     ap.add_argument("--workload", choices=["7b", "0.5b", "32b"], default="7b",
                     help="7b: the default measurement; 0.5b, 32b: the baseline's other workloads, served by the scheduler")
+    ap.add_argument("--temp", type=float, default=0.0,
+                    help="for --workload 0.5b | 32b: sample at this temperature (top-k 40, top-p 0.95, min-p 0.05) instead of greedy")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this engine runs on one GPU; --gpus must be 1")
         return 2
     if args.workload != "7b":
-        return serve_workload(args.workload, args.dtype)
+        return serve_workload(args.workload, args.dtype, args.temp)
     if args.steps + args.warmup > NEW:
         print(f"bench.py: --steps + --warmup must not exceed the {NEW} new tokens of the workload")
         return 2

@@ -186,7 +186,14 @@ __global__ __launch_bounds__(TOPK_THREADS) void topk_kernel(const float* __restr
     // ---- the row's maximum, and every thread's own ----
     __shared__ int n_cand;
     float mx = -INFINITY;
-    for (int i = tid; i < vocab; i += TOPK_THREADS) mx = fmaxf(mx, row[i]);
+    constexpr int AT_ONCE = 8;                               // loads of a thread on their way together
+    for (int i0 = tid; i0 < vocab; i0 += AT_ONCE * TOPK_THREADS) {
+        float v[AT_ONCE];
+#pragma unroll
+        for (int u = 0; u < AT_ONCE; u++) v[u] = i0 + u * TOPK_THREADS < vocab ? row[i0 + u * TOPK_THREADS] : -INFINITY;
+#pragma unroll
+        for (int u = 0; u < AT_ONCE; u++) mx = fmaxf(mx, v[u]);
+    }
     const float own = mx;
     mx = block_max(mx, red);
     float least = INFINITY;                                  // what a candidate of the short way has to reach
@@ -210,13 +217,20 @@ __global__ __launch_bounds__(TOPK_THREADS) void topk_kernel(const float* __restr
     // ---- the sum of exp(l - max), and the candidates of the short way ----
     float sum = 0.f;
     bool full = false;                                       // this thread met a full list: it stops offering
-    for (int i = tid; i < vocab; i += TOPK_THREADS) {
-        const float v = row[i];
-        sum += expf(v - mx);
-        if (!full && v >= least) {
-            const int at = atomicAdd(&n_cand, 1);
-            if (at < TOPK_MAX) { cand_v[at] = v; cand_i[at] = i; }
-            else full = true;
+    for (int i0 = tid; i0 < vocab; i0 += AT_ONCE * TOPK_THREADS) {
+        float v[AT_ONCE];
+#pragma unroll
+        for (int u = 0; u < AT_ONCE; u++) v[u] = i0 + u * TOPK_THREADS < vocab ? row[i0 + u * TOPK_THREADS] : -INFINITY;
+#pragma unroll
+        for (int u = 0; u < AT_ONCE; u++) {                  // in ascending order of the ids, as one by one
+            const int i = i0 + u * TOPK_THREADS;
+            if (i >= vocab) break;
+            sum += expf(v[u] - mx);
+            if (!full && v[u] >= least) {
+                const int at = atomicAdd(&n_cand, 1);
+                if (at < TOPK_MAX) { cand_v[at] = v[u]; cand_i[at] = i; }
+                else full = true;
+            }
         }
     }
     sum = block_sum(sum, red);

@@ -512,7 +512,7 @@ __global__ __launch_bounds__(DRAW_THREADS) void draw_rows_kernel(float* __restri
     float* p = vals + (size_t)row * vocab;
     const int* id = ids + (size_t)row * vocab;
     const float temp = params[4 * row], top_p = params[4 * row + 1], min_p = params[4 * row + 2], u = params[4 * row + 3];
-    const int m = cuts[row];                                  // candidates after the top-k cut
+    const int m = cuts[row] < 1 ? 1 : cuts[row] > vocab ? vocab : cuts[row];      // candidates after the top-k cut
     const float l0 = p[0];
     __syncthreads();                                          // p[0] is read by all before it is overwritten
     for (int i = tid; i < m; i += DRAW_THREADS) p[i] = ref_expf(__fdiv_rn(__fsub_rn(p[i], l0), temp));

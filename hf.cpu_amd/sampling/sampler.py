@@ -106,9 +106,13 @@ class Sampler:
         self.ops = ops
 
     def _draw(self, ids, vals, numbers, cuts):
-        device = vals.device
-        return self.ops.draw_rows(ids, vals, torch.from_numpy(numbers).to(device),
-                                  torch.from_numpy(cuts).to(device)).cpu().numpy()
+        """The device's draw for rows of candidates in order; the rows' numbers and cuts travel as one copy."""
+        n = len(cuts)
+        both = np.empty(5 * n, dtype=f32)
+        both[:4 * n] = numbers.reshape(-1)
+        both[4 * n:].view(np.int32)[:] = cuts
+        sent = torch.from_numpy(both).to(vals.device)
+        return self.ops.draw_rows(ids, vals, sent[:4 * n].view(n, 4), sent[4 * n:].view(torch.int32)).cpu().numpy()
 
     def sample(self, logits, wants):
         R = logits.shape[0]

@@ -31,7 +31,7 @@ WORKLOADS = {
                             vocab_size=151936, rope_theta=1000000.0, rms_norm_eps=1e-6, tie_word_embeddings=True,
                             use_sliding_window=False, max_position_embeddings=32768, hidden_act="silu"),
                  name="Qwen2.5-0.5B shape, random weights", requests=64, prompt_lo=16, prompt_hi=4096, new_tokens=128,
-                 ctx=32768, budget=2048),
+                 ctx=32768, budget=8192),
     "32b": dict(shape=dict(architectures=["Qwen2ForCausalLM"], model_type="qwen2", num_hidden_layers=64, hidden_size=5120,
                            num_attention_heads=40, num_key_value_heads=8, head_dim=128, intermediate_size=27648,
                            vocab_size=152064, rope_theta=1000000.0, rms_norm_eps=1e-5, tie_word_embeddings=False,
@@ -69,7 +69,7 @@ def prefill_flops(c, T):
     return 2.0 * T * L * per_layer + L * 4.0 * D * H * T * (T + 1) / 2 + 2.0 * head
 
 
-def serve_workload(which, dtype, temp=0.0):
+def serve_workload(which, dtype, temp=0.0, budget=0):
     """``--workload 0.5b | 32b``: all requests are submitted at once and served by the scheduler
     (prompt portions under the token budget beside decoded tokens; greedy, or with ``--temp``
     the reference's default sampling at that temperature); the second of two runs is timed. One JSON line: prompt and generated tokens per second of wall time."""
@@ -77,7 +77,9 @@ def serve_workload(which, dtype, temp=0.0):
     import torch
     import hf_cpu_amd
     import hf_cpu_amd.session as S
-    w = WORKLOADS[which]
+    w = dict(WORKLOADS[which])
+    if budget:
+        w["budget"] = budget
     cfg = hf_cpu_amd.config_from_dict(w["shape"])
     t0 = time.perf_counter()
     s = S.Session(cfg, dtype=dtype, ctx_max=w["ctx"], batch=w["budget"], page_size=PAGE, max_seqs=64,
@@ -129,12 +131,14 @@ def main():
                     help="7b: the default measurement; 0.5b, 32b: the baseline's other workloads, served by the scheduler")
     ap.add_argument("--temp", type=float, default=0.0,
                     help="for --workload 0.5b | 32b: sample at this temperature (top-k 40, top-p 0.95, min-p 0.05) instead of greedy")
+    ap.add_argument("--budget", type=int, default=0,
+                    help="for --workload 0.5b | 32b: the scheduler's token budget of a step (0 = the workload's own)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this engine runs on one GPU; --gpus must be 1")
         return 2
     if args.workload != "7b":
-        return serve_workload(args.workload, args.dtype, args.temp)
+        return serve_workload(args.workload, args.dtype, args.temp, args.budget)
     if args.steps + args.warmup > NEW:
         print(f"bench.py: --steps + --warmup must not exceed the {NEW} new tokens of the workload")
         return 2

@@ -702,10 +702,12 @@ int gemm_mfma_launch(const GemmArgs& g, void* workspace, size_t workspace_bytes,
         return gemm_finish_launch((const float*)workspace, parts, g.bias, g.out, mode, g.ldo, g.M, g.N, g.stream);
     } else if (dma_ok && 2 * tiles256 >= 128)
         rc = launch_dma<256, 128, 32, 4, 2, 6>(g, kmode, kout, 1, g.K);
-    else if (BM == 128)
-        rc = launch_mode<128, 128, 64, 2, 2>(g, kmode, kout, splits, k_per_split);
-    else if (BM == 64)
+    else if (BM == 128)                        // eight waves a block in both: about 2 % quicker than four with twice the accumulators
+        rc = launch_mode<128, 128, 64, 4, 2>(g, kmode, kout, splits, k_per_split);
+    else if (BM == 64 && kmode == OUT_SWIGLU)  // a wave needs 64 columns to pair gate and up
         rc = launch_mode<64, 128, 64, 2, 2>(g, kmode, kout, splits, k_per_split);
+    else if (BM == 64)
+        rc = launch_mode<64, 128, 64, 2, 4>(g, kmode, kout, splits, k_per_split);
     else if (kmode == OUT_SWIGLU)
         rc = launch_mode<32, 128, 64, 1, 2>(g, kmode, kout, splits, k_per_split);
     else

@@ -18,6 +18,7 @@ class Engine:
     GRAPH_MAX_TOKENS = 256        # decode-only steps up to this many requests replay a captured graph
     GRAPH_LEN_BUCKET = 256        # a graph serves request lengths up to a multiple of this
     BATCH_BUCKET = 8              # decode steps of more requests than this are filled up to a multiple of it
+    GRAPHS_KEPT = 96              # graphs held at a time; the one replayed longest ago goes first
 
     def __init__(self, model, ops, page_tokens=16, n_pages=None, max_tokens=None, max_seqs=8,
                  max_context=None, graphs=True):
@@ -238,6 +239,7 @@ class Engine:
         stamp = (self.ops.scratch_generation, self.staging.generation)
         hit = self._graphs.get(key)
         if hit is not None and hit[0] == stamp:
+            self._graphs[key] = self._graphs.pop(key)        # the dict's order is the order of last use
             hit[1].replay()
             self.graph_replays += 1
             return
@@ -249,7 +251,10 @@ class Engine:
             self.model.forward(self.ops, step, self.storage.views, logits)
         if (self.ops.scratch_generation, self.staging.generation) != stamp:
             fail(EINVAL, "a work buffer moved while a step was captured")
+        self._graphs.pop(key, None)
         self._graphs[key] = (stamp, graph)
+        while len(self._graphs) > self.GRAPHS_KEPT:
+            del self._graphs[next(iter(self._graphs))]
         graph.replay()
         self.graph_replays += 1
 

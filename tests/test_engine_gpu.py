@@ -219,7 +219,8 @@ def test_batches_of_every_size_share_a_few_graphs(gpu, tmp_path, dtype):
     from 19 down to 1 occurs: every row against the plain implementation, and sizes above 8 are
     filled up to a multiple of 8 with rows of no request (they live on a page and in a slot that
     the manager never hands out), so that 24 and 16 are the only shapes captured for them. A
-    second pass over the same sizes replays, and gives the bits of the first."""
+    second pass over the same sizes replays, and gives the bits of the first; the engine keeps
+    only its most recently used graphs."""
     import hf_cpu_amd
     cfg = helpers.CONFIG_B
     d = helpers.make_model_dir(str(tmp_path / "m"), cfg, seed=3)
@@ -228,6 +229,7 @@ def test_batches_of_every_size_share_a_few_graphs(gpu, tmp_path, dtype):
     reqs = helpers.random_requests(cfg, lengths, seed=31)
     want = helpers.plain_logits(d, reqs)
     engine = hf_cpu_amd.load_engine(d, dtype=dtype, page_tokens=8, max_tokens=64 * n_req, max_seqs=n_req)
+    engine.GRAPHS_KEPT = 4                      # fewer than the shapes that occur: graphs are dropped and captured again
     passes = []
     for again in range(2):
         got, sizes = {}, set()
@@ -248,7 +250,8 @@ def test_batches_of_every_size_share_a_few_graphs(gpu, tmp_path, dtype):
         helpers.compare(got, want, TOL[dtype], "batches of every size")
         passes.append(got)
     assert all(np.array_equal(passes[0][k], passes[1][k]) for k in passes[0])
-    assert {key[0] for key in engine._graphs if key[0] > 8} <= {16, 24}
+    assert {key[0] for key in engine._graph_seen if key[0] > 8} <= {16, 24}
+    assert 0 < len(engine._graphs) <= 4
     assert engine.graph_replays > 0
     assert not engine.manager.held and all(p.n_held == 0 for p in engine.manager.pools)
 

@@ -102,8 +102,8 @@ extern "C" int hfa_argmax(const float* logits, int ld, int* out, int n_rows, int
 #define TOPK_THREADS 1024
 #define TOPK_MAX 1024
 
-__device__ __forceinline__ uint32_t float_key(float v) {     // larger float <=> larger key
-    const uint32_t u = __float_as_uint(v);
+__device__ __forceinline__ uint32_t float_key(float v) {     // larger float <=> larger key; -0 and 0 are one value
+    const uint32_t u = __float_as_uint(v + 0.0f);
     return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
 

@@ -609,6 +609,14 @@ def test_argmax_and_topk(ops32):
             order = np.lexsort((np.arange(152064), -big_np[r]))[:k]
             assert np.array_equal(ids[r].cpu().numpy(), order), f"k={k} row {r}"
             assert np.array_equal(vals[r].cpu().numpy(), big_np[r, order])
+    zeros_np = np.round(rng.standard_normal((2, 5000)).astype(np.float32) * 0.3)     # 0.0, -0.0 and a few +-1: the cut
+    zeros_np[1] = np.minimum(zeros_np[1], 0.0)                                       # falls among zeros of either sign,
+    for k in (1, 40, 1024):                                                          # which are one value: ids decide
+        ids, vals, _ = ops32.topk(dev(zeros_np), k)
+        for r in range(2):
+            order = np.argsort(-zeros_np[r], kind="stable")[:k]
+            assert np.array_equal(ids[r].cpu().numpy(), order), f"signed zeros, k={k} row {r}"
+            assert np.array_equal(vals[r].cpu().numpy(), zeros_np[r, order])
     small = rng.standard_normal((2, 37)).astype(np.float32)     # fewer ids than threads; k = all of them
     ids, vals, stats = ops32.topk(dev(small), 37)
     assert ids.cpu().tolist() == [list(np.lexsort((np.arange(37), -r))) for r in small]

@@ -297,6 +297,24 @@ def test_generation_survives_a_cache_that_is_too_small(gpu, models):
     assert not tiny.engine.manager.held
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_twenty_requests_together_give_what_each_gives_alone(gpu, models, dtype):
+    """More requests at once than the engine decodes without filling a step up (above 8 rows a
+    decode step gets rows of no request, so that batch sizes share graphs), with prompts and
+    lengths that make them start and end at different steps: greedy and sampled, every request
+    ends with the tokens it gets alone."""
+    import hf_cpu_amd.session as S
+    cfg = helpers.CONFIG_B
+    rng = np.random.default_rng(3)
+    prompts = [[int(t) for t in rng.integers(0, cfg["vocab_size"], int(rng.integers(1, 60)))] for _ in range(20)]
+    s = S.Session(models["B"], dtype=dtype, ctx_max=128, batch=48, page_size=8, max_seqs=20)
+    for temp in (0.0, 0.8):
+        together = s.generate(prompts, temp=temp, seed=5, max_tokens=30)
+        for i, p in enumerate(prompts):
+            assert s.generate(p, temp=temp, seed=5, max_tokens=30)[0].tokens == together[i].tokens, f"temp {temp}, prompt {i}"
+    assert s.engine.graph_replays > 0 and any(key[0] > 8 for key in s.engine._graph_seen)
+
+
 @pytest.mark.parametrize("seed", range(6))
 def test_serving_at_random_with_forks_a_window_and_a_tight_cache(gpu, models, seed):
     """Configuration B (windowed layers, pages of 8) under a random load: prompts of 1 to 120

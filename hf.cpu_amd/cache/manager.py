@@ -23,6 +23,8 @@ src/model.c:217-230). Here pages come from shared pools:
 """
 from dataclasses import dataclass, field
 
+import numpy as np
+
 from ..parts.base import FixedState, PagedKV
 from ..status import EINVAL, ENOMEM, ENOTSUP, ERANGE, EngineError, fail
 from .pages import OutOfPages, PagePool
@@ -94,6 +96,9 @@ class CacheManager:
             fail(EINVAL, f"request {req_id!r} is released but not admitted")
         for g, table in enumerate(h.tables):
             self.pools[g].give_back([p for p in table if p >= 0])
+            # Entries not yet sent to the device name a slot that the next request may take before
+            # the next drain: two entries for one (slot, block) in one scatter have no order.
+            self.appended[g] = [a for a in self.appended[g] if a[0] != h.slot]
         self._free_slots.append(h.slot)
 
     def fork(self, src_id, new_id):
@@ -233,16 +238,18 @@ class CacheManager:
         """Cache row (page * page_tokens + offset) of positions start .. start + count - 1."""
         table = self.held[req_id].tables[group]
         P = self.page_tokens
-        rows = []
-        for pos in range(start, start + count):
-            page = table[pos // P]
-            assert page >= 0, "a position about to be written has no page"
-            rows.append(page * P + pos % P)
-        return rows
+        first, last = start // P, (start + count - 1) // P
+        pages = np.asarray(table[first:last + 1], dtype=np.int64)
+        assert count <= 0 or (len(pages) == last + 1 - first and pages.min() >= 0), \
+            "a position about to be written has no page"
+        pos = np.arange(start, start + count, dtype=np.int64)
+        return (pages[pos // P - first] * P + pos % P).astype(np.int32)
 
     def drain_appended(self, group):
         """(slot, block, page) entries added to block tables since the last call."""
         out, self.appended[group] = self.appended[group], []
+        if len({(a[0], a[1]) for a in out}) != len(out):       # the last entry of a (slot, block) is the one that holds
+            out = list({(a[0], a[1]): a for a in out}.values())
         return out
 
     # ---- accounting ----------------------------------------------------------

@@ -47,7 +47,7 @@ def test_reserve_commit_release_and_window():
     h = m.admit("a")
     m.reserve("a", 10)                       # blocks 0..2 in both groups
     assert [len(t) for t in h.tables] == [3, 3]
-    assert m.slot_rows("a", 0, 0, 10) == [h.tables[0][p // 4] * 4 + p % 4 for p in range(10)]
+    assert list(m.slot_rows("a", 0, 0, 10)) == [h.tables[0][p // 4] * 4 + p % 4 for p in range(10)]
     m.commit("a", 10)
     # next position 10, window 6: keys >= 5 stay visible, so block 0 (positions 0..3) goes
     assert h.tables[0] == [0, 1, 2] and h.tables[1][0] == -1 and h.tables[1][1:] == [1, 2]
@@ -63,6 +63,26 @@ def test_reserve_commit_release_and_window():
     assert m.pools[0].n_held == m.pools[1].n_held == 0
     with pytest.raises(EngineError):
         m.release("a")
+    m.check()
+
+
+def test_no_block_table_entry_is_sent_twice_after_a_released_slot_is_taken_again():
+    """A fork that ends before the next step leaves entries for its slot; the request that takes
+    the slot next must not find them beside its own in one drain (a scatter has no order)."""
+    m = manager(n_pages=8, page=4, slots=3)
+    m.admit("a")
+    m.reserve("a", 6)
+    m.commit("a", 6)
+    m.drain_appended(0), m.drain_appended(1)
+    m.fork("a", "c")
+    m.release("c")
+    m.admit("y")
+    m.reserve("y", 5)
+    for g in range(2):
+        sent = m.drain_appended(g)
+        keys = [(slot, block) for slot, block, _ in sent]
+        assert len(keys) == len(set(keys)), sent
+        assert {(s_, b): p for s_, b, p in sent} == {(m.held["y"].slot, b): p for b, p in enumerate(m.held["y"].tables[g])}
     m.check()
 
 

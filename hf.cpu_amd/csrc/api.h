@@ -83,6 +83,15 @@ int hfa_scatter_i32(int* dst, const int* idx, const int* val, int n, hipStream_t
 int hfa_argmax(const float* logits, int ld, int* out, int n_rows, int vocab, void* workspace,
                size_t workspace_bytes, hipStream_t stream);
 
+// hfa_argmax for callers that cannot allocate or bring a workspace: code under HIP graph capture,
+// tight serving loops, harnesses that forbid hipMalloc. It has no counterpart in the reference. The
+// candidates of the first stage lie in a device array that the library holds itself (128 KiB on every
+// GPU it runs on, until the process ends), so the call allocates nothing; the caller still passes
+// logits and out. At most HFA_ARGMAX_STATIC_ROWS rows; more are refused. Calls that overlap on one
+// GPU share that array and race; nothing needs clearing between calls that follow each other.
+#define HFA_ARGMAX_STATIC_ROWS 256
+int hfa_argmax_static(const float* logits, int ld, int* out, int n_rows, int vocab, hipStream_t stream);
+
 // All candidates of the chosen rows (rows[i], or row i if rows is null) in the order (logit
 // descending, id ascending), as the reference's sort leaves them when top-k is off
 // (src/sample.c:59-64, 93-98): ids and vals are [n_rows, vocab]. `scratch` needs

@@ -1,6 +1,8 @@
 // Kernels of the sampler: the greedy choice, and the ordered best-k of a row with the
 // row's log-sum-exp, from which the host finishes temperature / top-k / top-p / min-p
 // sampling exactly in the reference's order of operations.
+#include <mutex>
+
 #include "api.h"
 #include "common.h"
 
@@ -79,6 +81,60 @@ extern "C" int hfa_argmax(const float* logits, int ld, int* out, int n_rows, int
     argmax_part_kernel<<<dim3(n_rows, ARGMAX_PARTS), 256, 0, stream>>>(logits, ld, vocab, part_v, part_i);
     argmax_final_kernel<<<n_rows, WAVE, 0, stream>>>(part_v, part_i, out);
     HFA_LAUNCH_CHECK("argmax");
+    return 0;
+}
+
+// ---- the greedy choice for callers that cannot allocate ---------------------------------------
+// hfa_argmax_static is hfa_argmax with the first stage's candidates in a buffer that the library
+// itself holds: a file-scope device array, so nobody allocates, the caller brings no workspace, and
+// the call may sit in code that is captured into a graph or that forbids hipMalloc. Every GPU the
+// library runs on holds its own copy of the array (HFA_ARGMAX_STATIC_ROWS x 64 candidates of 8
+// bytes = 128 KiB) at its own address until the process ends. In host code the array's name is
+// only a stand-in: the address a kernel can use comes from hipGetSymbolAddress, asked once per
+// device with that device current, and host code uses nothing else.
+// The first stage writes every candidate that the second stage reads, so nothing has to be cleared
+// between calls; the array keeps the last call's candidates. Calls that overlap on one GPU (two
+// streams, two threads) share the array and race: callers keep them in order.
+static __device__ __align__(256) unsigned char scratch[(size_t)HFA_ARGMAX_STATIC_ROWS * ARGMAX_PARTS * 8];
+
+#define HFA_MAX_DEVICES 64
+static void* scratch_of_device[HFA_MAX_DEVICES];      // device address of `scratch` per GPU, null = not asked yet
+static std::mutex scratch_lock;
+
+static int scratch_address(void** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= HFA_MAX_DEVICES) {
+        hfa_set_error("argmax_static: no current device (%s, device %d)", hipGetErrorString(e), dev);
+        return 2;
+    }
+    std::lock_guard<std::mutex> hold(scratch_lock);
+    if (scratch_of_device[dev] == nullptr) {
+        void* ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));       // for the current device
+        if (e != hipSuccess || ptr == nullptr) {
+            hfa_set_error("argmax_static: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(e));
+            return 2;
+        }
+        scratch_of_device[dev] = ptr;
+    }
+    *out = scratch_of_device[dev];
+    return 0;
+}
+
+extern "C" int hfa_argmax_static(const float* logits, int ld, int* out, int n_rows, int vocab, hipStream_t stream) {
+    HFA_REQUIRE(n_rows > 0 && vocab > 0 && ld >= vocab, "argmax_static: bad sizes rows=%d vocab=%d ld=%d", n_rows, vocab, ld);
+    HFA_REQUIRE(n_rows <= HFA_ARGMAX_STATIC_ROWS,
+                "argmax_static: %d rows, the library's own buffer holds the candidates of %d (use hfa_argmax with a "
+                "workspace for more)", n_rows, HFA_ARGMAX_STATIC_ROWS);
+    HFA_REQUIRE(logits != nullptr && out != nullptr, "argmax_static: null logits or output");
+    void* ptr = nullptr;
+    if (int rc = scratch_address(&ptr)) return rc;
+    float* part_v = (float*)ptr;
+    int* part_i = (int*)(part_v + (size_t)n_rows * ARGMAX_PARTS);
+    argmax_part_kernel<<<dim3(n_rows, ARGMAX_PARTS), 256, 0, stream>>>(logits, ld, vocab, part_v, part_i);
+    argmax_final_kernel<<<n_rows, WAVE, 0, stream>>>(part_v, part_i, out);
+    HFA_LAUNCH_CHECK("argmax_static");
     return 0;
 }
 

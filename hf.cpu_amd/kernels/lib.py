@@ -23,6 +23,7 @@ _SIGNATURES = {
     "hfa_swiglu": [P, P, I, I, I, P],
     "hfa_scatter_i32": [P, P, P, I, P],
     "hfa_argmax": [P, I, P, I, I, P, c_size_t, P],
+    "hfa_argmax_static": [P, I, P, I, I, P],
     "hfa_topk": [P, I, P, P, P, I, I, I, P],
     "hfa_order_rows": [P, I, P, P, P, I, I, P, c_size_t, P],
     "hfa_draw_rows": [P, P, I, I, P, P, P, P],

@@ -10,7 +10,9 @@ between device synchronisations. One JSON line is printed: ``value`` is decoded 
 second; ``prefill`` is one 2,048-token prompt in one step; ``roofline`` prices the decode
 step against HBM bandwidth (every weight it uses once, plus the cache of the live
 requests); ``points`` holds decode at batch 1 and 64. Peaks: HBM 8 TB/s, dense bf16 MFMA
-2.5 PFLOP/s, fp32 157.3 TFLOP/s.
+2.5 PFLOP/s, fp32 157.3 TFLOP/s. ``measured_peaks`` is what this device's own probes reach (a
+streaming read, a copy, the matrix cores on random and on all-zero operands); ``kernels`` prices
+every dominant part of the decode step (bytes / time) and of the prefill (flops / time) against both.
 """
 import argparse
 import json
@@ -67,6 +69,52 @@ def prefill_flops(c, T):
     per_layer, head = matmul_params(c)
     L, H, D = c["num_hidden_layers"], c["num_attention_heads"], c["head_dim"]
     return 2.0 * T * L * per_layer + L * 4.0 * D * H * T * (T + 1) / 2 + 2.0 * head
+
+
+def part_work(c, elem, batch, mean_ctx, T):
+    """What each timed part of a step has to move or compute, all layers together:
+    ({part: bytes of a decode step}, {part: flops of a prefill of T tokens})."""
+    L, E, F, V = c["num_hidden_layers"], c["hidden_size"], c["intermediate_size"], c["vocab_size"]
+    H, D = c["num_attention_heads"], c["head_dim"]
+    QD, KD = H * D, c["num_key_value_heads"] * D
+    params = {"qkv": L * E * (QD + 2 * KD), "wo": L * QD * E, "gate_up": L * 2 * F * E, "down": L * F * E, "head": V * E}
+    dec = {k: v * elem for k, v in params.items()}
+    dec["attn"] = batch * mean_ctx * 2 * KD * L * elem
+    pre = {k: 2.0 * T * v for k, v in params.items() if k != "head"}
+    pre["attn"] = L * 4.0 * D * H * T * (T + 1) / 2
+    return dec, pre
+
+
+def kernel_fractions(eng, stage, step_fn, n, shape, elem, batch, mean_ctx, peaks, short):
+    """Times ``n`` steps of ``stage`` ("decode" or "prefill") by part (device events around each part's
+    kernels, steps run eagerly) and prices every dominant part: bytes / time for a decode step's parts
+    against HBM, flops / time for the prefill's against the matrix cores; against the published peak
+    ("frac") and, if measured, against what this device's own probes reach ("frac_measured")."""
+    eng.profile_start()
+    for _ in range(n):
+        step_fn()
+    book = eng.profile_stop()[stage]
+    dec_b, pre_f = part_work(shape, elem, batch, mean_ctx, PROMPT)
+    out = {}
+    if stage == "decode":
+        for part, nbytes in dec_b.items():
+            ms = book.get(part, 0.0) / n
+            if ms > 0:
+                e = {"us": round(ms * 1e3, 1), "GBps": round(nbytes / ms / 1e6, 1), "frac": round(nbytes / ms / 1e-3 / HBM_PEAK, 4)}
+                if peaks:
+                    e["frac_measured"] = round(nbytes / ms / 1e6 / peaks["hbm_read_GBps"], 4)
+                out["decode." + part] = e
+        out["decode.other"] = {"us": round(sum(v for k, v in book.items() if k not in dec_b) / n * 1e3, 1)}
+    else:
+        for part, flops in pre_f.items():
+            ms = book.get(part, 0.0) / n
+            if ms > 0:
+                e = {"us": round(ms * 1e3, 1), "TFLOPs": round(flops / ms / 1e9, 1), "frac": round(flops / ms / 1e-3 / FLOP_PEAK[short], 4)}
+                if peaks and short == "bf16":
+                    e["frac_measured"] = round(flops / ms / 1e9 / peaks["mfma_bf16_TFLOPs"], 4)
+                out["prefill." + part] = e
+        out["prefill.other"] = {"us": round(sum(v for k, v in book.items() if k not in pre_f) / n * 1e3, 1)}
+    return out
 
 
 def serve_workload(which, dtype, temp=0.0, budget=0):
@@ -127,6 +175,8 @@ def main():
     ap.add_argument("--prefill-reps", type=int, default=3)
     ap.add_argument("--only", choices=["prefill", "decode"], default=None,
                     help="run one phase only and print a short line (for profiling a phase by itself)")
+    ap.add_argument("--no-peaks", action="store_true", help="skip the probes of the device's own peaks")
+    ap.add_argument("--no-kernels", action="store_true", help="skip the timing by part")
     ap.add_argument("--workload", choices=["7b", "0.5b", "32b"], default="7b",
                     help="7b: the default measurement; 0.5b, 32b: the baseline's other workloads, served by the scheduler")
     ap.add_argument("--temp", type=float, default=0.0,
@@ -167,6 +217,14 @@ def main():
     def prompt():
         return [int(t) for t in rng.integers(0, cfg.vocab_size, PROMPT)]
 
+    peaks = None
+    if not args.no_peaks and args.only is None:
+        from hf_cpu_amd.probe import measure_peaks
+        peaks = measure_peaks(ops)
+        print(f"[bench] measured peaks: {peaks}", file=sys.stderr, flush=True)
+    kernels = {}
+    by_part = not args.no_kernels and args.only is None and args.steps + args.warmup + 4 <= NEW
+
     # ---- prefill: one prompt of 2,048 tokens in one step, logits for its last token ----
     times = []
     for rep in range(0 if args.only == "decode" else args.prefill_reps + 1):
@@ -183,11 +241,18 @@ def main():
     else:
         pre_s = sorted(times[1:])[len(times[1:]) // 2]        # the first run warms up
         print(f"[bench] prefill {PROMPT} tokens: {pre_s * 1e3:.1f} ms", file=sys.stderr, flush=True)
+    if by_part:
+
+        def one_prefill():
+            eng.step([("prefill", prompt(), [PROMPT - 1])])
+            eng.release("prefill")
+        kernels.update(kernel_fractions(eng, "prefill", one_prefill, 2, shape, elem, 1, PROMPT, peaks, short))
     if args.only == "prefill":
         print(json.dumps({"phase": "prefill", "tokens": PROMPT, "ms": round(pre_s * 1e3, 3)}))
         return 0
 
-    def decode(batch, steps, warmup):
+
+    def decode(batch, steps, warmup, by_part=False):
         ids = [("d", i) for i in range(batch)]
         last = []
         for r in ids:
@@ -205,11 +270,14 @@ def main():
             one()
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
+        if by_part:                           # after the timed steps, at the context they ended with
+            kernels.update(kernel_fractions(eng, "decode", one, 4, shape, elem, batch, PROMPT + warmup + steps + 2.5,
+                                            peaks, short))
         for r in ids:
             eng.release(r)
         return dt
 
-    dt = decode(args.batch, args.steps, args.warmup)
+    dt = decode(args.batch, args.steps, args.warmup, by_part=by_part)
     ms_step = dt / args.steps * 1e3
     value = args.batch * args.steps / dt
     print(f"[bench] decode batch {args.batch}: {ms_step:.3f} ms/step", file=sys.stderr, flush=True)
@@ -246,6 +314,14 @@ def main():
                      "frac": round(achieved * 1e9 / HBM_PEAK, 4)},
         "points": points,
     }
+    if peaks:                                  # against what this device's own probes reach
+        line["measured_peaks"] = peaks
+        line["roofline"]["measured_peak"] = peaks["hbm_read_GBps"]
+        line["roofline"]["frac_measured"] = round(achieved / peaks["hbm_read_GBps"], 4)
+        if short == "bf16":
+            line["prefill"]["frac_measured"] = round(flops / pre_s / 1e12 / peaks["mfma_bf16_TFLOPs"], 4)
+    if kernels:
+        line["kernels"] = kernels
     print(json.dumps(line))
     return 0
 

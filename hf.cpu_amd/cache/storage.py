@@ -3,6 +3,8 @@ from dataclasses import dataclass
 
 import torch
 
+from .. import memory
+
 
 @dataclass
 class PagedView:
@@ -40,13 +42,14 @@ class CacheStorage:
             rows = (pool.n_pages + 1) * manager.page_tokens
             for e in g.entries:
                 self.views[e] = PagedView(g.index,
-                                          torch.zeros((rows, g.k_width), dtype=dtype, device=device),
-                                          torch.zeros((rows, g.v_width), dtype=dtype, device=device),
+                                          memory.zeros((rows, g.k_width), dtype, device, f"keys of schedule entry {e}"),
+                                          memory.zeros((rows, g.v_width), dtype, device, f"values of schedule entry {e}"),
                                           manager.page_tokens, g.window)
         for e, n_floats in manager.state_entries.items():
-            self.views[e] = StateView(torch.zeros((manager.n_slots + 1, n_floats), dtype=torch.float32, device=device))
-        self.block_tables = [torch.zeros((manager.n_slots + 1, manager.max_blocks), dtype=torch.int32, device=device)
-                             for _ in manager.groups]
+            self.views[e] = StateView(memory.zeros((manager.n_slots + 1, n_floats), torch.float32, device,
+                                                    f"state of schedule entry {e}"))
+        self.block_tables = [memory.zeros((manager.n_slots + 1, manager.max_blocks), torch.int32, device, f"block table of group {g.index}")
+                             for g in manager.groups]
         self.pad_slot = manager.n_slots
         self.pad_pages = [pool.n_pages for pool in manager.pools]
         for table, page in zip(self.block_tables, self.pad_pages):

@@ -111,6 +111,17 @@ int hfa_draw_rows(float* vals, const int* ids, int n_rows, int vocab, const floa
 int hfa_topk(const float* logits, int ld, int* ids, float* vals, float* stats, int n_rows, int vocab, int k,
              hipStream_t stream);
 
+// The device's own peaks (the reference's read_sum and fma_burn, src/kern.h:17-23): a streaming read
+// of `bytes` (16-byte aligned; `sink` is 16 bytes that are almost never written) by `blocks_per_cu`
+// blocks of 256 threads a CU, a copy, and a burn of
+// the matrix cores on register operands (`zeros`: all-zero operands, else small pseudo-random ones):
+// `out` takes one float per thread of the launch, hfa_probe_mfma_threads() of them; *flops is what it
+// computed. The caller times them.
+int hfa_probe_read(const void* src, size_t bytes, void* sink, int blocks_per_cu, hipStream_t stream);
+int hfa_probe_copy(const void* src, void* dst, size_t bytes, hipStream_t stream);
+int hfa_probe_mfma_threads(void);
+int hfa_probe_mfma(float* out, int iters, int zeros, double* flops, hipStream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

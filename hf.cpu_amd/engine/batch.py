@@ -11,6 +11,8 @@ from dataclasses import dataclass
 import numpy as np
 import torch
 
+from .. import memory
+
 
 @dataclass
 class Entry:
@@ -70,11 +72,13 @@ class IntStaging:
 
     def _grow(self, capacity):
         torch.cuda.synchronize(self.device)
+        # all three first, then the switch: a failed allocation leaves the old buffers in use
+        host = [memory.empty(capacity, torch.int32, None, "pinned staging buffer", pin=True) for _ in range(2)]
+        dev = memory.empty(capacity, torch.int32, self.device, "device staging buffer")
         self.generation += 1                      # captured graphs hold the old address
         self.capacity = capacity
-        self.host = [torch.empty(capacity, dtype=torch.int32, pin_memory=True) for _ in range(2)]
+        self.host, self.dev = host, dev
         self.events = [None, None]
-        self.dev = torch.empty(capacity, dtype=torch.int32, device=self.device)
 
     def upload(self, arrays):
         """Copies the int32 numpy arrays one after the other; returns device views of them.

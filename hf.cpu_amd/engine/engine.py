@@ -9,6 +9,7 @@ Reference: ``forward_impl`` (src/model.c:545-640) with its two batch shapes
 import numpy as np
 import torch
 
+from .. import memory
 from ..cache import CacheManager, CacheStorage
 from ..status import EINVAL, fail
 from .batch import Entry, GroupInputs, IntStaging, StepInputs, as_i32
@@ -137,6 +138,7 @@ class Engine:
             if self.profile is not None:
                 self._book_times("prefill" if step.max_q_len > 1 else "decode")
         except BaseException:
+            self.ops.abandon()
             for r in reserved:
                 mgr.rollback(r)
             for r in admitted:
@@ -216,6 +218,7 @@ class Engine:
             if self.profile is not None:
                 self._book_times("decode")
         except BaseException:
+            self.ops.abandon()
             for r in reserved:
                 mgr.rollback(r)
             raise
@@ -246,6 +249,7 @@ class Engine:
         if key not in self._graph_seen:          # first sight: run eagerly, which also sizes the work buffers
             self._graph_seen.add(key)
             return self.model.forward(self.ops, step, self.storage.views, logits)
+        memory.note("a captured step")
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             self.model.forward(self.ops, step, self.storage.views, logits)

@@ -27,6 +27,9 @@ _SIGNATURES = {
     "hfa_topk": [P, I, P, P, P, I, I, I, P],
     "hfa_order_rows": [P, I, P, P, P, I, I, P, c_size_t, P],
     "hfa_draw_rows": [P, P, I, I, P, P, P, P],
+    "hfa_probe_read": [P, c_size_t, P, I, P],
+    "hfa_probe_copy": [P, P, c_size_t, P],
+    "hfa_probe_mfma": [P, I, I, P, P],
 }
 
 
@@ -44,6 +47,8 @@ def library():
             lib.hfa_version.restype = c_int
             lib.hfa_order_rows_scratch.restype = c_size_t
             lib.hfa_order_rows_scratch.argtypes = [c_int, c_int]
+            lib.hfa_probe_mfma_threads.restype = c_int
+            lib.hfa_probe_mfma_threads.argtypes = []
             lib.hfa_attention_prompt_rows.restype = c_int
             lib.hfa_attention_prompt_rows.argtypes = []
             for name, args in _SIGNATURES.items():

@@ -19,6 +19,7 @@ from dataclasses import dataclass
 
 import torch
 
+from .. import memory
 from ..status import EINVAL, ENOTSUP, EngineError, fail
 from .lib import last_error, library
 
@@ -100,8 +101,8 @@ class Ops:
         self._scratch_views = {}             # (name, shape, dtype) -> the view handed out last time
         self._stream_handle = None
         self.scratch_generation = 0
-        self.workspace = torch.empty(WORKSPACE_BYTES, dtype=torch.uint8, device=self.device)
-        self.attn_workspace = torch.empty(WORKSPACE_BYTES, dtype=torch.uint8, device=self.device)
+        self.workspace = memory.empty(WORKSPACE_BYTES, torch.uint8, self.device, "workspace of the matrix products")
+        self.attn_workspace = memory.empty(WORKSPACE_BYTES, torch.uint8, self.device, "workspace of attention")
         self._pending = None
         self._splits_out = ctypes.c_int(0)
         self._sections = None                # while timing: (name, start event, end event) of every section left
@@ -162,7 +163,7 @@ class Ops:
         if buf is None or buf.numel() < nbytes:
             if torch.cuda.is_current_stream_capturing():
                 fail(EINVAL, f"work buffer '{name}' would have to grow while a graph is being captured")
-            buf = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=self.device)
+            buf = memory.empty(max(nbytes, 256), torch.uint8, self.device, f"work buffer '{name}'")
             self._scratch[name] = buf
             self.scratch_generation += 1          # captured graphs hold the old address
             self._scratch_views = {k: v for k, v in self._scratch_views.items() if k[0] != name}
@@ -207,6 +208,10 @@ class Ops:
             self._pending = None
             return p
         return None
+
+    def abandon(self):
+        """Forgets a deferred product (after a step that failed: its partial sums are of no use)."""
+        self._pending = None
 
     def settle(self, tensor=None):
         """Adds up a deferred product now (all of them if ``tensor`` is None, else only one that
@@ -351,7 +356,7 @@ class Ops:
         if logits.dtype != torch.float32:
             fail(EINVAL, "argmax: logits must be fp32")
         if out is None:
-            out = torch.empty(R, dtype=torch.int32, device=logits.device)
+            out = memory.empty(R, torch.int32, logits.device, "argmax output")
         self._check(self.lib.hfa_argmax(logits.data_ptr(), _rows(logits, "argmax logits"), _ints(out, "argmax out", R),
                                         R, V, self.workspace.data_ptr(), self.workspace.numel(), self._stream()))
         return out
@@ -364,8 +369,8 @@ class Ops:
         if logits.dtype != torch.float32:
             fail(EINVAL, "order_rows: logits must be fp32")
         n = R if rows is None else int(rows.numel())
-        ids = torch.empty((n, V), dtype=torch.int32, device=logits.device)
-        vals = torch.empty((n, V), dtype=torch.float32, device=logits.device)
+        ids = memory.empty((n, V), torch.int32, logits.device, "ordered ids")
+        vals = memory.empty((n, V), torch.float32, logits.device, "ordered values")
         need = int(self.lib.hfa_order_rows_scratch(n, V))
         scratch = self.scratch("order_rows", (need,), torch.uint8)
         self._check(self.lib.hfa_order_rows(logits.data_ptr(), _rows(logits, "order_rows logits"),
@@ -382,7 +387,7 @@ class Ops:
             fail(EINVAL, "draw_rows: expected contiguous fp32 values and ids of one shape")
         if params.dtype != torch.float32 or not params.is_contiguous() or tuple(params.shape) != (n, 4):
             fail(EINVAL, f"draw_rows: expected [{n}, 4] fp32 parameters")
-        tokens = torch.empty((n,), dtype=torch.int32, device=vals.device)
+        tokens = memory.empty((n,), torch.int32, vals.device, "drawn tokens")
         self._check(self.lib.hfa_draw_rows(vals.data_ptr(), _ints(ids, "draw_rows ids", n * V), n, V, params.data_ptr(),
                                            _ints(cuts, "draw_rows cuts", n), tokens.data_ptr(), self._stream()))
         return tokens
@@ -394,9 +399,9 @@ class Ops:
         R, V = logits.shape
         if logits.dtype != torch.float32:
             fail(EINVAL, "topk: logits must be fp32")
-        ids = torch.empty((R, max(k, 1)), dtype=torch.int32, device=logits.device)
-        vals = torch.empty((R, max(k, 1)), dtype=torch.float32, device=logits.device)
-        stats = torch.empty((R, 2), dtype=torch.float32, device=logits.device) if want_stats else None
+        ids = memory.empty((R, max(k, 1)), torch.int32, logits.device, "top-k ids")
+        vals = memory.empty((R, max(k, 1)), torch.float32, logits.device, "top-k values")
+        stats = memory.empty((R, 2), torch.float32, logits.device, "row statistics") if want_stats else None
         self._check(self.lib.hfa_topk(logits.data_ptr(), _rows(logits, "topk logits"), ids.data_ptr(), vals.data_ptr(),
                                       None if stats is None else stats.data_ptr(), R, V, k, self._stream()))
         return ids[:, :k], vals[:, :k], stats

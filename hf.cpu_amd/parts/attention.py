@@ -4,6 +4,8 @@ import math
 
 import torch
 
+from .. import memory
+
 from ..registry import make_part, register_part
 from ..status import EINVAL, fail
 from .base import PagedKV, ParamSpec, Part
@@ -61,9 +63,9 @@ class Attention(Part):
         # One matrix for the three projections that share an input: rows of q, then k, then v.
         mats = [params[p + n + "_proj.weight"] for n in "qkv"]
         dt = torch.float32 if any(m.dtype == torch.float32 for m in mats) else mats[0].dtype
-        self.w_qkv = torch.cat([m.to(dt) for m in mats], dim=0).contiguous()
+        self.w_qkv = memory.cat([m.to(dt) for m in mats], 0, f"{p}q, k and v in one matrix")
         if self.qkv_bias:
-            self.b_qkv = torch.cat([params[p + n + "_proj.bias"] for n in "qkv"]).contiguous()
+            self.b_qkv = memory.cat([params[p + n + "_proj.bias"] for n in "qkv"], 0, f"{p}q, k and v biases in one vector")
         self.w_o = params[p + "o_proj.weight"]
         if self.out_bias:
             self.b_o = params[p + "o_proj.bias"]

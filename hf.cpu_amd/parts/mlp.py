@@ -1,6 +1,8 @@
 """Dense feed-forward parts."""
 import torch
 
+from .. import memory
+
 from ..registry import register_part
 from ..status import ENOTSUP, fail
 from .base import ParamSpec, Part
@@ -36,9 +38,10 @@ class GatedMLP(Part):
         # last step can form silu(gate) * up without storing gate and up.
         self.fused = ops.can_fuse_swiglu(g, u)
         if self.fused:
+            memory.note(f"{p}gate and up, interleaved")
             self.w_gate_up = ops.interleave_gate_up(g, u)
         else:
-            self.w_gate_up = torch.cat([g.to(dt), u.to(dt)], dim=0).contiguous()
+            self.w_gate_up = memory.cat([g.to(dt), u.to(dt)], 0, f"{p}gate and up in one matrix")
         self.w_down = params[p + "down_proj.weight"]
 
     def forward(self, ops, step, h, x):

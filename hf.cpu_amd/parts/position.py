@@ -2,6 +2,8 @@
 hand keys and values to the cache in the same pass."""
 import torch
 
+from .. import memory
+
 from ..registry import register_part
 from ..status import EINVAL, fail
 from .base import Part
@@ -32,7 +34,7 @@ class Rotary(Part):
     def bind(self, params, ops):
         i = torch.arange(self.rot_dim // 2, dtype=torch.float64)
         inv = torch.pow(torch.tensor(self.theta, dtype=torch.float64), -2.0 * i / self.rot_dim)
-        self.inv_freq = inv.to(torch.float32).to(ops.device)
+        self.inv_freq = memory.to_device(inv.to(torch.float32), ops.device, "rotary frequencies")
 
     def store(self, ops, step, qkv, n_heads, n_kv_heads, cache, write):
         """Rotates the queries (and keys) inside ``qkv`` at each token's position;

@@ -19,6 +19,8 @@ from dataclasses import dataclass
 import numpy as np
 import torch
 
+from .. import memory
+
 from ..status import EINVAL, fail
 from .mathx import hfc_expf
 
@@ -111,7 +113,7 @@ class Sampler:
         both = np.empty(5 * n, dtype=f32)
         both[:4 * n] = numbers.reshape(-1)
         both[4 * n:].view(np.int32)[:] = cuts
-        sent = torch.from_numpy(both).to(vals.device)
+        sent = memory.to_device(torch.from_numpy(both), vals.device, "the draws' numbers")
         return self.ops.draw_rows(ids, vals, sent[:4 * n].view(n, 4), sent[4 * n:].view(torch.int32)).cpu().numpy()
 
     def sample(self, logits, wants):
@@ -156,7 +158,7 @@ class Sampler:
             for i in few:
                 toks[i] = int(drawn[i])
         if whole:
-            chosen = None if len(whole) == R else torch.tensor(whole, dtype=torch.int32, device=logits.device)
+            chosen = None if len(whole) == R else memory.to_device(torch.tensor(whole, dtype=torch.int32), logits.device, "rows to order")
             all_ids, all_vals = self.ops.order_rows(logits, chosen)
             numbers = np.empty((len(whole), 4), dtype=f32)
             cuts = np.empty(len(whole), dtype=np.int32)

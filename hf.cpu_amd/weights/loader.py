@@ -7,6 +7,8 @@ wrong shape.
 """
 import torch
 
+from .. import memory
+
 from ..status import EFORMAT, fail
 from .safetensors_io import open_model_tensors
 
@@ -71,5 +73,5 @@ def load_tensors(model_dir, specs, compute_dtype, device):
         if e is None:
             continue
         t = e.file.read(s.name)
-        out[s.name] = t.to(held_dtype(s.kind, e.dtype, compute_dtype)).to(device).contiguous()
+        out[s.name] = memory.to_device(t, device, f"tensor '{s.name}'", held_dtype(s.kind, e.dtype, compute_dtype))
     return out

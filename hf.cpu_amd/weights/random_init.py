@@ -13,6 +13,8 @@ import os
 import numpy as np
 import torch
 
+from .. import memory
+
 from .safetensors_io import write_safetensors
 
 STORED = {"float32": torch.float32, "bfloat16": torch.bfloat16, "float16": torch.float16}
@@ -67,7 +69,7 @@ def random_device_tensors(specs, seed, compute_dtype, device):
         if s.kind == "table":
             out[s.name] = torch.randint(0, int(s.init[1]), s.shape, generator=gen, device=device, dtype=torch.int32)
             continue
-        t = torch.empty(s.shape, dtype=held, device=device)
+        t = memory.empty(s.shape, held, device, f"tensor '{s.name}'")
         t.normal_(0.0, float(s.init[1]), generator=gen)
         if s.init[0] == "one_plus_normal":
             t += 1.0

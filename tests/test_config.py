@@ -106,3 +106,22 @@ def test_plan_is_data_and_registry_is_open():
     with pytest.raises(EngineError) as e:
         hf_cpu_amd.registry.make_part("mixer", hf_cpu_amd.PartSpec("no_such_mixer", {}))
     assert "no_such_mixer" in str(e.value) and "attention" in str(e.value)
+
+
+def test_allocation_counter_fails_the_nth_once():
+    """The allocation choke point's injection (src/mem.c:12-30): the n-th allocation after
+    ``fail_after(n)`` fails with ENOMEM, once; the count goes on."""
+    from hf_cpu_amd import memory
+    from hf_cpu_amd.status import EngineError
+    memory.fail_after(3)
+    base = memory.allocations()
+    memory.note("a")
+    memory.note("b")
+    with pytest.raises(EngineError) as e:
+        memory.note("the third")
+    assert e.value.code == "ENOMEM" and "the third" in e.value.msg and "injected" in e.value.msg
+    for _ in range(5):
+        memory.note("later")
+    assert memory.allocations() == base + 8
+    memory.fail_after(0)
+    memory.note("none fails")

@@ -230,7 +230,32 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
             pf[kk].u = make_uint4(w[0], w[1], w[2], w[3]);
         }
     };
-    auto values = [&](const Frag (&vf)[NDB][2]) {
+    // Keys of a block that lie outside [k_begin, k_end] (before the first key any column sees, past the
+    // last one) have probability zero in every column, but what the cache holds there is not this
+    // request's: rows of a page it has not written yet, or of a page the window gave back, with
+    // whatever their last owner left, Inf and NaN included, and 0 x Inf is NaN. Their values are
+    // replaced by zeros; only the first and the last block of a walk have such keys.
+    auto values = [&](int key0, Frag (&vf)[NDB][2]) {
+        if (key0 < k_begin || key0 + KB - 1 > k_end) {         // uniform over the wave
+#pragma unroll
+            for (int kk = 0; kk < 2; kk++)
+#pragma unroll
+                for (int run = 0; run < 2; run++) {
+                    const int kb = key0 + 16 * kk + 8 * run + 4 * half;
+                    uint32_t mk[2];
+#pragma unroll
+                    for (int e = 0; e < 2; e++) {
+                        const bool lo_ok = kb + 2 * e >= k_begin && kb + 2 * e <= k_end;
+                        const bool hi_ok = kb + 2 * e + 1 >= k_begin && kb + 2 * e + 1 <= k_end;
+                        mk[e] = (lo_ok ? 0x0000ffffu : 0u) | (hi_ok ? 0xffff0000u : 0u);
+                    }
+#pragma unroll
+                    for (int db = 0; db < NDB; db++) {
+                        vf[db][kk].h[run].x &= mk[0];
+                        vf[db][kk].h[run].y &= mk[1];
+                    }
+                }
+        }
 #pragma unroll
         for (int kk = 0; kk < 2; kk++)
 #pragma unroll
@@ -247,7 +272,9 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
     const int first = (k_begin / KB) * KB;
     const int nb = first <= k_end ? (k_end - first) / KB + 1 : 0;
     const int k_top = first + nb * KB - 1 < hi ? first + nb * KB - 1 : hi;       // last key any load touches
-    const int win_blocks = (PG_MAX << psh) / KB;                                  // key blocks a window of pages covers
+    // key blocks a window of pages covers; a walk starts at a multiple of 32 keys, which with pages of more
+    // than 32 tokens may lie inside a page: the window's keys then touch one page more than they fill
+    const int win_blocks = ((P > KB ? PG_MAX - 1 : PG_MAX) << psh) / KB;
     for (int wb = 0; wb < nb; wb += win_blocks) {
         const int we = wb + win_blocks < nb ? wb + win_blocks : nb;               // blocks [wb, we)
         __syncthreads();                                                          // the old window is no longer read
@@ -268,12 +295,12 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
         for (int b = wb; b < we; b += 2) {
             scores(first + b * KB, k0f);
             load_k(at(b + 2), k0f);
-            values(v0f);
+            values(first + b * KB, v0f);
             load_v(at(b + 2), v0f);
             if (b + 1 >= we) break;
             scores(first + (b + 1) * KB, k1f);
             load_k(at(b + 3), k1f);
-            values(v1f);
+            values(first + (b + 1) * KB, v1f);
             load_v(at(b + 3), v1f);
         }
     }
@@ -317,7 +344,6 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
 // waves, so L2-to-CU traffic drops fourfold against the kernel above and several waves per SIMD
 // overlap their matrix products and softmax. Two LDS stages, one barrier per key block. Tiles
 // are numbered from the end of each request backwards, so the longest ones start first.
-#define PKS 136      // LDS row of a key: 128 dims + 8 pad (elements)
 #define PVS 36       // LDS row of a value dimension: 32 keys + 4 pad (elements)
 
 template <int NDB, bool SMALL_PAGES>
@@ -469,21 +495,33 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
             }
         }
     };
-    auto sstore = [&](int stage, const u32x4 (&rk)[NCH], const uint2 (&rv)[NCH][2]) {
+    // Values of keys outside [k_begin, hi] are stored as zeros (see the kernel above: their probabilities
+    // are zero, what the cache holds there may be anything); only a walk's first and last block have such.
+    auto sstore = [&](int stage, int key0, const u32x4 (&rk)[NCH], const uint2 (&rv)[NCH][2]) {
+        const bool edge = key0 < k_begin || key0 + KB - 1 > hi;           // uniform over the block
 #pragma unroll
         for (int i = 0; i < NCH; i++) {
             const int c = tid + i * 256;
             if (!EVEN && c >= TOT) break;
             *reinterpret_cast<u32x4*>(&k_s[stage][(c / (D / 8)) * KROW + (c % (D / 8)) * 8]) = rk[i];
             uint2* dst = reinterpret_cast<uint2*>(&v_s[stage][(c / 4) * PVS + 8 * (c % 4)]);
-            dst[0] = rv[i][0];
-            dst[1] = rv[i][1];
+            uint2 v0 = rv[i][0], v1 = rv[i][1];
+            if (edge) {
+                const int kb = key0 + 8 * (c % 4);
+                auto keep = [&](int k) { return k >= k_begin && k <= hi; };
+                v0.x &= (keep(kb) ? 0x0000ffffu : 0u) | (keep(kb + 1) ? 0xffff0000u : 0u);
+                v0.y &= (keep(kb + 2) ? 0x0000ffffu : 0u) | (keep(kb + 3) ? 0xffff0000u : 0u);
+                v1.x &= (keep(kb + 4) ? 0x0000ffffu : 0u) | (keep(kb + 5) ? 0xffff0000u : 0u);
+                v1.y &= (keep(kb + 6) ? 0x0000ffffu : 0u) | (keep(kb + 7) ? 0xffff0000u : 0u);
+            }
+            dst[0] = v0;
+            dst[1] = v1;
         }
     };
 
     const int first = (k_begin / KB) * KB;
     const int nb = hi >= k_begin ? (hi - first) / KB + 1 : 0;
-    const int win_blocks = (PG_MAX << psh) / KB;
+    const int win_blocks = ((P > KB ? PG_MAX - 1 : PG_MAX) << psh) / KB;     // see the kernel above
     for (int wb = 0; wb < nb; wb += win_blocks) {
         const int we = wb + win_blocks < nb ? wb + win_blocks : nb;               // blocks [wb, we)
         __syncthreads();                                                          // old window and stages are no longer read
@@ -499,7 +537,7 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
         const int last = first + (we - 1) * KB;
         auto at = [&](int b) { const int k = first + b * KB; return k < last ? k : last; };
         gload(at(wb), rk0, rv0);
-        sstore(wb & 1, rk0, rv0);
+        sstore(wb & 1, at(wb), rk0, rv0);
         gload(at(wb + 1), rk0, rv0);                          // unconditional: past the end the last block is fetched again
         gload(at(wb + 2), rk1, rv1);
         __syncthreads();
@@ -597,12 +635,12 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
         };
         for (int b = wb; b < we; b += 2) {
             one_block(b);
-            sstore((b & 1) ^ 1, rk0, rv0);                    // block b + 1
+            sstore((b & 1) ^ 1, at(b + 1), rk0, rv0);         // block b + 1
             gload(at(b + 3), rk0, rv0);
             __syncthreads();
             if (b + 1 >= we) break;
             one_block(b + 1);
-            sstore(b & 1, rk1, rv1);                          // block b + 2
+            sstore(b & 1, at(b + 2), rk1, rv1);               // block b + 2
             gload(at(b + 4), rk1, rv1);
             __syncthreads();
         }

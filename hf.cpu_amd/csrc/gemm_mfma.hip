@@ -684,7 +684,12 @@ int gemm_mfma_launch(const GemmArgs& g, void* workspace, size_t workspace_bytes,
     const bool halves = parts >= 2;
     // Tiles of 192 columns do three quarters of the work of 256 (a little less efficiently): they are
     // taken when they need fewer rounds over the CUs by more than that.
-    const int cus = 256;
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+            cus = 256;
+    }
     const int tiles192 = (rows256 / 256) * ((g.N + 191) / 192);
     const bool narrow = dma_ok && tiles256 >= 128 && mode != OUT_SWIGLU &&
                         ((tiles192 + cus - 1) / cus) * 80 < ((tiles256 + cus - 1) / cus) * 100;

@@ -11,7 +11,7 @@ import torch
 
 from .. import memory
 from ..cache import CacheManager, CacheStorage
-from ..status import EINVAL, fail
+from ..status import EINVAL, ENOTSUP, fail
 from .batch import Entry, GroupInputs, IntStaging, StepInputs, as_i32
 
 
@@ -57,6 +57,18 @@ class Engine:
     def release(self, req_id):
         """The request is finished: its pages and its slot are given back."""
         self.manager.release(req_id)
+
+    def truncate(self, req_id, length):
+        """Cuts the request back to its first ``length`` tokens (src/model.c:305): the next step's tokens
+        follow position ``length - 1``. Pages wholly beyond go back to the pool; rows beyond ``length`` on
+        the last page stay and are overwritten. Refused (ENOTSUP), with nothing changed, if the model
+        keeps per-request state of fixed size (it cannot be wound back), if a window has already given
+        back pages that the shorter sequence would see, or if the cut falls on a page shared with a fork."""
+        if req_id not in self.manager.held:
+            fail(EINVAL, f"request {req_id!r} is truncated but not admitted")
+        if self.manager.state_entries and length < self.manager.held[req_id].length:
+            fail(ENOTSUP, f"request {req_id!r}: a model with per-request state of fixed size cannot be cut back")
+        self.manager.truncate(req_id, int(length))
 
     def fork(self, src_id, new_id):
         """Admits ``new_id`` holding what ``src_id`` holds (src/model.c:271-301): whole pages are

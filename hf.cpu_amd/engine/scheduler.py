@@ -10,7 +10,8 @@ is reported but not fed (src/ops.c:881); the cap on new tokens is
 ``min(max_tokens, ctx_max - prompt)`` with stop reason ``length`` or ``ctx`` (src/ops.c:757-758).
 
 Each step:
- 1. every running request whose next token is a single decoded token brings it;
+ 1. every running request whose next token is a single decoded token brings it (if there are more
+    of them than the token budget, those that waited longest);
  2. what is left of the token budget goes to prompt portions, oldest request first:
     first those already running, then waiting ones, admitted while a state slot is free
     and fewer than ``max_seqs`` are live;
@@ -67,6 +68,7 @@ class Request:
     t_done: float = None
     admitted_at: int = -1                    # admission order, for the preemption choice
     forks: list = field(default_factory=list)     # continuations of the same prompt, forked when it is done
+    last_ran: int = -1                       # the step that last held tokens of this request
 
     @property
     def unfed(self):
@@ -165,10 +167,14 @@ class Scheduler:
         the decoded tokens fit."""
         mgr = self.manager
         decode = [r for r in self.running if r.unfed == 1 and r.n_fed > 0]
-        if not mgr.can_reserve([(r.req_id, 1) for r in decode]):
-            return None
         budget = self.token_budget
-        entries = [(r, 1, True) for r in decode[:budget]]
+        if len(decode) > budget:
+            # More requests decode than a step may hold tokens (the reference refuses --n above --batch,
+            # src/ops.c:810): they take turns, those that waited longest first, so every one advances.
+            decode = sorted(decode, key=lambda r: r.last_ran)[:budget]
+        if not mgr.can_reserve([(r.req_id, 1) for r in decode]):      # only for those that run
+            return None
+        entries = [(r, 1, True) for r in decode]
         budget -= len(entries)
         wanted = [(r.req_id, 1) for r, _, _ in entries]
         prefilling = [r for r in self.running if not (r.unfed == 1 and r.n_fed > 0)]
@@ -264,6 +270,7 @@ class Scheduler:
         sampled = [r for r, n, want in plan.entries if want]
         for r, n, _ in plan.entries:
             r.n_fed += n
+            r.last_ran = self.steps
         if sampled:
             t0 = time.perf_counter()
             choices = self.sampler.sample(logits, [(r.params, r.rng, r.logprobs) for r in sampled])

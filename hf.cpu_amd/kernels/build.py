@@ -72,6 +72,24 @@ def find_library():
     return found, False
 
 
+def build_extension(srcs, lib_path, verbose=True):
+    """Compiles HIP sources of a part that lives outside the package (its own kernels) into a shared
+    library of its own, with the flags the package's kernels are built with. Returns ``lib_path``."""
+    hipcc = hipcc_path()
+    env = dict(os.environ)
+    env.setdefault("HOME", tempfile.gettempdir())
+    os.makedirs(os.path.dirname(os.path.abspath(lib_path)), exist_ok=True)
+    tmp = lib_path + f".tmp{os.getpid()}"
+    r = subprocess.run([hipcc] + FLAGS + ["-shared", "-o", tmp] + list(srcs), stdout=subprocess.PIPE,
+                       stderr=subprocess.STDOUT, text=True, env=env)
+    if r.returncode != 0:
+        raise RuntimeError("hipcc failed:\n" + r.stdout)
+    os.replace(tmp, lib_path)
+    if verbose:
+        print(f"[hf_cpu_amd] extension library ready: {lib_path}", file=sys.stderr, flush=True)
+    return lib_path
+
+
 def hipcc_path():
     for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
         if cand and os.path.exists(cand):

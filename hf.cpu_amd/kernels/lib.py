@@ -60,5 +60,18 @@ def library():
         return _lib
 
 
+def load_extension(path, signatures):
+    """A shared library with kernels of a part that is not the package's: ``signatures`` maps each
+    entry point to its ctypes argument types (the stream last; it returns an int, 0 = done).
+    The part calls them through ``Ops.call``."""
+    lib = ctypes.CDLL(path)
+    for name, args in signatures.items():
+        fn = getattr(lib, name)
+        fn.argtypes = list(args)
+        fn.restype = c_int
+    lib.path = path
+    return lib
+
+
 def last_error():
     return library().hfa_last_error().decode("utf-8", "replace")

@@ -148,6 +148,16 @@ class Ops:
         if rc != 0:
             raise EngineError(EINVAL if rc == 1 else ENOTSUP, last_error())
 
+    def call(self, entry_point, *args, what=None):
+        """Launches an entry point of an extension library (``kernels.lib.load_extension``) on the step's
+        stream: ``args`` are its arguments but the last, the stream. A deferred product is added up first,
+        since the kernel may read any tensor. Raises EngineError unless it returns 0."""
+        self.settle()
+        rc = entry_point(*args, self._stream())
+        if rc != 0:
+            raise EngineError(EINVAL if rc == 1 else ENOTSUP,
+                              f"{what or getattr(entry_point, '__name__', 'extension kernel')} returned {rc}")
+
     def scratch(self, name, shape, dtype):
         """A named work buffer that is reused from step to step; its contents are
         undefined on return. The same name always aliases the same memory."""

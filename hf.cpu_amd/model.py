@@ -4,8 +4,6 @@
 architecture, the registry gives its configuration class and plan function, the
 plan gives the parts, the parts declare the tensors the loader must find.
 """
-from dataclasses import dataclass
-
 import torch
 
 from .config import config_from_dict, read_config
@@ -27,17 +25,20 @@ def compute_dtype(name):
     return COMPUTE_DTYPES[name]
 
 
-@dataclass
 class Layer:
-    label: str
-    block: object
-    norm1: object
-    mixer: object
-    norm2: object
-    feed_forward: object
+    """A layer's block and the parts it arranges, by the names the plan gave them (also as attributes)."""
+
+    def __init__(self, label, block, named):
+        self.label, self.block, self.named = label, block, dict(named)
+        for name, part in self.named.items():
+            setattr(self, name, part)
 
     def parts(self):
-        return [self.block, self.norm1, self.mixer, self.norm2, self.feed_forward]
+        return [self.block] + list(self.named.values())
+
+    def cache_parts(self):
+        """(name, part) of the parts that keep a cache, in the plan's order."""
+        return [(n, p) for n, p in self.named.items() if hasattr(p, "cache_need")]
 
 
 class Model:
@@ -46,9 +47,8 @@ class Model:
         self.plan = plan
         self.config = config
         self.embedding = make_part("embedding", plan.embedding)
-        self.layers = [Layer(lp.label, make_part("block", lp.block), make_part("norm", lp.norm1),
-                             make_part("mixer", lp.mixer), make_part("norm", lp.norm2),
-                             make_part("feed_forward", lp.feed_forward)) for lp in plan.layers]
+        self.layers = [Layer(lp.label, make_part("block", lp.block),
+                             {name: make_part(role, spec) for name, role, spec in lp.parts}) for lp in plan.layers]
         self.final_norm = make_part("norm", plan.final_norm)
         self.head = make_part("head", plan.head)
         self.schedule = plan.schedule
@@ -111,20 +111,25 @@ class Model:
 
     # ---- what the cache manager needs to know -----------------------------
     def cache_needs(self):
-        """For each schedule entry: PagedKV, FixedState, or None (no cache of its own)."""
-        needs = []
+        """One entry for every (schedule entry, part of its layer that keeps a cache): PagedKV,
+        FixedState, or None (an entry that reads another entry's cache keeps none of its own).
+        ``cache_slots[i]`` says which of them schedule entry ``i`` uses: {part name: index}."""
+        needs, self.cache_slots = [], []
         for e in self.schedule:
-            mixer = self.layers[e.layer].mixer
-            need = mixer.cache_need() if e.cache_of is None and hasattr(mixer, "cache_need") else None
-            if need is not None and not isinstance(need, (PagedKV, FixedState)):
-                raise TypeError(f"{type(mixer).__name__}.cache_need() returned {need!r}")
-            needs.append(need)
+            slots = {}
+            for name, part in self.layers[e.layer].cache_parts():
+                need = part.cache_need() if e.cache_of is None else None
+                if need is not None and not isinstance(need, (PagedKV, FixedState)):
+                    raise TypeError(f"{type(part).__name__}.cache_need() returned {need!r}")
+                slots[name] = len(needs)
+                needs.append(need)
+            self.cache_slots.append(slots)
         return needs
 
     # ---- the forward pass of one step ----------------------------------------
     def forward(self, ops, step, caches, logits_out):
-        """Runs ``step``'s tokens through the schedule. ``caches[i]`` is the cache view
-        of schedule entry ``i`` (None if it needs none). Writes fp32 logits for
+        """Runs ``step``'s tokens through the schedule. ``caches[k]`` is the cache view
+        of entry ``k`` of ``cache_needs()`` (None if it needs none). Writes fp32 logits for
         ``step.logit_rows`` into ``logits_out`` ([R, V]; R may be 0)."""
         with ops.on_current_stream(), ops.section("total"):
             self._forward(ops, step, caches, logits_out)
@@ -133,12 +138,13 @@ class Model:
         T = step.n_tokens
         x = ops.scratch("residual", (T, self.hidden_size), torch.float32)
         self.embedding.forward(ops, step, x)
+        if not hasattr(self, "cache_slots"):
+            self.cache_needs()
         for i, e in enumerate(self.schedule):
             layer = self.layers[e.layer]
             own = e.cache_of is None
-            cache = caches[i if own else e.cache_of]
-            layer.block.forward(ops, step, x, layer.norm1, layer.mixer, layer.norm2, layer.feed_forward,
-                                cache, write_cache=own)
+            mine = {name: caches[k] for name, k in self.cache_slots[i if own else e.cache_of].items()}
+            layer.block.forward(ops, step, x, layer.named, mine, write_cache=own)
         ops.settle()
         R = step.n_logit_rows
         if R:

@@ -17,9 +17,8 @@ def qwen2_plan(cfg):
     for l in range(cfg.num_hidden_layers):
         prefix = f"model.layers.{l}."
         rotary = PartSpec("rotary", dict(head_dim=cfg.head_dim, rot_dim=cfg.head_dim, theta=cfg.rope_theta))
-        layers.append(LayerPlan(
-            label=prefix,
-            block=PartSpec("prenorm", dict(hidden_size=E)),
+        layers.append(LayerPlan.of(
+            prefix, PartSpec("prenorm", dict(hidden_size=E)),
             norm1=PartSpec("rmsnorm", dict(size=E, eps=cfg.rms_norm_eps, prefix=prefix + "input_layernorm.")),
             mixer=PartSpec("attention", dict(
                 hidden_size=E, n_heads=cfg.num_attention_heads, n_kv_heads=cfg.num_key_value_heads,

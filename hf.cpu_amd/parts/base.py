@@ -12,7 +12,8 @@ Interfaces by role (``step`` is the engine's StepInputs, ``ops`` its kernels):
   position      bind_tables(ops); store(ops, step, qkv, heads, kv_heads, head_dim, cache, write)
   mixer         cache_need(); forward(ops, step, h, cache, x, write_cache=True)     x += mixer(h)
   feed_forward  forward(ops, step, h, x)                                             x += ffn(h)
-  block         forward(ops, step, x, norm1, mixer, norm2, feed_forward, cache, write_cache)
+  block         forward(ops, step, x, parts, caches, write_cache)    parts: {name: part} as the plan names them;
+                                                                     caches: {name: cache view} of those that keep one
   head          forward(ops, h, out_logits)                  activation [R, E] -> fp32 [R, V]
 """
 from dataclasses import dataclass

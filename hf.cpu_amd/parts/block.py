@@ -14,11 +14,12 @@ class PreNormBlock(Part):
         super().__init__(prefix)
         self.E = hidden_size
 
-    def forward(self, ops, step, x, norm1, mixer, norm2, feed_forward, cache, write_cache=True):
+    def forward(self, ops, step, x, parts, caches, write_cache=True):
+        """``parts``: norm1, mixer, norm2, feed_forward; ``caches``: the mixer's, under its name."""
         h = ops.scratch("normed", (x.shape[0], self.E), ops.act_dtype)
-        norm1.forward(ops, x, h)      # also adds up a product the previous part deferred into x
-        ops.settle(x)                 # (nothing left to do unless the norm could not)
-        mixer.forward(ops, step, h, cache, x, write_cache)
-        norm2.forward(ops, x, h)
+        parts["norm1"].forward(ops, x, h)      # also adds up a product the previous part deferred into x
+        ops.settle(x)                          # (nothing left to do unless the norm could not)
+        parts["mixer"].forward(ops, step, h, caches.get("mixer"), x, write_cache)
+        parts["norm2"].forward(ops, x, h)
         ops.settle(x)
-        feed_forward.forward(ops, step, h, x)
+        parts["feed_forward"].forward(ops, step, h, x)

@@ -21,14 +21,46 @@ class PartSpec:
 
 @dataclass(frozen=True)
 class LayerPlan:
-    """One layer's parts. ``block`` names the arrangement (where norms and residual
-    sums sit); ``label`` is for messages only."""
+    """One layer: ``block`` names the arrangement (where norms and residual sums sit, which
+    branches there are) and ``parts`` the parts it arranges, as a mapping from the name the block
+    knows a part by to ``(role, PartSpec)``. A block may have any number of parts of any role: four
+    norms, two mixers side by side, no feed-forward. ``label`` is for messages only.
+
+    ``LayerPlan.of(label, block, norm1=..., mixer=..., norm2=..., feed_forward=...)`` is the short
+    way for the usual four: the role of a part is taken from its name (``norm*`` are norms)."""
     label: str
     block: PartSpec
-    norm1: PartSpec
-    mixer: PartSpec
-    norm2: PartSpec
-    feed_forward: PartSpec
+    parts: tuple = ()            # of (name, role, PartSpec); a tuple so that the plan stays hashable
+
+    @classmethod
+    def of(cls, label, block, **named):
+        """Parts by keyword; the role follows from the name: ``mixer*``, ``feed_forward*``, ``norm*``,
+        ``position*``, or give ``name=(role, spec)``."""
+        parts = []
+        for name, spec in named.items():
+            if isinstance(spec, tuple):
+                role, spec = spec
+            else:
+                role = next((r for r in ("mixer", "feed_forward", "norm", "position") if name.startswith(r)), None)
+                if role is None:
+                    raise ValueError(f"layer {label!r}: the role of part '{name}' does not follow from its name; "
+                                     f"give {name}=(role, spec)")
+            parts.append((name, role, spec))
+        return cls(label, block, tuple(parts))
+
+    def part(self, name):
+        for n, _, spec in self.parts:
+            if n == name:
+                return spec
+        raise KeyError(f"layer {self.label!r} has no part '{name}'")
+
+    def __getattr__(self, name):             # plan.layers[1].mixer, for the parts a layer has
+        if name.startswith("_") or name in ("label", "block", "parts"):
+            raise AttributeError(name)
+        try:
+            return self.part(name)
+        except KeyError as e:
+            raise AttributeError(str(e)) from None
 
 
 @dataclass(frozen=True)

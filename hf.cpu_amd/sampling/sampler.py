@@ -9,10 +9,9 @@ one draw ``r = uniform * sum`` picks the first candidate whose running sum excee
 
 The GPU does all of it (kernels in csrc/sampling.hip): argmax; the ordered best-k and the
 row's log-sum-exp, or, with ``top_k`` off (0) or beyond the best-k kernel's 1024, the whole
-row in order; and the draw from these candidates, by the same fp32 operations in the same
-order as ``pick_rows`` below, which stays the statement of the draw and what the tests
-compare the kernel with. The host gives each request's uniform number and reads one token
-a row.
+row in order; and the draw from these candidates, with every operation rounded to fp32 and nothing
+fused, in the reference's order. The host gives each request's uniform number and reads one
+token a row.
 """
 from dataclasses import dataclass
 
@@ -20,9 +19,7 @@ import numpy as np
 import torch
 
 from .. import memory
-
 from ..status import EINVAL, fail
-from .mathx import hfc_expf
 
 TOPK_KERNEL_MAX = 1024
 f32 = np.float32
@@ -48,50 +45,6 @@ class SamplerParams:
     @property
     def greedy(self):
         return self.temp <= 0
-
-
-def pick_rows(ids, logits, params, rngs):
-    """The draw for several rows with the same parameters: ``ids`` and ``logits`` are [R, k]
-    candidates already ordered (logit descending, id ascending) and cut to top_k; ``rngs[r]``
-    is row r's generator. Steps 3 to 6 of the pipeline in fp32 (src/sample.c:99-114): every
-    sum is a running fp32 sum in candidate order, as in the reference's loops (``cumsum``
-    adds one element at a time in the array's precision)."""
-    logits = np.asarray(logits, dtype=f32)
-    ids = np.asarray(ids)
-    R, k = logits.shape
-    col = np.arange(k)[None, :]
-    p = hfc_expf((logits - logits[:, :1]) / f32(params.temp))               # src/sample.c:99, src/mathx.c:7-32
-    p = (p / np.cumsum(p, axis=1, dtype=f32)[:, -1:]).astype(f32)
-    kept = np.full(R, k)
-    if params.min_p > 0:
-        below = p < f32(params.min_p) * p[:, :1]                 # p does not increase along the order
-        kept = np.maximum(np.where(below.any(axis=1), below.argmax(axis=1), k), 1)
-    if 0 < params.top_p < 1:
-        live = col < kept[:, None]
-        reached = (np.cumsum(np.where(live, p, f32(0)), axis=1, dtype=f32) >= f32(params.top_p)) & live
-        kept = np.where(reached.any(axis=1), reached.argmax(axis=1) + 1, kept)
-    live = col < kept[:, None]
-    cum = np.cumsum(np.where(live, p, f32(0)), axis=1, dtype=f32)
-    u = np.array([rng.uniform() for rng in rngs], dtype=f32)     # 24 random bits: exact in fp32
-    r = u * cum[np.arange(R), kept - 1]
-    over = (r[:, None] < cum) & live
-    at = np.where(over.any(axis=1), over.argmax(axis=1), kept - 1)
-    return [int(t) for t in ids[np.arange(R), at]]
-
-
-def pick(ids, logits, params, rng):
-    """One row of ``pick_rows``."""
-    return pick_rows(np.asarray(ids)[None, :], np.asarray(logits, dtype=f32)[None, :], params, [rng])[0]
-
-
-def order_on_host(row, top_k):
-    """All candidates of a row in order, cut to top_k if it is on (src/sample.c:59-64, 81-98): the
-    order that the device's kernels give, written out in numpy for the tests of ``pick``."""
-    row = np.asarray(row, dtype=f32)
-    order = np.argsort(-row, kind="stable")                 # logit descending, ties by id ascending
-    if 0 < top_k < len(order):
-        order = order[:top_k]
-    return order.astype(np.int64), row[order]
 
 
 @dataclass
@@ -144,8 +97,8 @@ class Sampler:
                 few.append(i)
             else:
                 whole.append(i)
-        # Either way the device draws (csrc/sampling.hip: the same fp32 operations in the same order
-        # as ``pick_rows``); the host gives each request's uniform number and reads back one token a row.
+        # Either way the device draws (csrc/sampling.hip); the host gives each request's uniform number and
+        # reads back one token a row.
         if few:
             numbers = np.zeros((R, 4), dtype=f32)
             numbers[:, :2] = 1                    # rows that are not drawn here: any harmless draw

@@ -16,7 +16,7 @@ from .engine import Engine
 from .engine.scheduler import Request, Scheduler
 from .kernels import Ops
 from .model import Model, compute_dtype
-from .parts.base import PagedKV
+from .parts.base import FixedState, PagedKV
 from .sampling import Sampler, SamplerParams
 from .status import EINVAL, ENOMEM, fail
 
@@ -37,9 +37,14 @@ class Generation:
 
 
 def cache_bytes_per_token(model):
-    """Bytes of cache one token takes over all schedule entries."""
+    """Bytes of paged cache one token takes over all schedule entries."""
     elem = 4 if model.dtype == torch.float32 else 2
     return sum((n.k_width + n.v_width) * elem for n in model.cache_needs() if isinstance(n, PagedKV))
+
+
+def state_bytes_per_request(model):
+    """Bytes of fixed-size state one request holds over all schedule entries (fp32)."""
+    return sum(4 * n.n_floats for n in model.cache_needs() if isinstance(n, FixedState))
 
 
 class Session:
@@ -60,11 +65,15 @@ class Session:
             self.model_dir, self.identity = None, ("random", id(model), seed)
             self.model = Model.from_random(model, seed, dtype, self.ops)
         per_token = cache_bytes_per_token(self.model)
+        free, _ = torch.cuda.mem_get_info(self.ops.device)
+        free = int(free * 0.8) - (int(max_seqs) + 1) * state_bytes_per_request(self.model)
+        if free < 0:
+            fail(ENOMEM, f"no memory for the state of {max_seqs} requests "
+                         f"({state_bytes_per_request(self.model)} bytes each)")
         if kv_tokens is None:
             kv_tokens = int(ctx_max) * int(max_seqs)
             if per_token:
-                free, _ = torch.cuda.mem_get_info(self.ops.device)
-                kv_tokens = min(kv_tokens, int(free * 0.8) // per_token)
+                kv_tokens = min(kv_tokens, free // per_token)
         ctx_max = int(min(ctx_max, kv_tokens))
         if kv_tokens < page_size:
             fail(ENOMEM, f"no memory for a cache of even one page ({per_token} bytes per token)")

@@ -327,3 +327,88 @@ def test_decoded_tokens_between_prompt_portions_keep_their_places(gpu, tiny, dty
     # and the requests go on from there
     more = engine.step([(a, [reqs[a][21]], [0]), (b, reqs[b][30:33], [2])]).float().cpu().numpy()
     helpers.compare({(a, 21): more[0], (b, 32): more[1]}, want, TOL[dtype], f"{name} {dtype} the step after")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_truncate_then_other_tokens(gpu, tiny, dtype):
+    """A request is cut back (src/model.c:305) inside a page and to a page's edge, and fed other tokens:
+    the logits are those of the sequence as it then reads. With a window (configuration B) a cut that
+    would need pages the window has given back is refused and changes nothing; one that does not is
+    served, across the window's edge."""
+    from hf_cpu_amd.status import EngineError
+    import plain
+    name, cfg, d, reqs, _ = tiny
+    P = helpers.PAGE[name]
+    rng = np.random.default_rng(5)
+    toks = reqs["r3"]                                             # 70 (A) or 100 (B) tokens
+    pcfg, w = plain.read_model(d)
+    engine = engine_for(d, dtype, name, 256)
+    engine.step([("t", toks, [])])
+    # B's window of 32 lets go of pages as the request grows: only short cuts stay possible there
+    cuts = [len(toks) - 3, len(toks) - P - 5, (len(toks) - 2 * P) // P * P] if name == "A" else [len(toks) - 3, len(toks) + 3]
+    seq = list(toks)
+    for cut in cuts:
+        more = [int(t) for t in rng.integers(0, cfg["vocab_size"], 7)]
+        engine.truncate("t", cut)
+        assert engine.length("t") == cut
+        engine.manager.check()
+        seq = seq[:cut] + more
+        got = engine.step([("t", more[:5], [0, 4])]).float().cpu().numpy()
+        got = np.concatenate([got, engine.step([("t", more[5:6], [0])]).float().cpu().numpy(),
+                              engine.step([("t", more[6:], [0])]).float().cpu().numpy()])
+        want = plain.forward(pcfg, w, seq)
+        scale = float(np.max(np.abs(want)))
+        for row, pos in zip(got, (cut, cut + 4, cut + 5, cut + 6)):
+            err = float(np.max(np.abs(row - want[pos]))) / scale
+            assert err <= TOL[dtype], f"{name} {dtype}: cut to {cut}, position {pos}: {err:.3e}"
+    if name == "B":                                               # window 32: pages before position len - 32 are gone
+        before = (engine.length("t"), [list(t) for t in engine.manager.held["t"].tables])
+        with pytest.raises(EngineError) as e:
+            engine.truncate("t", 20)
+        assert e.value.code == "ENOTSUP"
+        assert (engine.length("t"), [list(t) for t in engine.manager.held["t"].tables]) == before
+    engine.release("t")
+    engine.manager.check()
+    assert all(p.n_held == 0 for p in engine.manager.pools)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_what_a_page_held_before_does_not_matter(gpu, tiny, dtype):
+    """Every row of the cache starts as NaN (as if each page's last owner had overflowed): a step reads
+    only rows that it or an earlier step of the same request wrote, and what it reads beside them
+    (rows past a request's end, pages a window has given back, whole blocks of keys fetched for a few)
+    has weight zero and must not reach the result: 0 x NaN is NaN. Mixed trace, pages used again."""
+    name, cfg, d, reqs, want = tiny
+    steps = helpers.trace_mixed(reqs, seed=11)
+    engine = engine_for(d, dtype, name, helpers.max_live_tokens(steps))
+    for view in engine.storage.views:
+        if hasattr(view, "k"):
+            view.k.fill_(float("nan"))
+            view.v.fill_(float("inf"))
+    got = helpers.run_trace_in_engine(engine, steps)
+    assert all(np.isfinite(row).all() for row in got.values()), "a stale row of the cache reached the logits"
+    helpers.compare(got, want, TOL[dtype], f"{name} {dtype} on a cache of NaN")
+    assert any(p.reused > 0 for p in engine.manager.pools)
+    # and with the pages poisoned again between a prompt and its decoded tokens: only rows of live requests are kept
+    whole = helpers.trace_tail({"r2": reqs["r2"]}, tail=8)
+    engine = engine_for(d, dtype, name, 256)
+    got, places = {}, helpers.wanted_places(whole)
+    for i, s in enumerate(whole):
+        rows = engine.step([(e["id"], e["tokens"], e["want"]) for e in s["entries"]]).float().cpu().numpy()
+        for row, key in zip(rows, places[s["step"]]):
+            got[key] = row.copy()
+        if i == 0:
+            h = engine.manager.held["r2"]
+            for g, group in enumerate(engine.manager.groups):
+                own = [p for p in h.tables[g] if p >= 0]
+                for e in group.entries:
+                    view = engine.storage.views[e]
+                    P = view.page_tokens
+                    keep_k = {p: view.k[p * P:(p + 1) * P].clone() for p in own}
+                    keep_v = {p: view.v[p * P:(p + 1) * P].clone() for p in own}
+                    view.k.fill_(float("inf"))
+                    view.v.fill_(float("nan"))
+                    for p in own:
+                        view.k[p * P:(p + 1) * P] = keep_k[p]
+                        view.v[p * P:(p + 1) * P] = keep_v[p]
+    helpers.compare(got, {"r2": want["r2"]}, TOL[dtype], f"{name} {dtype} decoding beside poisoned pages")

@@ -647,12 +647,15 @@ def test_order_rows(ops32, V):
 
 @pytest.mark.parametrize("V", [1, 7, 1000, 4097, 152064])
 def test_draw_rows(ops32, V):
-    """The device's draw over a whole ordered row against the sampler's written-out draw on the same
-    candidates with the same uniform numbers: the same token, row for row. The rows differ in
+    """The device's draw over a whole ordered row against the plain sampler (tests/plain.py, from the row's
+    logits, with its own ordering and its own exponential) with the same uniform numbers: the same token,
+    row for row; at the largest sizes, where the plain sampler's scalar loops take seconds a row, eight rows
+    against it and all of them against its vectorised stand-in in tests/host_draw.py. The rows differ in
     temperature, in each cut being on or off, and in how peaked they are (a peaked row ends the
     top-p cut within a few candidates, a flat one takes it far into the row: past several of the
     kernel's pieces); uniform numbers include 0 and the largest below 1."""
-    from hf_cpu_amd.sampling import SamplerParams, pick
+    from hf_cpu_amd.sampling import SamplerParams
+    from host_draw import pick
     rng = np.random.default_rng(V + 1)
 
     class Fixed:
@@ -680,9 +683,13 @@ def test_draw_rows(ops32, V):
     numbers = np.array([(t, tp, mp, u) for (t, _, tp, mp), u in zip(cases, us)], dtype=np.float32)
     cuts = np.array([k if 0 < k < V else V for _, k, _, _ in cases], dtype=np.int32)
     got = ops32.draw_rows(ids, vals, torch.from_numpy(numbers).cuda(), torch.from_numpy(cuts).cuda()).cpu().numpy()
+    by_plain = range(R) if V <= 1000 else range(0, R, 12)
     for r, (temp, top_k, top_p, min_p) in enumerate(cases):
+        what = f"row {r}: temp {temp} top_k {top_k} top_p {top_p} min_p {min_p} u {us[r]}"
+        if r in by_plain:
+            assert int(got[r]) == plain.sample(logits[r], temp, top_k, top_p, min_p, Fixed(us[r])), what
         want = pick(host_ids[r, :cuts[r]], host_vals[r, :cuts[r]], SamplerParams(temp, top_k, top_p, min_p), Fixed(us[r]))
-        assert int(got[r]) == want, f"row {r}: temp {temp} top_k {top_k} top_p {top_p} min_p {min_p} u {us[r]}"
+        assert int(got[r]) == want, what
 
 
 def test_sampler_with_rows_of_every_kind_in_one_step(ops32):

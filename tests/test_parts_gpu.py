@@ -156,31 +156,60 @@ def toy_plan_factory():
                     state.mul_(self.decay).add_(h[t].float(), alpha=1 - self.decay)
                     x[t] += self.w.float() @ state
 
+    @register_part("mixer", "toy_ema_kernel")
+    class ToyEmaKernel(ToyEma):
+        """The same mixer with a kernel of its own, from a library that is not the package's
+        (tests/toy_kernels/toy_ema.hip): the step's shape is all the host looks at, so steps that use it
+        may be captured into graphs."""
+        graph_safe = True
+        _lib = None
+
+        @classmethod
+        def lib(cls):
+            if cls._lib is None:
+                from ctypes import c_float, c_int, c_void_p as P
+                from hf_cpu_amd.kernels import load_extension
+                from hf_cpu_amd.kernels.build import build_extension
+                here = os.path.join(os.path.dirname(os.path.abspath(__file__)), "toy_kernels")
+                path = os.path.join(here, "libtoy.so")
+                if not os.path.exists(path):
+                    build_extension([os.path.join(here, "toy_ema.hip")], path)
+                cls._lib = load_extension(path, {"toy_ema": [P, c_int, P, P, c_int, P, P, P, c_int, c_int, c_float, P]})
+            return cls._lib
+
+        def forward(self, ops, step, h, cache, x, write_cache=True):
+            code = {torch.float32: 0, torch.bfloat16: 1}
+            ops.call(self.lib().toy_ema, h.data_ptr(), code[h.dtype], cache.state.data_ptr(), self.w.data_ptr(),
+                     code[self.w.dtype], x.data_ptr(), step.q_start.data_ptr(), step.seq_slot.data_ptr(), step.n_seqs,
+                     self.E, self.decay, what="toy_ema")
+
     @dataclasses.dataclass(frozen=True)
     class ToyConfig:
         architecture: str
         vocab_size: int
         hidden_size: int
         decay: float
+        mixer_kind: str = "toy_ema"
 
         @classmethod
         def from_dict(cls, obj, origin="config.json"):
-            return cls(obj["architectures"][0], obj["vocab_size"], obj["hidden_size"], obj["decay"])
+            return cls(obj["architectures"][0], obj["vocab_size"], obj["hidden_size"], obj["decay"],
+                       obj.get("mixer_kind", "toy_ema"))
 
     def toy_plan(cfg):
         E = cfg.hidden_size
 
         def layer(l, mixer):
             pre = f"layers.{l}."
-            return hf_cpu_amd.LayerPlan(
-                label=pre, block=PartSpec("prenorm", dict(hidden_size=E)),
+            return hf_cpu_amd.LayerPlan.of(
+                pre, PartSpec("prenorm", dict(hidden_size=E)),
                 norm1=PartSpec("rmsnorm", dict(size=E, eps=1e-5, prefix=pre + "norm1.")), mixer=mixer,
                 norm2=PartSpec("rmsnorm", dict(size=E, eps=1e-5, prefix=pre + "norm2.")),
                 feed_forward=PartSpec("gated_mlp", dict(hidden_size=E, intermediate_size=2 * E, prefix=pre + "mlp.")))
         att = PartSpec("attention", dict(hidden_size=E, n_heads=2, n_kv_heads=1, head_dim=16, qkv_bias=False,
                                          window=0, prefix="layers.0.attn.",
                                          position=PartSpec("rotary", dict(head_dim=16, rot_dim=16, theta=1e4))))
-        toy = PartSpec("toy_ema", dict(hidden_size=E, decay=cfg.decay, prefix="layers.1.ema."))
+        toy = PartSpec(cfg.mixer_kind, dict(hidden_size=E, decay=cfg.decay, prefix="layers.1.ema."))
         return hf_cpu_amd.ModelPlan(
             hidden_size=E, vocab_size=cfg.vocab_size,
             embedding=PartSpec("lookup", dict(vocab_size=cfg.vocab_size, hidden_size=E, prefix="embed.")),
@@ -230,10 +259,11 @@ def toy_reference(w, toks, decay):
     return plain.linear(plain.rmsnorm(x, w["final.weight"], 1e-5), w["embed.weight"])
 
 
-def test_toy_mixer_with_state_and_a_schedule_that_repeats(gpu, tmp_path):
+def make_toy_model(tmp_path, mixer_kind="toy_ema"):
     toy_plan_factory()
-    cfg = {"architectures": ["ToyEmaForCausalLM"], "vocab_size": 90, "hidden_size": 24, "decay": 0.8}
-    d = str(tmp_path / "toy")
+    cfg = {"architectures": ["ToyEmaForCausalLM"], "vocab_size": 90, "hidden_size": 24, "decay": 0.8,
+           "mixer_kind": mixer_kind}
+    d = str(tmp_path / ("toy_" + mixer_kind))
     os.makedirs(d)
     with open(os.path.join(d, "config.json"), "w") as f:
         json.dump(cfg, f)
@@ -247,6 +277,14 @@ def test_toy_mixer_with_state_and_a_schedule_that_repeats(gpu, tmp_path):
         std = {"embed.weight": 0.5}.get(s.name, 0.3 if s.kind == "matrix" else 0.1)
         w[s.name] = ((1.0 if s.kind == "vector" else 0.0) + rng.standard_normal(s.shape) * std).astype(np.float32)
     helpers.write_safetensors(os.path.join(d, "model.safetensors"), w)
+    return d, w, rng
+
+
+@pytest.mark.parametrize("mixer_kind", ["toy_ema", "toy_ema_kernel"])
+def test_toy_mixer_with_state_and_a_schedule_that_repeats(gpu, tmp_path, mixer_kind):
+    """The toy mixer in eager tensor arithmetic, and the same with a kernel of its own that the test
+    brings in a library of its own (no file of the package knows either)."""
+    d, w, rng = make_toy_model(tmp_path, mixer_kind)
     reqs = {f"r{i}": [int(t) for t in rng.integers(0, 90, n)] for i, n in enumerate([5, 23, 40, 31])}
     w64 = {k: v.astype(np.float64) for k, v in w.items()}
     want = {r: toy_reference(w64, t, 0.8) for r, t in reqs.items()}
@@ -255,6 +293,206 @@ def test_toy_mixer_with_state_and_a_schedule_that_repeats(gpu, tmp_path):
                                         max_seqs=3)
         got = helpers.run_trace_in_engine(engine, steps)
         helpers.compare(got, want, 2e-5, "toy model")
+        assert not engine.manager.held
+
+
+def test_toy_mixer_with_a_kernel_of_its_own_replays_from_graphs(gpu, tmp_path):
+    """The toy mixer's own kernel declares itself safe to capture: decode steps of a model that holds
+    it are replayed from graphs, and give what the model written out directly gives."""
+    d, w, rng = make_toy_model(tmp_path, "toy_ema_kernel")
+    w64 = {k: v.astype(np.float64) for k, v in w.items()}
+    reqs = {f"r{i}": [int(t) for t in rng.integers(0, 90, 30)] for i in range(3)}
+    want = {r: toy_reference(w64, t, 0.8) for r, t in reqs.items()}
+    engine = hf_cpu_amd.load_engine(d, dtype="float32", page_tokens=8, max_tokens=192, max_seqs=3)
+    assert engine.use_graphs
+    steps = [{"step": 0, "entries": [{"id": r, "tokens": t[:6], "want": [5]} for r, t in reqs.items()], "end": []}]
+    for i in range(6, 30):
+        steps.append({"step": len(steps), "entries": [{"id": r, "tokens": [t[i]], "want": [0]} for r, t in reqs.items()],
+                      "end": list(reqs) if i == 29 else []})
+    got = helpers.run_trace_in_engine(engine, steps)
+    helpers.compare(got, want, 2e-5, "toy model, decode steps from graphs")
+    assert engine.graph_replays >= 20
+
+
+def toy_greedy(w64, prompt, n, decay=0.8):
+    toks = list(prompt)
+    for _ in range(n):
+        toks.append(int(np.argmax(toy_reference(w64, toks, decay)[-1])))
+    return toks[len(prompt):]
+
+
+def test_toy_mixer_through_the_scheduler_with_forks_and_a_tight_cache(gpu, tmp_path):
+    """A model with per-request state of fixed size served by the scheduler: continuations forked from
+    one prompt take a copy of its state; a cache too small for everybody throws requests out, whose
+    state starts from zero again when they come back. Every sequence ends with the tokens that the
+    model written out directly gives it."""
+    import hf_cpu_amd.session as S
+    d, w, rng = make_toy_model(tmp_path, "toy_ema_kernel")
+    w64 = {k: v.astype(np.float64) for k, v in w.items()}
+    prompts = [[int(t) for t in rng.integers(0, 90, n)] for n in (9, 17, 5, 12)]
+    want = [toy_greedy(w64, p, 14) for p in prompts]
+    s = S.Session(d, dtype="float32", ctx_max=48, batch=8, page_size=4, max_seqs=4, kv_tokens=72)
+    gens = s.generate(prompts, n=2, temp=0.0, max_tokens=14)
+    assert len(gens) == 8 and all(g.error is None and g.stop == "length" for g in gens)
+    for i, g in enumerate(gens):
+        assert g.tokens == want[i // 2], f"sequence {i} (prompt {i // 2}): {g.tokens} != {want[i // 2]}"
+    assert sum(g.preemptions for g in gens) > 0, "the cache was meant to be too small for everybody"
+    s.engine.manager.check()
+    assert not s.engine.manager.held
+
+
+def blocks_plan_factory():
+    """Registers three toy arrangements of a layer, none of which is the package's: one with four norms
+    (a norm before and after each branch), one whose mixer and feed-forward read the same normed input
+    and are added together, and one that has a mixer and nothing else. The layer plan names the parts
+    each needs; the package's model passes them through as a mapping."""
+
+    @register_part("block", "toy_four_norms")
+    class FourNorms(Part):
+        def __init__(self, hidden_size, prefix=""):
+            super().__init__(prefix)
+            self.E = hidden_size
+
+        def branch(self, ops, x, pre, post, run):
+            h = torch.empty((x.shape[0], self.E), dtype=ops.act_dtype, device=x.device)
+            pre.forward(ops, x, h)
+            y = torch.zeros_like(x)
+            run(h, y)
+            ops.settle(y)
+            out = torch.empty_like(h)
+            post.forward(ops, y, out)
+            x += out.float()
+
+        def forward(self, ops, step, x, parts, caches, write_cache=True):
+            ops.settle(x)
+            self.branch(ops, x, parts["norm_in"], parts["norm_mixed"],
+                        lambda h, y: parts["mixer"].forward(ops, step, h, caches.get("mixer"), y, write_cache))
+            self.branch(ops, x, parts["norm_mid"], parts["norm_out"],
+                        lambda h, y: parts["feed_forward"].forward(ops, step, h, y))
+
+    @register_part("block", "toy_parallel")
+    class Parallel(Part):
+        def __init__(self, hidden_size, prefix=""):
+            super().__init__(prefix)
+            self.E = hidden_size
+
+        def forward(self, ops, step, x, parts, caches, write_cache=True):
+            h = torch.empty((x.shape[0], self.E), dtype=ops.act_dtype, device=x.device)
+            parts["norm"].forward(ops, x, h)
+            ops.settle(x)
+            parts["mixer"].forward(ops, step, h, caches.get("mixer"), x, write_cache)
+            parts["feed_forward"].forward(ops, step, h, x)            # the same input: both branches start at one norm
+
+    @register_part("block", "toy_mixer_only")
+    class MixerOnly(Part):
+        def __init__(self, hidden_size, prefix=""):
+            super().__init__(prefix)
+            self.E = hidden_size
+
+        def forward(self, ops, step, x, parts, caches, write_cache=True):
+            h = torch.empty((x.shape[0], self.E), dtype=ops.act_dtype, device=x.device)
+            parts["norm"].forward(ops, x, h)
+            ops.settle(x)
+            parts["mixer"].forward(ops, step, h, caches.get("mixer"), x, write_cache)
+
+    @dataclasses.dataclass(frozen=True)
+    class BlocksConfig:
+        architecture: str
+        vocab_size: int
+        hidden_size: int
+
+        @classmethod
+        def from_dict(cls, obj, origin="config.json"):
+            return cls(obj["architectures"][0], obj["vocab_size"], obj["hidden_size"])
+
+    def blocks_plan(cfg):
+        E = cfg.hidden_size
+
+        def norm(name):
+            return PartSpec("rmsnorm", dict(size=E, eps=1e-5, prefix=name + "."))
+
+        def attention(l, window=0):
+            return PartSpec("attention", dict(hidden_size=E, n_heads=2, n_kv_heads=2, head_dim=16, qkv_bias=False,
+                                              window=window, prefix=f"layers.{l}.attn.",
+                                              position=PartSpec("rotary", dict(head_dim=16, rot_dim=16, theta=1e4))))
+
+        def mlp(l):
+            return PartSpec("gated_mlp", dict(hidden_size=E, intermediate_size=2 * E, prefix=f"layers.{l}.mlp."))
+        layers = (
+            hf_cpu_amd.LayerPlan.of("layers.0.", PartSpec("toy_four_norms", dict(hidden_size=E)),
+                                    norm_in=norm("layers.0.n0"), mixer=attention(0), norm_mixed=norm("layers.0.n1"),
+                                    norm_mid=norm("layers.0.n2"), feed_forward=mlp(0), norm_out=norm("layers.0.n3")),
+            hf_cpu_amd.LayerPlan.of("layers.1.", PartSpec("toy_parallel", dict(hidden_size=E)),
+                                    norm=norm("layers.1.n0"), mixer=attention(1, window=7), feed_forward=mlp(1)),
+            hf_cpu_amd.LayerPlan.of("layers.2.", PartSpec("toy_mixer_only", dict(hidden_size=E)),
+                                    norm=norm("layers.2.n0"), mixer=attention(2)),
+        )
+        return hf_cpu_amd.ModelPlan(
+            hidden_size=E, vocab_size=cfg.vocab_size,
+            embedding=PartSpec("lookup", dict(vocab_size=cfg.vocab_size, hidden_size=E, prefix="embed.")),
+            layers=layers, schedule=tuple(ScheduleEntry(l) for l in range(3)),
+            final_norm=norm("final"),
+            head=PartSpec("linear", dict(vocab_size=cfg.vocab_size, hidden_size=E, tied=True, tied_to="embed.weight",
+                                         prefix="head.")))
+    register_architecture("ToyBlocksForCausalLM", BlocksConfig, blocks_plan)
+
+
+def blocks_reference(w, toks):
+    """The model of blocks_plan_factory over a whole sequence, written out directly (float64)."""
+    T = len(toks)
+    x = w["embed.weight"][toks]
+
+    def norm(x, name):
+        return plain.rmsnorm(x, w[name + ".weight"], 1e-5)
+
+    def attn(h, l, window=0):
+        pre = f"layers.{l}.attn."
+        q = plain.rope(plain.linear(h, w[pre + "q_proj.weight"]).reshape(T, 2, 16), range(T), 16, 1e4)
+        k = plain.rope(plain.linear(h, w[pre + "k_proj.weight"]).reshape(T, 2, 16), range(T), 16, 1e4)
+        v = plain.linear(h, w[pre + "v_proj.weight"]).reshape(T, 2, 16)
+        return plain.linear(plain.attention(q, k, v, window).reshape(T, 32), w[pre + "o_proj.weight"])
+
+    def mlp(h, l):
+        pre = f"layers.{l}.mlp."
+        return plain.swiglu_mlp(h, w[pre + "gate_proj.weight"], w[pre + "up_proj.weight"], w[pre + "down_proj.weight"])
+    x = x + norm(attn(norm(x, "layers.0.n0"), 0), "layers.0.n1")
+    x = x + norm(mlp(norm(x, "layers.0.n2"), 0), "layers.0.n3")
+    h = norm(x, "layers.1.n0")
+    x = x + attn(h, 1, window=7) + mlp(h, 1)
+    x = x + attn(norm(x, "layers.2.n0"), 2)
+    return plain.linear(norm(x, "final"), w["embed.weight"])
+
+
+def test_toy_blocks_with_four_norms_with_parallel_branches_and_without_a_feed_forward(gpu, tmp_path):
+    """Layers that are not 'norm, mixer, norm, feed-forward': the plan names each layer's parts, the
+    block gets them as a mapping. Whole, in portions and mixed, against the model written out."""
+    blocks_plan_factory()
+    cfg = {"architectures": ["ToyBlocksForCausalLM"], "vocab_size": 80, "hidden_size": 24}
+    d = str(tmp_path / "blocks")
+    os.makedirs(d)
+    with open(os.path.join(d, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    model = hf_cpu_amd.Model.from_config(hf_cpu_amd.config_from_dict(cfg))
+    assert sorted(model.layers[0].named) == ["feed_forward", "mixer", "norm_in", "norm_mid", "norm_mixed", "norm_out"]
+    assert sorted(model.layers[2].named) == ["mixer", "norm"]
+    needs = model.cache_needs()
+    assert [n.window for n in needs] == [0, 7, 0] and model.cache_slots == [{"mixer": 0}, {"mixer": 1}, {"mixer": 2}]
+    rng = np.random.default_rng(9)
+    w = {}
+    for s in model.param_specs():
+        if s.optional:
+            continue
+        std = {"embed.weight": 0.5}.get(s.name, 0.3 if s.kind == "matrix" else 0.1)
+        w[s.name] = ((1.0 if s.kind == "vector" else 0.0) + rng.standard_normal(s.shape) * std).astype(np.float32)
+    helpers.write_safetensors(os.path.join(d, "model.safetensors"), w)
+    reqs = {f"r{i}": [int(t) for t in rng.integers(0, 80, n)] for i, n in enumerate([4, 21, 38, 30])}
+    w64 = {k: v.astype(np.float64) for k, v in w.items()}
+    want = {r: blocks_reference(w64, t) for r, t in reqs.items()}
+    for steps in (helpers.trace_whole(reqs), helpers.trace_portions(reqs), helpers.trace_mixed(reqs, seed=6, max_live=3)):
+        engine = hf_cpu_amd.load_engine(d, dtype="float32", page_tokens=8, max_tokens=helpers.max_live_tokens(steps),
+                                        max_seqs=3)
+        got = helpers.run_trace_in_engine(engine, steps)
+        helpers.compare(got, want, 2e-5, "toy blocks")
         assert not engine.manager.held
 
 
@@ -349,8 +587,8 @@ def routed_plan_factory():
 
         def layer(l, mixer, ffn):
             pre = f"layers.{l}."
-            return hf_cpu_amd.LayerPlan(
-                label=pre, block=PartSpec("prenorm", dict(hidden_size=E)),
+            return hf_cpu_amd.LayerPlan.of(
+                pre, PartSpec("prenorm", dict(hidden_size=E)),
                 norm1=PartSpec("rmsnorm", dict(size=E, eps=1e-6, prefix=pre + "norm1.")), mixer=mixer,
                 norm2=PartSpec("rmsnorm", dict(size=E, eps=1e-6, prefix=pre + "norm2.")), feed_forward=ffn)
         learned = PartSpec("toy_learned", dict(head_dim=16, max_positions=cfg.max_positions, prefix="layers.0.attn."))

@@ -83,6 +83,9 @@ def test_attention_reduces_to_library_routines():
     assert np.allclose(plain.attention(q[:1], k[:1], v[:1])[0, 0], v[0, 0])
     z = plain.attention(np.zeros((T, H, D)), k, v)
     assert np.allclose(z[-1, 0], v[:, 0].mean(axis=0)) and np.allclose(z[-1, 5], v[:, 1].mean(axis=0))
+    # heads 1 and 4 of six on two key/value heads: h // (H / G) gives 0 and 1, h % G would give 1 and 0
+    assert np.allclose(z[-1, 1], v[:, 0].mean(axis=0)) and np.allclose(z[-1, 4], v[:, 1].mean(axis=0))
+    assert not np.allclose(z[-1, 1], v[:, 1].mean(axis=0))
 
 
 def test_window_mask_edges():
@@ -156,7 +159,7 @@ def test_exponential_of_the_reference():
     relative error below 4e-7 from -87 to 88 in steps of 0.0137, exp(0) = 1, exp(-100) = 0, a finite
     value for 1000. The product's vectorised routine gives the same bits as the plain one."""
     import math
-    from hf_cpu_amd.sampling.mathx import hfc_expf
+    from host_draw import hfc_expf
     xs = np.arange(-87.0, 88.0, 0.0137, dtype=np.float32)
     got = np.array([plain.expf(x) for x in xs], dtype=np.float32)
     ref = np.exp(xs.astype(np.float64))

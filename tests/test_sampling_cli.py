@@ -7,7 +7,8 @@ import pytest
 import plain
 from hf_cpu_amd.cli import opts as O
 from hf_cpu_amd.cli.proto import Out, Reader, quote
-from hf_cpu_amd.sampling import Rng, SamplerParams, order_on_host, pick
+from host_draw import order_on_host, pick, pick_rows
+from hf_cpu_amd.sampling import Rng, SamplerParams
 from hf_cpu_amd.status import EngineError
 
 
@@ -36,7 +37,6 @@ def test_rows_drawn_together_are_drawn_as_alone(params):
     """Many rows of one step in one call: each row's token is what the plain sampler draws for
     that row with that row's generator, whatever the other rows hold (a row that keeps one
     candidate beside rows that keep all of them)."""
-    from hf_cpu_amd.sampling.sampler import pick_rows
     rng = np.random.default_rng(1)
     temp, top_k, top_p, min_p = params
     logits = (rng.standard_normal((17, 500)) * 3).astype(np.float32)

@@ -280,3 +280,31 @@ def test_a_cancellation_deep_in_a_long_queue_is_seen_within_32_steps():
         s.step()
     assert victim.error is not None and victim.error.code == "ECANCEL" and victim.admitted_at == -1
     assert all(350 not in [r for r, _, _ in step] for step in eng.log)
+
+
+def test_more_decoding_requests_than_the_token_budget_take_turns():
+    """Four requests decode under a budget of 3 tokens a step: every step holds three decoded tokens,
+    nobody waits more than one step in a row, pages are reserved only for those that run, and every
+    request ends with the tokens it gets alone."""
+    eng, sch = make(budget=3, n_pages=16, page=4, slots=4, ctx=64)
+    reqs = [sch.submit(Request(f"r{i}", [1, 2, 3][:1 + i % 3], greedy(), max_tokens=9)) for i in range(4)]
+    sch.run()
+    assert all(r.stop == "length" and len(r.generated) == 9 for r in reqs)
+    assert all(r.generated == [10 + i for i in range(9)] for r in reqs)          # the script's tokens, in order
+    decode_steps = [s for s in eng.log if all(n == 1 for _, n, _ in s) and len(s) > 1]
+    full = [s for s in decode_steps if len(s) == 3]
+    assert len(full) >= 8
+    for r in reqs:                               # between its first and its last step nobody waits two steps in a row
+        ran = [i for i, s in enumerate(eng.log) if any(e[0] == r.req_id for e in s)]
+        assert max(b - a for a, b in zip(ran, ran[1:])) <= 2, (r.req_id, ran)
+    assert not eng.manager.held
+    # Three requests at a page's edge, two free pages, a budget of two: pages are asked for the two that
+    # run, not for all three (which would not fit and cost one of them its cache).
+    eng2, sch2 = make(budget=16, n_pages=5, page=4, slots=3, ctx=12)
+    rs = [sch2.submit(Request(f"q{i}", [1, 2, 3], greedy(), max_tokens=3)) for i in range(3)]
+    sch2.step()
+    sch2.step()
+    assert [eng2.manager.held[r.req_id].length for r in rs] == [4, 4, 4] and eng2.manager.pools[0].n_free == 2
+    sch2.token_budget = 2
+    sch2.run()
+    assert all(r.error is None and len(r.generated) == 3 for r in rs) and sum(r.preemptions for r in rs) == 0

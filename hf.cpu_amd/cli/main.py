@@ -47,19 +47,24 @@ class Cli:
         except OSError as e:
             from ..status import EIO
             fail(EIO, f"cannot read {cfg}: {e.strerror}")
-        ident = (os.path.abspath(path), st.st_size, st.st_mtime, eff["random-weights"])
+        ident = (os.path.abspath(path), st.st_size, st.st_mtime, eff["random-weights"], eff["window"])
         if self.session is not None and self.session.cli_identity == ident:
             return self.session
         self.session = None
         so = self.opts
+        over = None
+        if eff["window"] is not None:               # the window of config.json replaced (0: no window)
+            over = {"use_sliding_window": eff["window"] > 0}
+            if eff["window"] > 0:
+                over["sliding_window"] = eff["window"]
         if eff["random-weights"] is not None:
             from ..config import read_config
-            model, seed = read_config(path), eff["random-weights"]
+            model, seed = read_config(path, over), eff["random-weights"]
         else:
             model, seed = path, 0
         t0 = time.monotonic()
         s = Session(model, dtype=so["dtype"], ctx_max=so["ctx-max"], batch=so["batch"], page_size=so["page-size"],
-                    max_seqs=so["max-seqs"], kv_tokens=so["kv-tokens"] or None, seed=seed)
+                    max_seqs=so["max-seqs"], kv_tokens=so["kv-tokens"] or None, seed=seed, config_overrides=over)
         s.cli_identity = ident
         self.log("info", f"model={path} dtype={so['dtype']} load_ms={(time.monotonic() - t0) * 1e3:.0f} "
                          f"kv_bytes={s.engine.storage.nbytes()}")
@@ -150,6 +155,15 @@ class Cli:
                         q.cancel = True
                 return orig_submit(r, forks=forks)
             sch.submit = submit
+            if LEVELS.index(cli.opts["log-level"]) >= LEVELS.index("debug"):
+                def on_step(number, plan):           # what each step holds, at the debug level
+                    decoded = sum(1 for r, n, _ in plan.entries if n == 1 and r.n_fed > 0)
+                    portions = " ".join(f"{r.req_id}:{r.n_fed}+{n}" for r, n, _ in plan.entries if not (n == 1 and r.n_fed > 0))
+                    free = min((p.n_free for p in s.engine.manager.pools), default=0)
+                    cli.log("debug", f"step={number} tokens={sum(n for _, n, _ in plan.entries)} decoded={decoded} "
+                                     f"portions=[{portions}] preempted={len(plan.preempted)} waiting={len(sch.waiting)} "
+                                     f"free_pages={free}")
+                sch.on_step = on_step
             return sch
         s.scheduler = watched
         try:

@@ -43,6 +43,8 @@ DEFS = (
     OptDef("kv-tokens", SIZE, SESSION, 0, help="ours: tokens the cache pools hold, 0 = ctx-max x max-seqs "
                                                 "within free memory"),
     OptDef("max-seqs", INT, SESSION, 64, 1, 4096, help="ours: most sequences decoded together"),
+    OptDef("window", INT, SESSION, None, 0, 1 << 30, help="ours: sliding window in tokens for the layers that config.json "
+                                                        "lets have one, instead of config.json's (0 = none)"),
 
     OptDef("op", STR, REQUEST, "generate", help="generate | bench | echo"),
     OptDef("model", STR, REQUEST, None, help="model folder (config.json + model.safetensors)"),

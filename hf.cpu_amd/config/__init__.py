@@ -14,9 +14,14 @@ def config_from_dict(obj, origin="config.json"):
     return config_cls.from_dict(obj, origin)
 
 
-def read_config(model_dir):
+def read_config(model_dir, overrides=None):
+    """The typed configuration of the folder's config.json; ``overrides`` replaces keys of the file
+    before they are read and checked (the command line's ``--window``)."""
     path = config_path(model_dir)
-    return config_from_dict(read_json_file(path), path)
+    obj = read_json_file(path)
+    if overrides:
+        obj = dict(obj, **overrides)
+    return config_from_dict(obj, path)
 
 
 __all__ = ["KeyReader", "Qwen2Config", "config_from_dict", "read_config", "read_json_file"]

@@ -111,6 +111,14 @@ int hfa_draw_rows(float* vals, const int* ids, int n_rows, int vocab, const floa
 int hfa_topk(const float* logits, int ld, int* ids, float* vals, float* stats, int n_rows, int vocab, int k,
              hipStream_t stream);
 
+// Random weights on the device: element e of the tensor with `key` by the counter-based rule that
+// weights/random_init.py states (the host's writer computes the same bits). dtype HFA_F32 or HFA_BF16
+// with rule 0 (N(0, std): scale = std / sqrt(8 (65536^2 - 1) / 12)) or 1 (1 + that); dtype 2 (int32)
+// with rule 2 (uniform below `bound`). The reference's one generator for model and oracle:
+// tools/mkmodel.pl:104-127.
+int hfa_random_fill(void* out, int dtype, size_t n, uint64_t key, float scale, int rule, int bound,
+                    hipStream_t stream);
+
 // The device's own peaks (the reference's read_sum and fma_burn, src/kern.h:17-23): a streaming read
 // of `bytes` (16-byte aligned; `sink` is 16 bytes that are almost never written) by `blocks_per_cu`
 // blocks of 256 threads a CU, a copy, and a burn of

@@ -385,3 +385,49 @@ extern "C" int hfa_scatter_i32(int* dst, const int* idx, const int* val, int n, 
     HFA_LAUNCH_CHECK("scatter_i32");
     return 0;
 }
+
+// ---- random weights -------------------------------------------------------------------------
+// Element e of the tensor with `key`: the two words mix(key + 2e), mix(key + 2e + 1) with the
+// finishing function of splitmix64; their eight 16-bit fields added up, less the mean 262140, as an
+// exact fp32 integer times `scale` (rule 0), 1 + that (rule 1), or the first word modulo `bound`
+// (rule 2). Integers and single fp32 operations only, so the host computes the same bits.
+#pragma clang fp contract(off)        // to the end of the file: 1 + x * scale is a product and a sum, each rounded
+__device__ __forceinline__ uint64_t mix64(uint64_t z) {
+    z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ull;
+    z = (z ^ (z >> 27)) * 0x94d049bb133111ebull;
+    return z ^ (z >> 31);
+}
+
+__global__ void random_fill_kernel(void* __restrict__ out, int dtype, size_t n, uint64_t key, float scale, int rule,
+                                   uint32_t bound) {
+    for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (size_t)gridDim.x * blockDim.x) {
+        const uint64_t a = mix64(key + 2 * (uint64_t)e);
+        if (rule == 2) {
+            reinterpret_cast<int*>(out)[e] = (int)(a % bound);
+            continue;
+        }
+        const uint64_t b = mix64(key + 2 * (uint64_t)e + 1);
+        int total = 0;
+#pragma unroll
+        for (int s = 0; s < 64; s += 16) total += (int)((a >> s) & 0xffff) + (int)((b >> s) & 0xffff);
+        float v = (float)(total - 262140) * scale;
+        if (rule == 1) v = 1.0f + v;
+        if (dtype == HFA_F32)
+            reinterpret_cast<float*>(out)[e] = v;
+        else
+            reinterpret_cast<uint16_t*>(out)[e] = bf16_bits(v);
+    }
+}
+
+extern "C" int hfa_random_fill(void* out, int dtype, size_t n, uint64_t key, float scale, int rule, int bound,
+                               hipStream_t stream) {
+    HFA_REQUIRE(out != nullptr && n > 0, "random_fill: nothing to fill");
+    HFA_REQUIRE(rule >= 0 && rule <= 2, "random_fill: unknown rule %d", rule);
+    HFA_REQUIRE(rule == 2 ? (dtype == 2 && bound > 0) : (dtype == HFA_F32 || dtype == HFA_BF16),
+                "random_fill: rule %d does not fit dtype %d (bound %d)", rule, dtype, bound);
+    size_t blocks = (n + 255) / 256;
+    if (blocks > 16384) blocks = 16384;
+    random_fill_kernel<<<(int)blocks, 256, 0, stream>>>(out, dtype, n, key, scale, rule, (uint32_t)bound);
+    HFA_LAUNCH_CHECK("random_fill");
+    return 0;
+}

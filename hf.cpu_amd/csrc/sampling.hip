@@ -512,23 +512,33 @@ extern "C" int hfa_order_rows(const float* logits, int ld, const int* rows, int*
 #define DRAW_THREADS 1024
 #define DRAW_PIECE 4096
 
+// From here to the end of the file no product is fused with a sum (the library is built with
+// -ffp-contract=fast-honor-pragmas): one bit of a probability can move a draw to another token.
+// The toolchain's own "round to nearest" operators are plain operators compiled outside this
+// pragma, which the compiler does join into fused multiply-adds; the ones below are compiled inside it.
+#pragma clang fp contract(off)
+__device__ __forceinline__ float mul_rn(float a, float b) { return a * b; }
+__device__ __forceinline__ float add_rn(float a, float b) { return a + b; }
+__device__ __forceinline__ float sub_rn(float a, float b) { return a - b; }
+__device__ __forceinline__ float div_rn(float a, float b) { return a / b; }
+
 __device__ __forceinline__ float ref_expf(float x) {
     if (x != x) return x;
     if (x > 88.3762626647949f) x = 88.3762626647949f;
     if (x < -87.3365478515625f) return 0.0f;
-    const float fx = floorf(__fadd_rn(__fmul_rn(x, 1.44269504088896341f), 0.5f));
+    const float fx = floorf(add_rn(mul_rn(x, 1.44269504088896341f), 0.5f));
     const int n = (int)fx;
-    x = __fsub_rn(x, __fmul_rn(fx, 0.693359375f));
-    x = __fsub_rn(x, __fmul_rn(fx, -2.12194440e-4f));
-    const float z = __fmul_rn(x, x);
+    x = sub_rn(x, mul_rn(fx, 0.693359375f));
+    x = sub_rn(x, mul_rn(fx, -2.12194440e-4f));
+    const float z = mul_rn(x, x);
     float y = 1.9875691500e-4f;
-    y = __fadd_rn(__fmul_rn(y, x), 1.3981999507e-3f);
-    y = __fadd_rn(__fmul_rn(y, x), 8.3334519073e-3f);
-    y = __fadd_rn(__fmul_rn(y, x), 4.1665795894e-2f);
-    y = __fadd_rn(__fmul_rn(y, x), 1.6666665459e-1f);
-    y = __fadd_rn(__fmul_rn(y, x), 5.0000001201e-1f);
-    y = __fadd_rn(__fadd_rn(__fmul_rn(y, z), x), 1.0f);
-    return __fmul_rn(y, __uint_as_float((uint32_t)(n + 127) << 23));
+    y = add_rn(mul_rn(y, x), 1.3981999507e-3f);
+    y = add_rn(mul_rn(y, x), 8.3334519073e-3f);
+    y = add_rn(mul_rn(y, x), 4.1665795894e-2f);
+    y = add_rn(mul_rn(y, x), 1.6666665459e-1f);
+    y = add_rn(mul_rn(y, x), 5.0000001201e-1f);
+    y = add_rn(add_rn(mul_rn(y, z), x), 1.0f);
+    return mul_rn(y, __uint_as_float((uint32_t)(n + 127) << 23));
 }
 
 // One thread's running sum of p[0 .. n) in order, started from `start`; stops after the first element
@@ -544,7 +554,7 @@ __device__ int draw_running(const float* __restrict__ p, int n, float start, flo
         __syncthreads();
         if (threadIdx.x == 0 && hit == n) {
             for (int i = 0; i < len; i++) {
-                sum = __fadd_rn(sum, piece[i]);
+                sum = add_rn(sum, piece[i]);
                 if (stop(sum)) { hit = c0 + i; break; }
             }
             shared2[0] = sum;
@@ -571,18 +581,18 @@ __global__ __launch_bounds__(DRAW_THREADS) void draw_rows_kernel(float* __restri
     const int m = cuts[row] < 1 ? 1 : cuts[row] > vocab ? vocab : cuts[row];      // candidates after the top-k cut
     const float l0 = p[0];
     __syncthreads();                                          // p[0] is read by all before it is overwritten
-    for (int i = tid; i < m; i += DRAW_THREADS) p[i] = ref_expf(__fdiv_rn(__fsub_rn(p[i], l0), temp));
+    for (int i = tid; i < m; i += DRAW_THREADS) p[i] = ref_expf(div_rn(sub_rn(p[i], l0), temp));
     __threadfence_block();
     draw_running(p, m, 0.0f, piece, shared2, [](float) { return false; });
     const float total = shared2[0];
     __syncthreads();
-    for (int i = tid; i < m; i += DRAW_THREADS) p[i] = __fdiv_rn(p[i], total);
+    for (int i = tid; i < m; i += DRAW_THREADS) p[i] = div_rn(p[i], total);
     if (tid == 0) first_below = m;
     __threadfence_block();
     __syncthreads();
     int kept = m;
     if (min_p > 0.0f) {                                       // the leading run with p >= min_p * p_0, at least one
-        const float least = __fmul_rn(min_p, p[0]);
+        const float least = mul_rn(min_p, p[0]);
         int mine = m;
         for (int i = tid; i < m; i += DRAW_THREADS)
             if (p[i] < least) { mine = i; break; }            // a thread's indices ascend: its first is its least
@@ -600,7 +610,7 @@ __global__ __launch_bounds__(DRAW_THREADS) void draw_rows_kernel(float* __restri
         sum = shared2[0];
     }
     __syncthreads();
-    const float r = __fmul_rn(u, sum);
+    const float r = mul_rn(u, sum);
     const int at = draw_running(p, kept, 0.0f, piece, shared2, [r](float s) { return r < s; });
     if (tid == 0) tokens[row] = id[at < kept ? at : kept - 1];
 }

@@ -100,6 +100,7 @@ class Scheduler:
         self.on_token = None          # callback(request, choice)
         self.on_finish = None         # callback(request)
         self.on_prefill = None        # callback(request)
+        self.on_step = None           # callback(step number, plan) before the step runs
 
     # ---- submission --------------------------------------------------------
     def submit(self, req, forks=()):
@@ -263,6 +264,8 @@ class Scheduler:
                 r.admitted_at = self._admissions
                 self._admissions += 1
                 self.running.append(r)
+        if self.on_step:
+            self.on_step(self.steps, plan)
         step_entries = [(r.req_id, r.tokens[r.n_fed:r.n_fed + n], [n - 1] if want else [])
                         for r, n, want in plan.entries]
         logits = self.engine.step(step_entries)

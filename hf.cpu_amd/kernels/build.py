@@ -19,7 +19,9 @@ CSRC = os.path.join(PKG, "csrc")
 LIB_NAME = "libhfamd.so"
 ARCH = "gfx950"
 # -packed-fp32-ops off: the compiler must not form packed fp32 instructions.
-FLAGS = ["--offload-arch=" + ARCH, "-O3", "-fPIC", "-std=c++17", "-ffp-contract=fast",
+# -ffp-contract=fast-honor-pragmas: products and sums are fused, except where a source says
+# `#pragma clang fp contract(off)` (the sampler's draw, the random weights: bits the host must match).
+FLAGS = ["--offload-arch=" + ARCH, "-O3", "-fPIC", "-std=c++17", "-ffp-contract=fast-honor-pragmas",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
 
 

@@ -27,6 +27,7 @@ _SIGNATURES = {
     "hfa_topk": [P, I, P, P, P, I, I, I, P],
     "hfa_order_rows": [P, I, P, P, P, I, I, P, c_size_t, P],
     "hfa_draw_rows": [P, P, I, I, P, P, P, P],
+    "hfa_random_fill": [P, I, c_size_t, ctypes.c_uint64, F, I, I, P],
     "hfa_probe_read": [P, c_size_t, P, I, P],
     "hfa_probe_copy": [P, P, c_size_t, P],
     "hfa_probe_mfma": [P, I, I, P, P],

@@ -65,8 +65,8 @@ class Model:
         return cls(plan_fn(config), config)
 
     @classmethod
-    def from_dir(cls, model_dir, dtype, ops):
-        model = cls.from_config(read_config(model_dir))
+    def from_dir(cls, model_dir, dtype, ops, overrides=None):
+        model = cls.from_config(read_config(model_dir, overrides))
         dt = compute_dtype(dtype)
         model._bind(load_tensors(model_dir, model.param_specs(), dt, ops.device), dt, ops)
         return model

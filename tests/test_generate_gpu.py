@@ -219,6 +219,31 @@ def test_command_line_generate(gpu, models):
     assert rc == 1 and "code=EIO" in out
 
 
+def test_command_line_window_override_and_step_log(gpu, models):
+    """``--window N`` replaces config.json's window for the layers that may have one (B: layers 1 and 2),
+    ``--window 0`` takes it away; the tokens are the plain implementation's for the configuration so
+    changed. ``--log-level debug`` says what every step held."""
+    import plain
+    prompt = helpers.random_requests(helpers.CONFIG_B, [60], seed=8)["r0"]
+    base = ["--stdin-mode", "none", "--model", models["B"], "--dtype", "float32", "--ctx-max", "128", "--page-size", "8",
+            "--max-seqs", "2", "--batch", "16", "--prompt-ids", " ".join(map(str, prompt)), "--temp", "0", "--max-tokens", "6"]
+    got = {}
+    for window in (None, 0, 9):
+        rc, out, err = run_cli(base + ([] if window is None else ["--window", str(window)]) + ["--log-level", "debug"])
+        assert rc == 0, err
+        got[window] = [int(e[1]["id"]) for e in events(out) if e[0] == "token"]
+        steps = [line for line in err.splitlines() if line.startswith("debug step=")]
+        assert len(steps) == 4 + 5 and "portions=[0:0+16]" in steps[0] and "decoded=1" in steps[-1], steps
+        cfg, w = plain.read_model(models["B"])
+        if window is not None:
+            cfg = dict(cfg, use_sliding_window=window > 0, sliding_window=window or None)
+        toks = list(prompt)
+        for _ in range(6):
+            toks.append(int(np.argmax(plain.forward(cfg, w, toks)[-1])))
+        assert got[window] == toks[len(prompt):], f"--window {window}"
+    assert got[None] != got[9] or got[None] != got[0]
+
+
 def test_command_line_profile(gpu, models):
     """``--profile`` adds the reference's two @profile events (docs/PROTOCOL.md:93): per stage the
     milliseconds by part of the forward pass, plus sampling; the tokens are the same as without."""

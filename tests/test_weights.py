@@ -120,6 +120,63 @@ def test_random_weights_folder(tmp_path):
     assert logits.shape == (3, 512) and np.isfinite(logits).all()
 
 
+def test_random_generator_is_the_stated_rule():
+    """The counter-based generator of the random weights, element by element against its statement
+    in plain integers (splitmix64's finishing function on key + 2e and key + 2e + 1, the eight 16-bit
+    fields added up, one fp32 product); pieces of a tensor equal the whole; the moments are a Gaussian's."""
+    from hf_cpu_amd.weights.random_init import random_values, tensor_key
+    M = (1 << 64) - 1
+
+    def mix(z):
+        z &= M
+        z = ((z ^ (z >> 30)) * 0xbf58476d1ce4e5b9) & M
+        z = ((z ^ (z >> 27)) * 0x94d049bb133111eb) & M
+        return z ^ (z >> 31)
+    key = tensor_key(7, 3)
+    assert key == mix(7 * 0x9e3779b97f4a7c15 + 3)
+    got = random_values(key, 50, "normal", 0.02)
+    scale = np.float32(0.02 / np.sqrt(8 * (65536.0 ** 2 - 1) / 12))
+    for e in (0, 1, 17, 49):
+        a, b = mix(key + 2 * e), mix(key + 2 * e + 1)
+        total = sum((w >> s) & 0xffff for w in (a, b) for s in (0, 16, 32, 48))
+        assert got[e] == np.float32(total - 262140) * scale
+    assert np.array_equal(random_values(key, 20, "normal", 0.02, first=30), got[30:])
+    assert np.array_equal(random_values(key, 50, "one_plus_normal", 0.02), np.float32(1.0) + got)
+    table = random_values(key, 1000, "table", 37)
+    assert table.dtype == np.int32 and table.min() >= 0 and table.max() < 37 and table[5] == mix(key + 10) % 37
+    big = random_values(tensor_key(0, 0), 400000, "normal", 1.0).astype(np.float64)
+    assert abs(big.mean()) < 0.01 and abs(big.std() - 1.0) < 0.01
+    assert abs(np.mean(big ** 4) - 3.0) < 0.2 and np.abs(big).max() < 4.9        # kurtosis 3 - 1.2 / 8
+    assert not np.array_equal(random_values(tensor_key(0, 1), 50, "normal", 0.02), random_values(tensor_key(1, 0), 50, "normal", 0.02))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+def test_random_weights_are_the_same_bits_from_the_file_and_on_the_device(gpu, tmp_path, dtype):
+    """``Model.from_random(config, seed)`` (weights made by a kernel) holds what ``Model.from_dir`` loads
+    from the folder that ``write_random_model(config, seed)`` wrote: one generator for both."""
+    import hf_cpu_amd
+    from hf_cpu_amd.kernels import Ops
+    from hf_cpu_amd.model import compute_dtype
+    cfg = config_from_dict(helpers.CONFIG_B)
+    d = write_random_model(str(tmp_path / "r"), cfg, seed=11, dtype=dtype)
+    ops = Ops(compute_dtype(dtype), gpu)
+    a = hf_cpu_amd.Model.from_dir(d, dtype, ops)
+    b = hf_cpu_amd.Model.from_random(cfg, 11, dtype, ops)
+    seen = 0
+    for la, lb in zip(a._all_parts(), b._all_parts()):
+        for name, ta in vars(la).items():
+            if isinstance(ta, torch.Tensor):
+                tb = getattr(lb, name)
+                assert ta.dtype == tb.dtype and torch.equal(ta, tb), f"{type(la).__name__}.{name}"
+                seen += 1
+    assert seen >= 3 * 6 + 3
+    c = hf_cpu_amd.Model.from_random(cfg, 12, dtype, ops)
+    assert not torch.equal(c.embedding.table if hasattr(c.embedding, "table") else next(
+        t for t in vars(c.embedding).values() if isinstance(t, torch.Tensor)), next(
+        t for t in vars(b.embedding).values() if isinstance(t, torch.Tensor)))
+
+
 def test_writer_round_trip(tmp_path):
     t = {"a": torch.arange(6, dtype=torch.float32).reshape(2, 3), "b": torch.tensor([1.5, -2.0]).bfloat16(),
          "c": torch.tensor([[1, 2], [3, 4]], dtype=torch.int32)}

@@ -517,3 +517,51 @@ def test_layer_sizes_of_the_family(gpu, tmp_path, member):
     worst = helpers.compare(helpers.run_trace_in_engine(engine, steps), want, 2e-2, f"{member} layer")
     print(f"{member}-sized layer: worst relative difference {worst:.2e}")
     assert not engine.manager.held
+
+
+def test_the_whole_7b_shape_in_bf16_against_fp32(gpu):
+    """All 28 layers of the 7B shape with random weights N(0, 0.02) made on the device (one generator, one
+    seed; the bf16 weights are the fp32 ones rounded): a prompt in two portions and four decoded tokens
+    through the true 32-bit engine, through the same with every tensor rounded to bf16 first, and through
+    the bf16 engine. The baseline's "bf16 plus fp32 check" at full depth. A random network of this depth
+    magnifies a rounding many times (each layer's output is roughly quadratic in its normalised input), so
+    the yardstick is measured in the same run: what rounding the weights alone does to the 32-bit engine's
+    logits. The bf16 engine rounds about as many activations per layer as there are weight matrices; it
+    must stay within three times that, and choose the same token wherever the 32-bit logits' two best
+    are further apart than the difference seen."""
+    import torch
+    import bench
+    import hf_cpu_amd
+    from hf_cpu_amd.engine import Engine
+    from hf_cpu_amd.kernels import Ops
+    cfg = hf_cpu_amd.config_from_dict(dict(bench.SHAPE_7B))
+    rng = np.random.default_rng(3)
+    toks = [int(t) for t in rng.integers(0, cfg.vocab_size, 100)]
+    rows = {}
+    for run, dtype in (("exact", "float32"), ("rounded", "float32"), ("bf16", "bfloat16")):
+        ops = Ops(torch.float32 if dtype == "float32" else torch.bfloat16, gpu)
+        model = hf_cpu_amd.Model.from_random(cfg, 0, dtype, ops)
+        if run == "rounded":
+            for part in model._all_parts():
+                for t in vars(part).values():
+                    if isinstance(t, torch.Tensor) and t.dtype == torch.float32:
+                        t.copy_(t.bfloat16().float())
+        engine = Engine(model, ops, page_tokens=16, max_tokens=128, max_seqs=1)
+        got = [engine.step([("a", toks[:70], [0, 69])]).float().cpu().numpy()]
+        got.append(engine.step([("a", toks[70:96], [25])]).float().cpu().numpy())
+        for t in toks[96:]:
+            got.append(engine.step([("a", [t], [0])]).float().cpu().numpy())
+        rows[run] = np.concatenate(got).astype(np.float64)
+        del engine, model, ops
+        torch.cuda.empty_cache()
+    scale = np.max(np.abs(rows["exact"]))
+    by_weights = float(np.max(np.abs(rows["rounded"] - rows["exact"])) / scale)
+    by_activations = float(np.max(np.abs(rows["bf16"] - rows["rounded"])) / scale)
+    print(f"7B shape, 28 layers, |diff| / max |logit| ({scale:.2f}): weights rounded {by_weights:.3e}, "
+          f"bf16 engine against that {by_activations:.3e}")
+    assert np.isfinite(rows["bf16"]).all() and 1e-3 < by_weights < 0.2
+    assert by_activations < 3 * by_weights
+    for i in range(rows["rounded"].shape[0]):
+        order = np.argsort(-rows["rounded"][i])
+        if rows["rounded"][i, order[0]] - rows["rounded"][i, order[1]] > 2 * by_activations * scale:
+            assert int(np.argmax(rows["bf16"][i])) == int(order[0]), f"row {i}"

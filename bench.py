@@ -259,9 +259,17 @@ def main():
             logits = eng.step([(r, prompt(), [PROMPT - 1])])
             last.append(int(ops.argmax(logits).cpu()[0]))
 
+        # The serving loop's way of decoding: a step takes its tokens from where the sampler left them on
+        # the device, and the host reads every step's tokens one step late, while the next step runs.
+        state = {"dev": torch.tensor(last, dtype=torch.int32, device=ops.device), "read": lambda: last}
+        fed_rows = {i: i for i in range(batch)}
+
         def one():
-            logits = eng.step([(r, [t], [0]) for r, t in zip(ids, last)])
-            last[:] = ops.argmax(logits).cpu().tolist()
+            logits = eng.step([(r, [0], [0]) for r in ids], fed=(state["dev"], fed_rows))
+            chosen = ops.argmax(logits)
+            later = s.sampler._to_host_later(chosen)     # the copy is enqueued behind the choice; it is read a step late
+            state["tokens"] = state["read"]()
+            state["dev"], state["read"] = chosen, later
         for _ in range(warmup):
             one()
         torch.cuda.synchronize()

@@ -78,6 +78,9 @@ int hfa_swiglu(const void* gate_up, void* out, int dtype, int n_tokens, int widt
 // dst[idx[i]] = val[i]
 int hfa_scatter_i32(int* dst, const int* idx, const int* val, int n, hipStream_t stream);
 
+// dst[dst_idx[i]] = src[src_idx[i]] (tokens sampled on the device go into the next step's inputs)
+int hfa_move_i32(int* dst, const int* dst_idx, const int* src, const int* src_idx, int n, hipStream_t stream);
+
 // out[r] = first index of the maximum of logits[r, :].  (src/sample.c:72-77)
 // `workspace` holds the candidates of the first of its two stages (n_rows * 64 * 8 bytes).
 int hfa_argmax(const float* logits, int ld, int* out, int n_rows, int vocab, void* workspace,

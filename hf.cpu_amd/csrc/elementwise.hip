@@ -386,6 +386,20 @@ extern "C" int hfa_scatter_i32(int* dst, const int* idx, const int* val, int n, 
     return 0;
 }
 
+// dst[dst_idx[i]] = src[src_idx[i]]: a step's tokens that were sampled on the device and never went to the host.
+__global__ void move_i32_kernel(int* __restrict__ dst, const int* __restrict__ dst_idx, const int* __restrict__ src,
+                                const int* __restrict__ src_idx, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) dst[dst_idx[i]] = src[src_idx[i]];
+}
+
+extern "C" int hfa_move_i32(int* dst, const int* dst_idx, const int* src, const int* src_idx, int n, hipStream_t stream) {
+    HFA_REQUIRE(n > 0 && dst && dst_idx && src && src_idx, "move_i32: nothing to move");
+    move_i32_kernel<<<(n + 255) / 256, 256, 0, stream>>>(dst, dst_idx, src, src_idx, n);
+    HFA_LAUNCH_CHECK("move_i32");
+    return 0;
+}
+
 // ---- random weights -------------------------------------------------------------------------
 // Element e of the tensor with `key`: the two words mix(key + 2e), mix(key + 2e + 1) with the
 // finishing function of splitmix64; their eight 16-bit fields added up, less the mean 262140, as an

@@ -108,31 +108,46 @@ class Engine:
             book[k] = book.get(k, 0.0) + v
 
     # ---- one step ------------------------------------------------------------
-    def step(self, entries):
+    def step(self, entries, fed=None):
         """``entries``: a list of Entry or (req_id, tokens, want). A request seen for the
         first time is admitted. Returns fp32 logits [R, vocab] on the device, rows in the
         order of the entries and of each entry's ``want``; the tensor is a view of a work
         buffer and is overwritten by the next step. On an error nothing is kept: lengths,
-        pages and admissions are as before the call."""
+        pages and admissions are as before the call.
+
+        ``fed``: ``(source, {entry index: row})``: the single token of each of these entries is
+        ``source[row]``, an int32 tensor on the device (what the sampler chose after the step before,
+        not yet read by the host); the token the entry itself names is ignored. The host can then
+        enqueue a step before it knows the tokens of the one before."""
         entries = [e if isinstance(e, Entry) else Entry(*e) for e in entries]
         if not entries:
             fail(EINVAL, "step: no entries")
+        fed_rows = {} if fed is None else dict(fed[1])
+        for i in fed_rows:
+            if not 0 <= i < len(entries) or len(entries[i].tokens) != 1:
+                fail(EINVAL, "step: a token taken from the device belongs to an entry with exactly one token")
+            entries[i] = Entry(entries[i].req_id, [0], entries[i].want)
+        if fed_rows and (fed[0].dtype != torch.int32 or not fed[0].is_contiguous()
+                         or not all(0 <= r < fed[0].numel() for r in fed_rows.values())):
+            fail(EINVAL, "step: tokens taken from the device come from a contiguous int32 tensor that holds their rows")
         if self._is_plain_decode(entries):
-            return self._decode_step(entries)
+            return self._decode_step(entries, fed, fed_rows)
         seen = set()
         for e in entries:
             if e.req_id in seen:
                 fail(EINVAL, f"step: request {e.req_id!r} appears twice")
             seen.add(e.req_id)
-            if len(e.tokens) == 0:
+            n = len(e.tokens)
+            if n == 0:
                 fail(EINVAL, f"step: request {e.req_id!r} brings no tokens")       # src/model.c:555
-            for t in e.tokens:
-                if not 0 <= int(t) < self.vocab_size:
-                    fail(EINVAL, f"step: token id {t} of request {e.req_id!r} is outside the "
-                                 f"vocabulary of {self.vocab_size}")                # src/model.c:568
-            for w in e.want:
-                if not 0 <= int(w) < len(e.tokens):
-                    fail(EINVAL, f"step: request {e.req_id!r} wants logits at place {w} of {len(e.tokens)} tokens")
+            toks = np.asarray(e.tokens, dtype=np.int64)
+            if toks.min() < 0 or toks.max() >= self.vocab_size:
+                bad = int(toks[(toks < 0) | (toks >= self.vocab_size)][0])
+                fail(EINVAL, f"step: token id {bad} of request {e.req_id!r} is outside the "
+                             f"vocabulary of {self.vocab_size}")                    # src/model.c:568
+            if len(e.want) and not all(0 <= int(w) < n for w in e.want):
+                w = next(int(w) for w in e.want if not 0 <= int(w) < n)
+                fail(EINVAL, f"step: request {e.req_id!r} wants logits at place {w} of {n} tokens")
         mgr = self.manager
         admitted, reserved = [], []
         try:
@@ -143,7 +158,7 @@ class Engine:
                     self.storage.clear_slot(h.slot)
                 mgr.reserve(e.req_id, len(e.tokens))
                 reserved.append(e.req_id)
-            step = self._inputs(entries)
+            step = self._inputs(entries, fed, fed_rows)
             logits = self.ops.scratch("logits", (max(step.n_logit_rows, 1), self.vocab_size), torch.float32)
             logits = logits[:step.n_logit_rows]
             self._run(step, logits)
@@ -171,7 +186,7 @@ class Engine:
         except TypeError:
             return False
 
-    def _decode_step(self, entries):
+    def _decode_step(self, entries, fed=None, fed_rows=None):
         """``step`` for entries that pass ``_is_plain_decode``: the same checks, books and arrays,
         built with one pass over the requests instead of several per request."""
         mgr = self.manager
@@ -221,9 +236,10 @@ class Engine:
             rows = np.arange(N, dtype=np.int32)
             q_start = np.arange(N + 1, dtype=np.int32)
             arrays = [tokens, lengths, slots, q_start, slots, seq_len, rows, np.zeros(1, np.int32)] + slot_maps
+            moves = (fed[0], as_i32(list(fed_rows)), as_i32(list(fed_rows.values()))) if fed_rows else None
             step = self._upload(arrays, N, N, N, 1, int(seq_len.max()),
                                 dict(tokens=tokens, positions=lengths, token_slot=slots, q_start=q_start,
-                                     seq_slot=slots, seq_len=seq_len, logit_rows=rows), short=(N, N, 1))
+                                     seq_slot=slots, seq_len=seq_len, logit_rows=rows), short=(N, N, 1), moves=moves)
             logits = self.ops.scratch("logits", (N, self.vocab_size), torch.float32)
             self._run(step, logits)
             logits = logits[:S]
@@ -274,8 +290,9 @@ class Engine:
         graph.replay()
         self.graph_replays += 1
 
-    def _inputs(self, entries):
+    def _inputs(self, entries, fed=None, fed_rows=None):
         mgr = self.manager
+        fed_dst, fed_src = [], []
         T = sum(len(e.tokens) for e in entries)
         S = len(entries)
         tokens = np.empty(T, np.int32)
@@ -299,6 +316,9 @@ class Engine:
             if n < few:
                 n_short, n_short_tokens, max_short = n_short + 1, n_short_tokens + n, max(max_short, n)
             tokens[at:at + n] = e.tokens
+            if fed_rows and i in fed_rows:
+                fed_dst.append(at)
+                fed_src.append(fed_rows[i])
             positions[at:at + n] = np.arange(h.length, h.length + n, dtype=np.int32)
             token_slot[at:at + n] = h.slot
             q_start[s + 1] = at + n
@@ -316,9 +336,10 @@ class Engine:
         return self._upload(arrays, T, S, len(rows), max_q, max_len,
                             dict(tokens=tokens, positions=positions, token_slot=token_slot, q_start=q_start,
                                  seq_slot=seq_slot, seq_len=seq_len, logit_rows=rows),
-                            short=(n_short, n_short_tokens, max_short))
+                            short=(n_short, n_short_tokens, max_short),
+                            moves=(fed[0], as_i32(fed_dst), as_i32(fed_src)) if fed_dst else None)
 
-    def _upload(self, arrays, T, S, R, max_q, max_len, host, short):
+    def _upload(self, arrays, T, S, R, max_q, max_len, host, short, moves=None):
         """Sends a step's arrays (tokens, positions, token_slot, q_start, seq_slot, seq_len,
         logit_rows, q_start_long, then one slot map per group) and the block-table entries appended
         since the last step; returns the StepInputs. ``short``: number of the leading requests with
@@ -333,6 +354,8 @@ class Engine:
             dirty.append(len(app))
             arrays.append(as_i32([slot * mgr.max_blocks + block for slot, block, _ in app]))
             arrays.append(as_i32([page for _, _, page in app]))
+        if moves is not None:                 # tokens that lie on the device: where they go, where they come from
+            arrays += [moves[1], moves[2]]
         views = self.staging.upload(arrays)
         step = StepInputs(T, S, R)
         (step.tokens, step.positions, step.token_slot, step.q_start, step.seq_slot, step.seq_len,
@@ -347,4 +370,6 @@ class Engine:
             if dirty[g]:
                 self.ops.scatter_i32(table.view(-1), idx, val)
             step.groups.append(GroupInputs(table, slot_map))
+        if moves is not None:
+            self.ops.move_i32(step.tokens, views[-2], moves[0], views[-1])
         return step

@@ -23,6 +23,14 @@ Each step:
     free again (so it is not thrown out again at once). A request that does not fit even
     alone fails with ERANGE.
 
+The host does not wait for a step's tokens before it enqueues the next step: where the sampler can
+leave the chosen tokens on the device (``sample_start``: all rows greedy, or all drawn from their best
+k), the next step takes them from there (``Engine.step(..., fed=...)``) and the host reads them
+while that step runs. What the host then learns one step late: an end-of-sequence token (the
+request ran one step more, whose row is dropped and whose cache goes back with the request).
+Steps in which a request is about to end by its length, a prompt's continuations are about to be
+forked, or pages are short wait for the tokens first, as do samplers without ``sample_start``.
+
 Several continuations of one prompt (``--n``, src/ops.c:808-825): the prompt is computed once;
 when its last portion is done the other continuations are forked from the first one's cache
 (whole pages shared), and each samples its own first token from the same logits with its own
@@ -69,10 +77,21 @@ class Request:
     admitted_at: int = -1                    # admission order, for the preemption choice
     forks: list = field(default_factory=list)     # continuations of the same prompt, forked when it is done
     last_ran: int = -1                       # the step that last held tokens of this request
+    pending: int = None                      # its next token is not read yet: row of the sample under way
 
     @property
     def unfed(self):
         return len(self.tokens) - self.n_fed
+
+
+PLACEHOLDER = -1         # in Request.tokens: a token that the device has and the host has not read yet
+
+
+@dataclass
+class Inflight:
+    """A step's sampling under way: the requests of its rows and the sampler's handle."""
+    sampled: list
+    started: object
 
 
 @dataclass
@@ -83,7 +102,8 @@ class StepPlan:
 
 
 class Scheduler:
-    def __init__(self, engine, sampler, token_budget=64, max_seqs=None, ctx_max=None, clock=time.monotonic):
+    def __init__(self, engine, sampler, token_budget=64, max_seqs=None, ctx_max=None, clock=time.monotonic,
+                 pipeline=True):
         self.engine, self.sampler = engine, sampler
         self.manager = engine.manager
         self.token_budget = int(token_budget)                          # --batch, src/opts.c:44
@@ -101,6 +121,9 @@ class Scheduler:
         self.on_finish = None         # callback(request)
         self.on_prefill = None        # callback(request)
         self.on_step = None           # callback(step number, plan) before the step runs
+        self.pipeline = bool(pipeline) and hasattr(sampler, "sample_start")
+        self._inflight = None         # the step whose tokens the host has not read yet
+        self.steps_ahead = 0          # steps that were enqueued before the tokens of the one before were read
 
     # ---- submission --------------------------------------------------------
     def submit(self, req, forks=()):
@@ -135,7 +158,7 @@ class Scheduler:
 
     @property
     def idle(self):
-        return not self.waiting and not self.running
+        return not self.waiting and not self.running and self._inflight is None
 
     # ---- planning ------------------------------------------------------------
     def plan(self):
@@ -226,6 +249,9 @@ class Scheduler:
             self.running.remove(r)
             if self.engine.has(r.req_id):
                 self.engine.release(r.req_id)
+        elif r.status == WAITING and r in self.waiting:
+            self.waiting.remove(r)
+        r.pending = None
         r.status, r.stop, r.error, r.t_done = FINISHED, stop, error, self.clock()
         self.finished.append(r)
         if self.on_finish:
@@ -246,16 +272,23 @@ class Scheduler:
         for r in polled:                                                        # src/ops.c:790, 829
             expired = r.timeout > 0 and now - r.t_submit > r.timeout
             if r.cancel or expired:
-                if r.status == WAITING:
-                    self.waiting.remove(r)
-                if r.t_first is None:       # still in its prompt: an error, as in the reference
+                if r.t_first is None and r.pending is None:     # still in its prompt: an error, as in the reference
                     self._finish(r, error=EngineError(ECANCEL, "cancelled" if r.cancel else "timeout during prefill"))
                 else:
                     self._finish(r, stop="cancel" if r.cancel else "timeout")
+        if self._inflight is not None:
+            # Tokens are read before the plan where the plan turns on them: a request that is about to end
+            # by its length holds pages until its last token is booked; short pages may be freed by an
+            # end-of-sequence token that the host has not seen.
+            decoders = [r for r in self.running if r.unfed == 1 and r.n_fed > 0][:self.token_budget]
+            if not self.running or any(r.unfed == 0 for r in self.running) \
+                    or not self.manager.can_reserve([(r.req_id, 1) for r in decoders]):
+                self._land()
         if self.idle:
             return None
         plan = self.plan()
         if not plan.entries:
+            self._land()
             return plan
         for r, _, _ in plan.entries:
             if r.status == WAITING:
@@ -268,25 +301,57 @@ class Scheduler:
             self.on_step(self.steps, plan)
         step_entries = [(r.req_id, r.tokens[r.n_fed:r.n_fed + n], [n - 1] if want else [])
                         for r, n, want in plan.entries]
-        logits = self.engine.step(step_entries)
+        fed = None
+        if self._inflight is not None:
+            rows = {i: r.pending for i, (r, n, _) in enumerate(plan.entries) if r.pending is not None}
+            if rows:
+                fed = (self._inflight.started.device_tokens, rows)
+                self.steps_ahead += 1
+        logits = self.engine.step(step_entries, fed=fed) if fed else self.engine.step(step_entries)
         self.steps += 1
         sampled = [r for r, n, want in plan.entries if want]
         for r, n, _ in plan.entries:
             r.n_fed += n
             r.last_ran = self.steps
+        self._land()                  # the step before: its tokens are read while this one runs
         if sampled:
             t0 = time.perf_counter()
-            choices = self.sampler.sample(logits, [(r.params, r.rng, r.logprobs) for r in sampled])
+            wants = [(r.params, r.rng, r.logprobs) for r in sampled]
+            ahead = self.pipeline and not any(r.forks and r.t_first is None for r in sampled)
+            started = self.sampler.sample_start(logits, wants) if ahead else None
+            if started is not None and started.device_tokens is not None:
+                self._inflight = Inflight(sampled, started)
+                for i, r in enumerate(sampled):
+                    # a request that goes on decoding gets its next token's place now; one that this token
+                    # ends (by its length) or that has ended meanwhile only has the token booked later
+                    if r.status == RUNNING and len(r.generated) + 1 < r.n_cap:
+                        r.tokens.append(PLACEHOLDER)
+                        r.pending = i
+            else:
+                choices = started.finish() if started is not None else self.sampler.sample(logits, wants)
+                for i, (r, ch) in enumerate(zip(sampled, choices)):
+                    if r.status != RUNNING:
+                        continue              # ended by a token of the step before, which the host has just read
+                    forked = self._fork(r, logits[i:i + 1]) if r.forks and r.t_first is None else []
+                    self._accept(r, ch)
+                    for c, cch in forked:
+                        self._accept(c, cch)
             book = getattr(self.engine, "profile", None)
             if book is not None:               # sampling is timed on the host, as in src/ops.c:845-847
                 stage = book["prefill" if any(n > 1 for _, n, _ in plan.entries) else "decode"]
                 stage["sample"] = stage.get("sample", 0.0) + (time.perf_counter() - t0) * 1e3
-            for i, (r, ch) in enumerate(zip(sampled, choices)):
-                forked = self._fork(r, logits[i:i + 1]) if r.forks and r.t_first is None else []
-                self._accept(r, ch)
-                for c, cch in forked:
-                    self._accept(c, cch)
         return plan
+
+    def _land(self):
+        """Reads the tokens of the step whose sampling is under way and books them."""
+        flight, self._inflight = self._inflight, None
+        if flight is None:
+            return
+        choices = flight.started.finish()
+        for i, (r, ch) in enumerate(zip(flight.sampled, choices)):
+            if r.status == FINISHED:
+                continue                      # cancelled, or ended while this token was on its way
+            self._accept(r, ch, placed=r.pending == i)
 
     def _fork(self, r, row):
         """``r``'s prompt is done: its other continuations take its cache and draw their first
@@ -310,12 +375,17 @@ class Scheduler:
             out.append((c, self.sampler.sample(row, [(c.params, c.rng, c.logprobs)])[0]))
         return out
 
-    def _accept(self, r, ch):
+    def _accept(self, r, ch, placed=False):
+        """Books a sampled token. ``placed``: the token already has its place at the end of ``r.tokens``
+        (and may have been fed from the device); the place is filled, or dropped with the request."""
+        r.pending = None
         if r.t_first is None:
             r.t_first = self.clock()
             if self.on_prefill:
                 self.on_prefill(r)
         if ch.token in r.eos_ids:                                              # src/ops.c:849
+            if placed:
+                r.tokens.pop()
             return self._finish(r, stop="eos")
         r.generated.append(ch.token)
         r.choices.append(ch)
@@ -323,7 +393,10 @@ class Scheduler:
             self.on_token(r, ch)
         if len(r.generated) >= r.n_cap:                                        # src/ops.c:881, 758
             return self._finish(r, stop="length" if r.n_cap == r.max_tokens else "ctx")
-        r.tokens.append(ch.token)
+        if placed:
+            r.tokens[-1] = ch.token
+        else:
+            r.tokens.append(ch.token)
 
     def run(self):
         """Steps until every submitted request is finished; returns them in finishing order."""

@@ -22,6 +22,7 @@ _SIGNATURES = {
     "hfa_paged_attention": [P, I, I, P, P, I, P, I, P, P, P, I, I, I, P, I, I, I, I, I, I, I, F, P, c_size_t, I, P],
     "hfa_swiglu": [P, P, I, I, I, P],
     "hfa_scatter_i32": [P, P, P, I, P],
+    "hfa_move_i32": [P, P, P, P, I, P],
     "hfa_argmax": [P, I, P, I, I, P, c_size_t, P],
     "hfa_argmax_static": [P, I, P, I, I, P],
     "hfa_topk": [P, I, P, P, P, I, I, I, P],

@@ -360,6 +360,15 @@ class Ops:
             self._check(self.lib.hfa_scatter_i32(_ints(dst, "scatter dst"), _ints(idx, "scatter idx"),
                                                  _ints(val, "scatter val", n), n, self._stream()))
 
+    def move_i32(self, dst, dst_idx, src, src_idx):
+        """dst[dst_idx[i]] = src[src_idx[i]] for int32 tensors on the device."""
+        n = dst_idx.numel()
+        if n:
+            if src_idx.numel() != n:
+                fail(EINVAL, "move_i32: as many places to read as to write")
+            self._check(self.lib.hfa_move_i32(_ints(dst, "move dst"), _ints(dst_idx, "move dst_idx"), _ints(src, "move src"),
+                                              _ints(src_idx, "move src_idx", n), n, self._stream()))
+
     def argmax(self, logits, out=None):
         self.settle()
         R, V = logits.shape

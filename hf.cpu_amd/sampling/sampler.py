@@ -54,20 +54,82 @@ class Choice:
     top: list = None               # [(id, logprob), ...] best first, if asked for
 
 
+class Started:
+    """A step's sampling under way (``Sampler.sample_start``)."""
+
+    def __init__(self, device_tokens, choices, read=None):
+        self.device_tokens, self._choices, self._read = device_tokens, choices, read
+
+    def finish(self):
+        if self._choices is None:
+            self._choices = self._read()
+        return self._choices
+
+
 class Sampler:
     """Samples one token per row of a step's logits. ``wants[i]`` = (params, rng, n_logprobs)."""
 
     def __init__(self, ops):
         self.ops = ops
+        self._landing = []            # pinned host buffers that chosen tokens are copied to, used in turn
+        self._turn = 0
 
-    def _draw(self, ids, vals, numbers, cuts):
+    def _to_host_later(self, tokens):
+        """Enqueues the copy of ``tokens`` (int32 on the device) to pinned host memory right behind the
+        kernel that writes them, and returns a function that waits for that copy alone and gives the
+        numbers: a plain read would wait for everything enqueued since, the next step included."""
+        n = tokens.numel()
+        if len(self._landing) < 4:
+            self._landing.append(memory.empty(max(n, 256), torch.int32, None, "pinned buffer for chosen tokens", pin=True))
+        self._turn = (self._turn + 1) % len(self._landing)
+        if self._landing[self._turn].numel() < n:
+            self._landing[self._turn] = memory.empty(2 * n, torch.int32, None, "pinned buffer for chosen tokens", pin=True)
+        host = self._landing[self._turn][:n]
+        host.copy_(tokens, non_blocking=True)
+        done = torch.cuda.Event()
+        done.record()
+
+        def read():
+            done.synchronize()
+            return host.numpy().copy()
+        return read
+
+    def _draw(self, ids, vals, numbers, cuts, on_device=False):
         """The device's draw for rows of candidates in order; the rows' numbers and cuts travel as one copy."""
         n = len(cuts)
         both = np.empty(5 * n, dtype=f32)
         both[:4 * n] = numbers.reshape(-1)
         both[4 * n:].view(np.int32)[:] = cuts
         sent = memory.to_device(torch.from_numpy(both), vals.device, "the draws' numbers")
-        return self.ops.draw_rows(ids, vals, sent[:4 * n].view(n, 4), sent[4 * n:].view(torch.int32)).cpu().numpy()
+        drawn = self.ops.draw_rows(ids, vals, sent[:4 * n].view(n, 4), sent[4 * n:].view(torch.int32))
+        return drawn if on_device else drawn.cpu().numpy()
+
+    def sample_start(self, logits, wants):
+        """Begins the sampling of a step's rows and returns a ``Started``: ``device_tokens`` is the int32
+        tensor of the chosen tokens on the device if they can be had without the host (all rows greedy, or
+        all rows drawn from their best k, none asking for log-probabilities), else None; ``finish()``
+        returns the list of Choice (and waits for the device). Between the two the caller may enqueue
+        the next step with ``device_tokens`` as its input: ``logits`` is not read after this call returns
+        unless ``device_tokens`` is None, in which case everything has been computed already. Each
+        request's generator moves on here, by one draw, as in ``sample``."""
+        R, V = logits.shape
+        if R != len(wants):
+            fail(EINVAL, f"sampler: {R} rows of logits for {len(wants)} requests")
+        if any(n_lp for _, _, n_lp in wants):
+            return Started(None, self.sample(logits, wants))
+        if all(p.greedy for p, _, _ in wants):
+            arg = self.ops.argmax(logits)
+            read = self._to_host_later(arg)
+            return Started(arg, None, lambda: [Choice(int(t)) for t in read()])
+        if all(not p.greedy and 0 < p.top_k <= TOPK_KERNEL_MAX and p.top_k < V for p, _, _ in wants):
+            k = max(p.top_k for p, _, _ in wants)
+            ids, vals, _ = self.ops.topk(logits, k, want_stats=False)
+            numbers = np.array([(p.temp, p.top_p, p.min_p, rng.uniform()) for p, rng, _ in wants], dtype=f32)
+            cuts = np.array([p.top_k for p, _, _ in wants], dtype=np.int32)
+            drawn = self._draw(ids, vals, numbers, cuts, on_device=True)
+            read = self._to_host_later(drawn)
+            return Started(drawn, None, lambda: [Choice(int(t)) for t in read()])
+        return Started(None, self.sample(logits, wants))
 
     def sample(self, logits, wants):
         R = logits.shape[0]

@@ -16,6 +16,7 @@ class FakeEngine:
         self.manager = CacheManager([PagedKV(4, 4, 0), PagedKV(4, 4, window)], page, n_pages, slots, ctx)
         self.vocab_size = vocab
         self.log = []
+        self.fed_steps = 0
 
     def has(self, r):
         return r in self.manager.held
@@ -27,8 +28,14 @@ class FakeEngine:
         self.manager.fork(src, new)
         self.log.append([("fork", src, new)])
 
-    def step(self, entries):
+    def step(self, entries, fed=None):
         m = self.manager
+        if fed is not None:
+            self.fed_steps += 1
+            assert all(len(entries[i][1]) == 1 for i in fed[1])
+        for r, toks, want in entries:
+            if fed is None or entries.index((r, toks, want)) not in fed[1]:
+                assert all(t >= 0 for t in toks), "a token that was never read went to the engine as if known"
         for r, toks, want in entries:
             if r not in m.held:
                 m.admit(r)
@@ -308,3 +315,54 @@ def test_more_decoding_requests_than_the_token_budget_take_turns():
     sch2.token_budget = 2
     sch2.run()
     assert all(r.error is None and len(r.generated) == 3 for r in rs) and sum(r.preemptions for r in rs) == 0
+
+
+class AheadSampler(ScriptSampler):
+    """The script sampler with the interface that leaves tokens "on the device": the choices exist at
+    once, but the scheduler may only look at them through ``finish``."""
+
+    def sample_start(self, logits, wants):
+        choices = self.sample(logits, wants)
+
+        class Started:
+            device_tokens = object()
+
+            def finish(self):
+                return choices
+        return Started()
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_steps_enqueued_ahead_give_what_steps_in_turn_give(seed):
+    """Random workloads (prompt lengths, caps, end-of-sequence tokens at scripted places, a pool that is
+    too small, a budget below the number of decoders) served with the next step enqueued before the
+    last one's tokens are read, and served in turn: every request ends with the same tokens and the
+    same reason, nothing stays held, and steps did run ahead."""
+    import random
+    rnd = random.Random(seed)
+    n_req = rnd.randint(3, 9)
+    spec = []
+    for i in range(n_req):
+        n_prompt, cap = rnd.randint(1, 14), rnd.randint(1, 12)
+        script = [10 + j for j in range(cap)]
+        if rnd.random() < 0.5:
+            script[rnd.randrange(cap)] = 99                     # the end-of-sequence token somewhere
+        spec.append((f"r{i}", list(range(1, n_prompt + 1)), cap, script))
+    kw = dict(n_pages=rnd.choice([6, 9, 40]), page=4, slots=rnd.choice([2, 4]), ctx=48)
+    budget = rnd.choice([2, 5, 16])
+    outcomes = []
+    for ahead in (False, True):
+        eng = FakeEngine(**kw)
+        sampler = (AheadSampler if ahead else ScriptSampler)({name: script for name, _, _, script in spec})
+        sch = Scheduler(eng, sampler, token_budget=budget)
+        reqs = [sch.submit(Request(name, prompt, greedy(), max_tokens=cap, eos_ids=(99,))) for name, prompt, cap, _ in spec]
+        sch.run()
+        eng.manager.check()
+        assert not eng.manager.held and sch.idle
+        outcomes.append([(r.req_id, r.generated, r.stop, r.error.code if r.error else None) for r in reqs])
+        if ahead:
+            assert sch.steps_ahead == eng.fed_steps
+            assert all(t != -1 for r in reqs for t in r.tokens)
+            ran_ahead = sch.steps_ahead
+    assert outcomes[0] == outcomes[1]
+    assert ran_ahead > 0 or all(len(g) <= 1 for _, g, _, _ in outcomes[0])

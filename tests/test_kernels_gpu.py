@@ -742,3 +742,35 @@ def test_probes_of_the_device_peaks(ops16):
     assert 1000 < p["hbm_copy_GBps"] and 1000 < p["hbm_read_GBps"] < 8000
     assert 200 < p["mfma_bf16_TFLOPs"] <= p["mfma_bf16_zero_TFLOPs"] * 1.05 < 2700
     assert 0.5 < p["grid_barrier_us"] < 50
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 4608, 3584), (8, 3584, 18944), (3, 2016, 896), (9, 37888, 3584), (16, 1000, 1024),
+                                   (17, 4608, 3584), (32, 3584, 3584), (8, 152064, 3584), (5, 33, 8192), (32, 40, 16384)])
+def test_products_of_few_rows_streamed_wave_by_wave(ops16, M, N, K):
+    """The product for up to 32 rows in which every wave streams a run of the weights by itself (gemm_wave.hip),
+    against a float64 product of the same bf16 operands: one to 32 rows (one, two and four requests for A a
+    unit), widths that are no multiple of the 32-column tiles (the last tile repeats its last row), runs of
+    a few units and of hundreds, results stored, accumulated and left for the next kernel; and the same bits
+    twice (no wave's sum depends on another's timing)."""
+    torch.manual_seed(M + N)
+    a = (torch.randn((M, K), device="cuda") * 0.5).bfloat16()
+    w = (torch.randn((N, K), device="cuda") / K ** 0.5).bfloat16()
+    bias = torch.randn((N,), device="cuda")
+    want = a.double() @ w.double().T
+    out = torch.empty((M, N), device="cuda")
+    ops16.gemm(a, w, out, bias=bias)
+    err = ((out.double() - (want + bias.double())).abs().max() / want.abs().max()).item()
+    assert err < 1e-5, f"stored: {err:.3e}"
+    again = torch.empty_like(out)
+    ops16.gemm(a, w, again, bias=bias)
+    assert torch.equal(out, again)
+    x = torch.randn((M, N), device="cuda")
+    x0 = x.clone()
+    ops16.gemm(a, w, x, accumulate=True, defer=True)            # left as planes; settle adds them up
+    ops16.settle()
+    err = ((x.double() - (x0.double() + want)).abs().max() / want.abs().max()).item()
+    assert err < 1e-5, f"accumulated: {err:.3e}"
+    o16 = torch.empty((M, N), device="cuda", dtype=torch.bfloat16)
+    ops16.gemm(a, w, o16)
+    err = ((o16.double() - want).abs().max() / want.abs().max()).item()
+    assert err < 1e-2, f"bf16 output: {err:.3e}"

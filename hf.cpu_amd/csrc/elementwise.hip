@@ -41,6 +41,10 @@ extern "C" int hfa_embed(const void* table, int table_dtype, const int* tokens, 
     return 0;
 }
 
+// Planes of partial sums are fetched this many at a time (all of a batch asked for before the first is added).
+// The products of few rows leave about twenty planes; batches of 12 and of 24 changed nothing in a step's time.
+#define PLANE_BATCH 8
+
 // ---- RMS norm ---------------------------------------------------------------------------
 // One block per output row. The sum of squares is taken in a fixed order (each thread over
 // its strided elements, then waves, then the block), so a row's result does not depend on
@@ -71,15 +75,15 @@ __global__ __launch_bounds__(1024) void rmsnorm_kernel(float* __restrict__ x, co
             float4 v = *reinterpret_cast<const float4*>(src + i);
             if (splits > 0) {
                 // loads in batches of 8 that do not wait for one another, added in ascending order
-                for (int s0 = 0; s0 < splits; s0 += 8) {
-                    float4 p[8];
+                for (int s0 = 0; s0 < splits; s0 += PLANE_BATCH) {
+                    float4 p[PLANE_BATCH];
 #pragma unroll
-                    for (int u = 0; u < 8; u++)
+                    for (int u = 0; u < PLANE_BATCH; u++)
                         p[u] = s0 + u < splits
                                    ? *reinterpret_cast<const float4*>(partial + ((size_t)(s0 + u) * n_rows + xr) * width + i)
                                    : make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
-                    for (int u = 0; u < 8; u++) { v.x += p[u].x; v.y += p[u].y; v.z += p[u].z; v.w += p[u].w; }
+                    for (int u = 0; u < PLANE_BATCH; u++) { v.x += p[u].x; v.y += p[u].y; v.z += p[u].z; v.w += p[u].w; }
                 }
                 if (pbias) {
                     const float4 b = *reinterpret_cast<const float4*>(pbias + i);
@@ -168,12 +172,12 @@ struct QkvSource {
     __device__ __forceinline__ float at(int c) const {
         if (splits == 0) return to_f32(row[c]);
         float v = 0.f;
-        for (int s0 = 0; s0 < splits; s0 += 8) {           // batches of loads that do not wait for one another
-            float p[8];
+        for (int s0 = 0; s0 < splits; s0 += PLANE_BATCH) {           // batches of loads that do not wait for one another
+            float p[PLANE_BATCH];
 #pragma unroll
-            for (int u = 0; u < 8; u++) p[u] = s0 + u < splits ? partial[(s0 + u) * split_stride + c] : 0.f;
+            for (int u = 0; u < PLANE_BATCH; u++) p[u] = s0 + u < splits ? partial[(s0 + u) * split_stride + c] : 0.f;
 #pragma unroll
-            for (int u = 0; u < 8; u++) v += p[u];
+            for (int u = 0; u < PLANE_BATCH; u++) v += p[u];
         }
         return bias ? v + bias[c] : v;
     }

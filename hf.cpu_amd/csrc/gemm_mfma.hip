@@ -17,8 +17,8 @@
 // bias and the output mode. Nothing is accumulated with atomics: results are reproducible.
 //
 // Which kernel takes which shape (gemm_mfma_launch, at the end of this file):
-//   M <= 32          gemm_wave_kernel (gemm_wave.hip) if K is a multiple of 64 and there are as many units as waves;
-//                    else gemm_mfma_kernel, tiles of 32 x 128, K split, two register sets of loads in flight
+//   M <= 8           gemm_wave_kernel (gemm_wave.hip) if K is a multiple of 64 and there are as many units as waves; else as
+//   M <= 32          gemm_mfma_kernel, tiles of 32 x 128, K split, two register sets of loads in flight
 //   M in 33 .. 128   gemm_stream_kernel (gemm_stream.hip) if N is a multiple of 128 and K of 64, the output
 //                    has fewer than 512 tiles and a block gets 16 units or more; else gemm_mfma_kernel
 //                    with tiles of 64 x 128 or 128 x 128
@@ -627,7 +627,7 @@ int gemm_mfma_launch(const GemmArgs& g, void* workspace, size_t workspace_bytes,
         hfa_set_error("gemm: the gate/up epilogue needs N a multiple of 64, no bias and a bf16 output");
         return 1;
     }
-    if (g.M <= 32) {                         // few rows: every wave streams its own run of the weights
+    if (g.M <= 8) {                          // very few rows: every wave streams its own run of the weights
         const int slots = gemm_wave_slots(g, workspace ? workspace_bytes : 0);
         if (slots > 0) {
             const int rc = gemm_wave_launch(g, workspace, slots);

@@ -1,4 +1,4 @@
-// bf16 matrix product for up to 32 rows (decode), bound by the speed at which the weights stream in:
+// bf16 matrix product for up to 8 rows (decode), bound by the speed at which the weights stream in:
 // out[m, n] = sum_k a[m, k] * w[n, k], left as partial sums in a workspace.
 //
 // Every wave streams by itself. The work is the list of (tile of 32 output columns, 64 columns of K) units in
@@ -6,7 +6,7 @@
 // none of which waits for another. A wave has a ring of its own in LDS, filled by direct loads
 // (global_load_lds_dwordx4: 64 lanes x 16 bytes = 8 rows of 128 bytes a request; see gemm_mfma.hip for the
 // swizzled layout and the reason for the inline assembly): a unit is four requests for its 32 rows of W and one
-// to four for the rows of A (8, 16 or 32), requested R units ahead. There is no barrier and no other traffic
+// for the 8 rows of A, requested R units ahead. There is no barrier and no other traffic
 // between the waves of a block: the only wait is the wave's own, for its oldest unit.
 //
 // A column tile's K range is shared by the waves whose runs touch it. The workspace holds `slots` planes of
@@ -17,7 +17,9 @@
 //
 // Against the product that stages tiles of 32 x 128 through LDS shared by four waves with a barrier a step
 // (gemm_mfma_kernel), at 8 rows on the 7B shape: gate+up 51 against 56 us, down 24.5 against 30, q/k/v 9.5
-// against 11.8, o 8.4 against 10.1.
+// against 11.8, o 8.4 against 10.1. With 16 and 32 rows of A in the ring (two and four requests a unit, which the
+// template still allows) fewer bytes of W are on their way for the same LDS, and a step was slower than with the
+// tiled kernel (4.56 against 4.49 ms at 16 rows, 5.53 against 5.07 at 32): those rows stay there.
 #include "common.h"
 #include "gemm_internal.h"
 
@@ -161,7 +163,7 @@ static int wave_cu_count() {
 
 // The number of workspace planes a product of this shape needs, or 0 if this kernel does not take it.
 int gemm_wave_slots(const GemmArgs& g, size_t workspace_bytes) {
-    if (g.M > 32 || g.K % 64 != 0 || g.lda >= (1 << 22) || g.ldw >= (1 << 22) || g.N < 32) return 0;
+    if (g.M > 8 || g.K % 64 != 0 || g.lda >= (1 << 22) || g.ldw >= (1 << 22) || g.N < 32) return 0;
     const long long nk = g.K / 64, tiles = (g.N + 31) / 32, U = tiles * nk;
     const int G = wave_cu_count() * WAVES;
     if (U < G) return 0;                                     // fewer units than waves: the tiled kernel's splits do as well
@@ -191,8 +193,4 @@ static int launch_wave(const GemmArgs& g, float* partial, int slots) {
     return 0;
 }
 
-int gemm_wave_launch(const GemmArgs& g, void* workspace, int slots) {
-    if (g.M <= 8) return launch_wave<1, 3>(g, (float*)workspace, slots);
-    if (g.M <= 16) return launch_wave<2, 3>(g, (float*)workspace, slots);
-    return launch_wave<4, 2>(g, (float*)workspace, slots);
-}
+int gemm_wave_launch(const GemmArgs& g, void* workspace, int slots) { return launch_wave<1, 3>(g, (float*)workspace, slots); }

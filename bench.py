@@ -175,6 +175,9 @@ def main():
     ap.add_argument("--prefill-reps", type=int, default=3)
     ap.add_argument("--only", choices=["prefill", "decode"], default=None,
                     help="run one phase only and print a short line (for profiling a phase by itself)")
+    ap.add_argument("--context", type=int, default=PROMPT,
+                    help="with --only decode: tokens every sequence holds before the timed steps (prefilled in portions "
+                         "of 2,048); the default run's is 2,048")
     ap.add_argument("--no-peaks", action="store_true", help="skip the probes of the device's own peaks")
     ap.add_argument("--no-kernels", action="store_true", help="skip the timing by part")
     ap.add_argument("--workload", choices=["7b", "0.5b", "32b"], default="7b",
@@ -189,6 +192,9 @@ def main():
         return 2
     if args.workload != "7b":
         return serve_workload(args.workload, args.dtype, args.temp, args.budget)
+    if args.context != PROMPT and args.only != "decode":
+        print("bench.py: --context goes with --only decode (the default measurement has 2,048-token prompts)")
+        return 2
     if args.steps + args.warmup > NEW:
         print(f"bench.py: --steps + --warmup must not exceed the {NEW} new tokens of the workload")
         return 2
@@ -207,8 +213,8 @@ def main():
     elem = 2 if short == "bf16" else 4
     biggest = max(args.batch, 1 if args.no_points else 64)
     t_load = time.perf_counter()
-    s = S.Session(cfg, dtype=args.dtype, ctx_max=PROMPT + NEW, batch=PROMPT, page_size=PAGE, max_seqs=biggest,
-                  kv_tokens=biggest * (PROMPT + NEW), seed=0)
+    s = S.Session(cfg, dtype=args.dtype, ctx_max=args.context + NEW, batch=PROMPT, page_size=PAGE, max_seqs=biggest,
+                  kv_tokens=biggest * (args.context + NEW), seed=0)
     eng, ops = s.engine, s.ops
     torch.cuda.synchronize()
     print(f"[bench] weights and cache ready in {time.perf_counter() - t_load:.1f} s", file=sys.stderr, flush=True)
@@ -256,7 +262,9 @@ def main():
         ids = [("d", i) for i in range(batch)]
         last = []
         for r in ids:
-            logits = eng.step([(r, prompt(), [PROMPT - 1])])
+            for at in range(0, args.context, PROMPT):            # the prompt in portions of 2,048 tokens
+                n = min(PROMPT, args.context - at)
+                logits = eng.step([(r, prompt()[:n], [n - 1] if at + n == args.context else [])])
             last.append(int(ops.argmax(logits).cpu()[0]))
 
         # The serving loop's way of decoding: a step takes its tokens from where the sampler left them on
@@ -290,7 +298,9 @@ def main():
     value = args.batch * args.steps / dt
     print(f"[bench] decode batch {args.batch}: {ms_step:.3f} ms/step", file=sys.stderr, flush=True)
     if args.only == "decode":
-        print(json.dumps({"phase": "decode", "batch": args.batch, "ms_per_step": round(ms_step, 4)}))
+        nbytes = decode_bytes(shape, elem, args.batch, args.context + args.warmup + (args.steps + 1) / 2.0)
+        print(json.dumps({"phase": "decode", "batch": args.batch, "context": args.context, "ms_per_step": round(ms_step, 4),
+                          "tok_per_s": round(value, 1), "GBps": round(nbytes / (dt / args.steps) / 1e9, 1)}))
         return 0
     mean_ctx = PROMPT + args.warmup + (args.steps + 1) / 2.0
     nbytes = decode_bytes(shape, elem, args.batch, mean_ctx)

@@ -694,6 +694,29 @@ int gemm_mfma_launch(const GemmArgs& g, void* workspace, size_t workspace_bytes,
             parts = (g.K + part_k - 1) / part_k;
         }
     }
+    // One row of tiles (up to 256 rows): tiles of 256 x 128, and as many parts of K as make the sum of two costs
+    // least: the product itself, which takes the longer the fewer CUs have a block, and the planes of partial
+    // sums, which are written and read again (measured at 256 rows on the 7B shape: about 4 us for a part of
+    // q/k/v, 3.3 for o and down, that is 2.2 TB/s; q/k/v 37 to 29 us, o 31 to 26, down 70 to 63).
+    bool half_wide = false;
+    if (parts >= 2 && rows256 == 256) {
+        const int tiles128 = (g.N + 127) / 128;
+        const double weights_us = (double)g.N * g.K * 2 / 5.0e6, flops_us = 2.0 * 256 * g.N * g.K / 0.95e9;
+        const double product_us = weights_us > flops_us ? weights_us : flops_us;
+        const double plane_us = 2.0 * g.M * g.N * sizeof(float) / 2.2e6;
+        int best = 0;
+        double best_us = 0;
+        for (int p = 2; p <= parts && p <= g.K / 512; p++) {
+            const int blocks = tiles128 * p < 256 ? tiles128 * p : 256;
+            const double us = product_us * 256 / blocks + p * plane_us;
+            if (best == 0 || us < best_us) best = p, best_us = us;
+        }
+        if (best >= 2) {
+            half_wide = true;
+            part_k = ((g.K / 32 + best - 1) / best) * 32;
+            parts = (g.K + part_k - 1) / part_k;
+        }
+    }
     const bool halves = parts >= 2;
     // Tiles of 192 columns do three quarters of the work of 256 (a little less efficiently): they are
     // taken when they need fewer rounds over the CUs by more than that.
@@ -711,7 +734,8 @@ int gemm_mfma_launch(const GemmArgs& g, void* workspace, size_t workspace_bytes,
     else if (dma_ok && tiles256 >= 128)
         rc = launch_dma<256, 256, 32, 2, 4, 4>(g, kmode, kout, 1, g.K);
     else if (halves) {
-        rc = launch_dma<256, 256, 32, 2, 4, 4>(g, OUT_PARTIAL, workspace, parts, part_k);
+        rc = half_wide ? launch_dma<256, 128, 32, 4, 2, 6>(g, OUT_PARTIAL, workspace, parts, part_k)
+                       : launch_dma<256, 256, 32, 2, 4, 4>(g, OUT_PARTIAL, workspace, parts, part_k);
         if (rc) return rc;
         if (defer && pending_splits) {
             *pending_splits = parts;

@@ -120,7 +120,8 @@ def test_fp32_rows_do_not_depend_on_the_batch(ops32, N, K):
                                    (64, 4608, 3584), (48, 3584, 18944), (33, 37888, 256), (40, 1024, 8192),
                                    (150, 4608, 3584), (300, 3584, 4736), (1900, 4624, 192), (50, 33024, 320), (64, 65536, 64),
                                    (100, 3584, 18944), (128, 4096, 8192), (65, 37888, 1024),      # the stream kernel's tiles of 128 rows
-                                   (400, 3584, 18944), (256, 4608, 3584), (700, 3584, 3584)])     # 256-row tiles, K cut into parts
+                                   (400, 3584, 18944), (256, 4608, 3584), (700, 3584, 3584),      # 256-row tiles, K cut into parts
+                                   (200, 3584, 18944), (250, 3584, 3584), (192, 896, 4864)])      # one row of 256 x 128 tiles, parts by cost
 def test_gemm_on_matrix_cores(ops16, M, N, K):
     """bf16 x bf16 with K a multiple of 8 runs on the matrix cores (K split for small M; tiles of
     256 rows loaded straight into LDS for long prompts and wide outputs, with edges in M and N

@@ -178,6 +178,8 @@ def main():
     ap.add_argument("--context", type=int, default=PROMPT,
                     help="with --only decode: tokens every sequence holds before the timed steps (prefilled in portions "
                          "of 2,048); the default run's is 2,048")
+    ap.add_argument("--shape", choices=["7b", "0.5b", "32b"], default="7b",
+                    help="with --only: the layer sizes of the step (the default measurement's are the 7B shape's)")
     ap.add_argument("--no-peaks", action="store_true", help="skip the probes of the device's own peaks")
     ap.add_argument("--no-kernels", action="store_true", help="skip the timing by part")
     ap.add_argument("--workload", choices=["7b", "0.5b", "32b"], default="7b",
@@ -195,6 +197,9 @@ def main():
     if args.context != PROMPT and args.only != "decode":
         print("bench.py: --context goes with --only decode (the default measurement has 2,048-token prompts)")
         return 2
+    if args.shape != "7b" and args.only is None:
+        print("bench.py: --shape goes with --only prefill | decode (the default measurement is of the 7B shape)")
+        return 2
     if args.steps + args.warmup > NEW:
         print(f"bench.py: --steps + --warmup must not exceed the {NEW} new tokens of the workload")
         return 2
@@ -204,7 +209,7 @@ def main():
     import hf_cpu_amd
     import hf_cpu_amd.session as S
 
-    shape = dict(SHAPE_7B)
+    shape = dict(SHAPE_7B if args.shape == "7b" else WORKLOADS[args.shape]["shape"])
     layers_of_shape = shape["num_hidden_layers"]
     if args.layers:
         shape["num_hidden_layers"] = args.layers
@@ -254,7 +259,7 @@ def main():
             eng.release("prefill")
         kernels.update(kernel_fractions(eng, "prefill", one_prefill, 2, shape, elem, 1, PROMPT, peaks, short))
     if args.only == "prefill":
-        print(json.dumps({"phase": "prefill", "tokens": PROMPT, "ms": round(pre_s * 1e3, 3)}))
+        print(json.dumps({"phase": "prefill", "shape": args.shape, "tokens": PROMPT, "ms": round(pre_s * 1e3, 3)}))
         return 0
 
 
@@ -299,7 +304,8 @@ def main():
     print(f"[bench] decode batch {args.batch}: {ms_step:.3f} ms/step", file=sys.stderr, flush=True)
     if args.only == "decode":
         nbytes = decode_bytes(shape, elem, args.batch, args.context + args.warmup + (args.steps + 1) / 2.0)
-        print(json.dumps({"phase": "decode", "batch": args.batch, "context": args.context, "ms_per_step": round(ms_step, 4),
+        print(json.dumps({"phase": "decode", "shape": args.shape, "batch": args.batch, "context": args.context,
+                          "ms_per_step": round(ms_step, 4),
                           "tok_per_s": round(value, 1), "GBps": round(nbytes / (dt / args.steps) / 1e9, 1)}))
         return 0
     mean_ctx = PROMPT + args.warmup + (args.steps + 1) / 2.0

@@ -6,14 +6,19 @@
 // none of which waits for another. A wave has a ring of its own in LDS, filled by direct loads
 // (global_load_lds_dwordx4: 64 lanes x 16 bytes = 8 rows of 128 bytes a request; see gemm_mfma.hip for the
 // swizzled layout and the reason for the inline assembly): a unit is four requests for its 32 rows of W and one
-// for the 8 rows of A, requested R units ahead. There is no barrier and no other traffic
+// for the 8 rows of A, requested R units ahead. While they stream there is no barrier and no other traffic
 // between the waves of a block: the only wait is the wave's own, for its oldest unit.
 //
-// A column tile's K range is shared by the waves whose runs touch it. The workspace holds `slots` planes of
-// [M][N] fp32; the waves that work on a tile write their sums into planes 0, 1, ... in the order of their
-// numbers, and the wave that owns the tile's last unit clears the planes the tile did not need. The sum over the
-// planes in ascending order (by the next kernel, or by gemm_finish) is the product: which wave adds what is fixed
-// by the sizes alone, so results are reproducible.
+// A column tile's K range is shared by the waves whose runs touch it. The waves of a block add their parts of a
+// tile together in LDS when all are done (a wave's run touches at most two tiles in part: the one it begins in and
+// the one it ends in; tiles it covers whole it writes itself), so a tile has one partial sum per block that
+// touches it. The workspace holds `slots` planes of [M][N] fp32; the blocks that work on a tile write into planes
+// 0, 1, ... in the order of their numbers, and the block that owns the tile's last unit clears the planes the tile
+// did not need. The sum over the planes in ascending order (by the next kernel, or by gemm_finish) is the product:
+// which wave adds what, and in which order, is fixed by the sizes alone, so results are reproducible. (With a plane
+// per wave the o and down products of the 7B shape left 20 planes for the norm that follows to add up, with a
+// plane per block 4: the norm takes 4.9 instead of 7.0 us, rotary and cache store 4.95 instead of 6.3, the
+// products themselves 0.1 to 0.8 us more; a step of 8 rows 3.92 instead of 4.06 ms.)
 //
 // Against the product that stages tiles of 32 x 128 through LDS shared by four waves with a barrier a step
 // (gemm_mfma_kernel), at 8 rows on the 7B shape: gate+up 51 against 56 us, down 24.5 against 30, q/k/v 9.5
@@ -48,8 +53,7 @@ __global__ __launch_bounds__(WAVES* WAVE) void gemm_wave_kernel(const uint16_t* 
     const long long U = (long long)tiles * nk;
     const int G = gridDim.x * WAVES, g = blockIdx.x * WAVES + wave;
     const int u0 = (int)((long long)g * U / G), u1 = (int)((long long)(g + 1) * U / G);
-    const int n_units = u1 - u0;
-    if (n_units <= 0) return;
+    const int n_units = u1 - u0 > 0 ? u1 - u0 : 0;       // (the launcher sees to it that every wave has units)
 
     uint16_t* ring = smem + wave * (R * UNIT);
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint16_t*)ring;
@@ -96,13 +100,45 @@ __global__ __launch_bounds__(WAVES* WAVE) void gemm_wave_kernel(const uint16_t* 
     const int row = lane & 31;
     const bool has_a = row < 8 * AR;                          // this lane's row of A exists in the ring
 
+    // Parts of tiles that this wave shares with others wait in LDS behind the rings: two records a wave of
+    // 4 AR floats a lane, with the tile's number (-1: unused) and whether the part holds the tile's last unit.
+    float* seg = reinterpret_cast<float*>(smem + WAVES * R * UNIT);
+    int* seg_tile = reinterpret_cast<int*>(seg + WAVES * 2 * 4 * AR * WAVE);
+    int* seg_ends = seg_tile + 2 * WAVES;
+    if (lane < 2) {
+        seg_tile[2 * wave + lane] = -1;
+        seg_ends[2 * wave + lane] = 0;
+    }
+    auto store_rows = [&](float* plane, int tile, const float* v) {     // a lane's 4 AR values of a tile into a plane
+        const int c = tile * 32 + row;
+        if (c < N) {
+#pragma unroll
+            for (int r = 0; r < 4 * AR; r++) {
+                const int m = 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
+                if (m < M) plane[(size_t)m * N + c] = v[r];
+            }
+        }
+    };
+    auto clear_from = [&](int tile, int from) {                         // planes the tile did not need
+        const int c = tile * 32 + row;
+        if (c < N) {
+#pragma unroll
+            for (int r = 0; r < 4 * AR; r++) {
+                const int m = 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
+                if (m < M)
+                    for (int sl = from; sl < slots; sl++) partial[((size_t)sl * M + m) * N + c] = 0.f;
+            }
+        }
+    };
+
     floatx16 acc;
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[r] = 0.f;
 #pragma unroll
     for (int p = 0; p < R; p++)
         if (p < n_units) request(u0 + p, p);
-    int slot = 0, tile = u0 / nk, kt = u0 % nk;
+    int slot = 0, tile = n_units > 0 ? u0 / nk : 0, kt = n_units > 0 ? u0 % nk : 0;
+    int kt_first = kt, n_parts = 0;                                     // where this wave began the tile; records used
     for (int u = 0; u < n_units; u++) {
         // the unit has landed when at most the R - 1 newer units' requests are out (at the run's end fewer are
         // out than that: then all are waited for, which by then are on their way anyway)
@@ -124,27 +160,67 @@ __global__ __launch_bounds__(WAVES* WAVE) void gemm_wave_kernel(const uint16_t* 
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");    // the fragments are read: the slot may be filled again
         if (u + R < n_units) request(u0 + u + R, slot);
         slot = slot + 1 < R ? slot + 1 : 0;
-        // The tile's last unit, or this wave's: the sums go to the wave's plane of the workspace. Element r of a
-        // lane is row 8 (r / 4) + 4 (lane / 32) + r % 4, column lane % 32 of the tile.
+        // The tile's last unit, or this wave's: element r of a lane is row 8 (r / 4) + 4 (lane / 32) + r % 4,
+        // column lane % 32 of the tile. A tile that this wave covered whole goes to plane 0; a part waits in LDS.
         if (kt == nk - 1 || u == n_units - 1) {
-            const int first = wave_of_unit((long long)tile * nk, U, G);
-            float* plane = partial + (size_t)(g - first) * M * N;
-            const int col = tile * 32 + row;
-            if (col < N) {
+            float v[4 * AR];
 #pragma unroll
-                for (int r = 0; r < 4 * AR; r++) {
-                    const int m = 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
-                    if (m < M) {
-                        plane[(size_t)m * N + col] = acc[r];
-                        if (kt == nk - 1)                    // planes that this tile did not need
-                            for (int s = g - first + 1; s < slots; s++) partial[((size_t)s * M + m) * N + col] = 0.f;
-                    }
+            for (int r = 0; r < 4 * AR; r++) v[r] = acc[r];
+            if (kt_first == 0 && kt == nk - 1) {
+                store_rows(partial, tile, v);
+                clear_from(tile, 1);
+            } else {
+                float4* rec = reinterpret_cast<float4*>(seg) + (size_t)((2 * wave + n_parts) * WAVE + lane) * AR;
+#pragma unroll
+                for (int i = 0; i < AR; i++) rec[i] = make_float4(v[4 * i], v[4 * i + 1], v[4 * i + 2], v[4 * i + 3]);
+                if (lane == 0) {
+                    seg_tile[2 * wave + n_parts] = tile;
+                    seg_ends[2 * wave + n_parts] = kt == nk - 1;
                 }
+                n_parts++;
             }
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[r] = 0.f;
+            kt_first = 0;
         }
         if (++kt == nk) { kt = 0; tile++; }
+    }
+    __syncthreads();
+    // The records in the order of the waves; those of one tile are neighbours. The wave that holds the first of
+    // a tile's records adds them up in that order and writes the block's plane of the tile. Every lane reads one
+    // record's tags, and all records are asked for at once: a loop over the tile's records would be a chain of
+    // LDS round trips at the very end of the kernel.
+    const int tag = seg_tile[lane & (2 * WAVES - 1)], tag_ends = seg_ends[lane & (2 * WAVES - 1)];
+    float4 rec[2 * WAVES][AR];
+#pragma unroll
+    for (int k = 0; k < 2 * WAVES; k++)
+#pragma unroll
+        for (int i = 0; i < AR; i++) rec[k][i] = reinterpret_cast<const float4*>(seg)[(size_t)(k * WAVE + lane) * AR + i];
+    for (int j = 0; j < 2; j++) {
+        const int q = 2 * wave + j, t = __builtin_amdgcn_readlane(tag, q);
+        if (t < 0) continue;
+        int before = q - 1;
+        while (before >= 0 && __builtin_amdgcn_readlane(tag, before) < 0) before--;
+        if (before >= 0 && __builtin_amdgcn_readlane(tag, before) == t) continue;      // another wave leads this tile
+        float v[4 * AR];
+#pragma unroll
+        for (int r = 0; r < 4 * AR; r++) v[r] = 0.f;
+        bool ends = false;
+#pragma unroll
+        for (int k = 0; k < 2 * WAVES; k++) {
+            if (__builtin_amdgcn_readlane(tag, k) != t) continue;                        // uniform over the wave
+#pragma unroll
+            for (int i = 0; i < AR; i++) {
+                v[4 * i] += rec[k][i].x;
+                v[4 * i + 1] += rec[k][i].y;
+                v[4 * i + 2] += rec[k][i].z;
+                v[4 * i + 3] += rec[k][i].w;
+            }
+            ends = ends || __builtin_amdgcn_readlane(tag_ends, k) != 0;
+        }
+        const int mine = (int)blockIdx.x - wave_of_unit((long long)t * nk, U, G) / WAVES;
+        store_rows(partial + (size_t)mine * M * N, t, v);
+        if (ends) clear_from(t, mine + 1);
     }
 }
 
@@ -161,21 +237,25 @@ static int wave_cu_count() {
 // Eight waves a block. Four where eight leave a wave only three or four units (q/k/v and o of the 7B shape), which
 // halves the planes of partial sums that the next kernel reads, was slower a step (4.08 against 4.06 ms at 8 rows).
 
-// The number of workspace planes a product of this shape needs, or 0 if this kernel does not take it.
+// The number of workspace planes a product of this shape needs (the most blocks that touch one tile), or 0 if
+// this kernel does not take it.
 int gemm_wave_slots(const GemmArgs& g, size_t workspace_bytes) {
     if (g.M > 8 || g.K % 64 != 0 || g.lda >= (1 << 22) || g.ldw >= (1 << 22) || g.N < 32) return 0;
     const long long nk = g.K / 64, tiles = (g.N + 31) / 32, U = tiles * nk;
     const int G = wave_cu_count() * WAVES;
     if (U < G) return 0;                                     // fewer units than waves: the tiled kernel's splits do as well
-    const long long per_wave = U / G;                        // the shortest run
-    const long long slots = (nk + per_wave - 1) / per_wave + 1;
+    int slots = 1;
+    for (long long t = 0; t < tiles; t++) {
+        const int n = wave_of_unit(t * nk + nk - 1, U, G) / WAVES - wave_of_unit(t * nk, U, G) / WAVES + 1;
+        if (n > slots) slots = n;
+    }
     if (slots > 64 || (size_t)slots * g.M * g.N * sizeof(float) > workspace_bytes) return 0;
-    return (int)slots;
+    return slots;
 }
 
 template <int AR, int R>
 static int launch_wave(const GemmArgs& g, float* partial, int slots) {
-    constexpr int SMEM = WAVES * R * (4 + AR) * 1024;
+    constexpr int SMEM = WAVES * R * (4 + AR) * 1024 + WAVES * 2 * 4 * AR * WAVE * 4 + 4 * WAVES * 4;   // rings, records, their tags
     static_assert(SMEM <= 160 * 1024, "the rings must fit into a CU's LDS");
     auto kernel = gemm_wave_kernel<AR, R>;
     static bool configured = false;

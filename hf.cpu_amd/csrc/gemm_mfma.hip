@@ -627,7 +627,7 @@ int gemm_mfma_launch(const GemmArgs& g, void* workspace, size_t workspace_bytes,
         hfa_set_error("gemm: the gate/up epilogue needs N a multiple of 64, no bias and a bf16 output");
         return 1;
     }
-    if (g.M <= 8) {                          // very few rows: every wave streams its own run of the weights
+    if (g.M <= 16) {                         // very few rows: every wave streams its own run of the weights
         const int slots = gemm_wave_slots(g, workspace ? workspace_bytes : 0);
         if (slots > 0) {
             const int rc = gemm_wave_launch(g, workspace, slots);

@@ -1,4 +1,4 @@
-// bf16 matrix product for up to 8 rows (decode), bound by the speed at which the weights stream in:
+// bf16 matrix product for up to 16 rows (decode), bound by the speed at which the weights stream in:
 // out[m, n] = sum_k a[m, k] * w[n, k], left as partial sums in a workspace.
 //
 // Every wave streams by itself. The work is the list of (tile of 32 output columns, 64 columns of K) units in
@@ -10,8 +10,9 @@
 // between the waves of a block: the only wait is the wave's own, for its oldest unit.
 //
 // A column tile's K range is shared by the waves whose runs touch it. The waves of a block add their parts of a
-// tile together in LDS when all are done (a wave's run touches at most two tiles in part: the one it begins in and
-// the one it ends in; tiles it covers whole it writes itself), so a tile has one partial sum per block that
+// tile together in LDS when all are done: a wave's run touches at most two tiles in part, the one it begins in and
+// the one it ends in (tiles it covers whole it writes itself); it keeps the two parts in registers until its run
+// is done and then puts them into its ring, which is free by then. So a tile has one partial sum per block that
 // touches it. The workspace holds `slots` planes of [M][N] fp32; the blocks that work on a tile write into planes
 // 0, 1, ... in the order of their numbers, and the block that owns the tile's last unit clears the planes the tile
 // did not need. The sum over the planes in ascending order (by the next kernel, or by gemm_finish) is the product:
@@ -22,9 +23,10 @@
 //
 // Against the product that stages tiles of 32 x 128 through LDS shared by four waves with a barrier a step
 // (gemm_mfma_kernel), at 8 rows on the 7B shape: gate+up 51 against 56 us, down 24.5 against 30, q/k/v 9.5
-// against 11.8, o 8.4 against 10.1. With 16 and 32 rows of A in the ring (two and four requests a unit, which the
-// template still allows) fewer bytes of W are on their way for the same LDS, and a step was slower than with the
-// tiled kernel (4.56 against 4.49 ms at 16 rows, 5.53 against 5.07 at 32): those rows stay there.
+// against 11.8, o 8.4 against 10.1. For 9 to 16 rows a unit has two requests for A: fewer bytes of W are on their
+// way for the same LDS and the products are a little slower than the tiled kernel's, but the few planes make up for
+// it in the kernels that follow (a step of 16 rows 4.28 against 4.40 ms). With four requests (32 rows) a step
+// was slower (5.53 against 5.07 ms): those rows stay with the tiled kernel.
 #include "common.h"
 #include "gemm_internal.h"
 
@@ -100,15 +102,12 @@ __global__ __launch_bounds__(WAVES* WAVE) void gemm_wave_kernel(const uint16_t* 
     const int row = lane & 31;
     const bool has_a = row < 8 * AR;                          // this lane's row of A exists in the ring
 
-    // Parts of tiles that this wave shares with others wait in LDS behind the rings: two records a wave of
-    // 4 AR floats a lane, with the tile's number (-1: unused) and whether the part holds the tile's last unit.
-    float* seg = reinterpret_cast<float*>(smem + WAVES * R * UNIT);
-    int* seg_tile = reinterpret_cast<int*>(seg + WAVES * 2 * 4 * AR * WAVE);
+    // Parts of tiles that this wave shares with others (at most two: the end of the tile it began in, the
+    // beginning of the tile it ends in) stay in registers until its run is done, then go into its ring, which
+    // is free by then: two records a wave of 4 AR floats a lane. Their tags lie behind the rings: the tile's
+    // number (-1: unused) and whether the part holds the tile's last unit.
+    int* seg_tile = reinterpret_cast<int*>(smem + WAVES * R * UNIT);
     int* seg_ends = seg_tile + 2 * WAVES;
-    if (lane < 2) {
-        seg_tile[2 * wave + lane] = -1;
-        seg_ends[2 * wave + lane] = 0;
-    }
     auto store_rows = [&](float* plane, int tile, const float* v) {     // a lane's 4 AR values of a tile into a plane
         const int c = tile * 32 + row;
         if (c < N) {
@@ -138,7 +137,11 @@ __global__ __launch_bounds__(WAVES* WAVE) void gemm_wave_kernel(const uint16_t* 
     for (int p = 0; p < R; p++)
         if (p < n_units) request(u0 + p, p);
     int slot = 0, tile = n_units > 0 ? u0 / nk : 0, kt = n_units > 0 ? u0 % nk : 0;
-    int kt_first = kt, n_parts = 0;                                     // where this wave began the tile; records used
+    int kt_first = kt;                                                  // where this wave began the tile
+    float head[4 * AR], tail[4 * AR];                                   // the two parts and their tiles (-1: none)
+    int head_tile = -1, tail_tile = -1;
+#pragma unroll
+    for (int r = 0; r < 4 * AR; r++) head[r] = tail[r] = 0.f;
     for (int u = 0; u < n_units; u++) {
         // the unit has landed when at most the R - 1 newer units' requests are out (at the run's end fewer are
         // out than that: then all are waited for, which by then are on their way anyway)
@@ -161,29 +164,45 @@ __global__ __launch_bounds__(WAVES* WAVE) void gemm_wave_kernel(const uint16_t* 
         if (u + R < n_units) request(u0 + u + R, slot);
         slot = slot + 1 < R ? slot + 1 : 0;
         // The tile's last unit, or this wave's: element r of a lane is row 8 (r / 4) + 4 (lane / 32) + r % 4,
-        // column lane % 32 of the tile. A tile that this wave covered whole goes to plane 0; a part waits in LDS.
+        // column lane % 32 of the tile. A tile that this wave covered whole goes to plane 0.
         if (kt == nk - 1 || u == n_units - 1) {
-            float v[4 * AR];
-#pragma unroll
-            for (int r = 0; r < 4 * AR; r++) v[r] = acc[r];
             if (kt_first == 0 && kt == nk - 1) {
+                float v[4 * AR];
+#pragma unroll
+                for (int r = 0; r < 4 * AR; r++) v[r] = acc[r];
                 store_rows(partial, tile, v);
                 clear_from(tile, 1);
-            } else {
-                float4* rec = reinterpret_cast<float4*>(seg) + (size_t)((2 * wave + n_parts) * WAVE + lane) * AR;
+            } else if (kt == nk - 1) {                         // the end of a tile that another wave began
 #pragma unroll
-                for (int i = 0; i < AR; i++) rec[i] = make_float4(v[4 * i], v[4 * i + 1], v[4 * i + 2], v[4 * i + 3]);
-                if (lane == 0) {
-                    seg_tile[2 * wave + n_parts] = tile;
-                    seg_ends[2 * wave + n_parts] = kt == nk - 1;
-                }
-                n_parts++;
+                for (int r = 0; r < 4 * AR; r++) head[r] = acc[r];
+                head_tile = tile;
+            } else {                                           // the beginning of a tile that another wave ends
+#pragma unroll
+                for (int r = 0; r < 4 * AR; r++) tail[r] = acc[r];
+                tail_tile = tile;
             }
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[r] = 0.f;
             kt_first = 0;
         }
         if (++kt == nk) { kt = 0; tile++; }
+    }
+    // all requests of this wave have landed and its fragments are read: the ring takes the records
+    float4* mine_rec = reinterpret_cast<float4*>(ring);
+    {
+        const float* first = head_tile >= 0 ? head : tail;    // the records in the order of their tiles
+        const int t0 = head_tile >= 0 ? head_tile : tail_tile, t1 = head_tile >= 0 ? tail_tile : -1;
+#pragma unroll
+        for (int i = 0; i < AR; i++) {
+            mine_rec[lane * AR + i] = make_float4(first[4 * i], first[4 * i + 1], first[4 * i + 2], first[4 * i + 3]);
+            mine_rec[(WAVE + lane) * AR + i] = make_float4(tail[4 * i], tail[4 * i + 1], tail[4 * i + 2], tail[4 * i + 3]);
+        }
+        if (lane == 0) {
+            seg_tile[2 * wave] = t0;
+            seg_ends[2 * wave] = head_tile >= 0;
+            seg_tile[2 * wave + 1] = t1;
+            seg_ends[2 * wave + 1] = 0;
+        }
     }
     __syncthreads();
     // The records in the order of the waves; those of one tile are neighbours. The wave that holds the first of
@@ -195,7 +214,8 @@ __global__ __launch_bounds__(WAVES* WAVE) void gemm_wave_kernel(const uint16_t* 
 #pragma unroll
     for (int k = 0; k < 2 * WAVES; k++)
 #pragma unroll
-        for (int i = 0; i < AR; i++) rec[k][i] = reinterpret_cast<const float4*>(seg)[(size_t)(k * WAVE + lane) * AR + i];
+        for (int i = 0; i < AR; i++)
+            rec[k][i] = reinterpret_cast<const float4*>(smem + (k / 2) * (R * UNIT))[((k % 2) * WAVE + lane) * AR + i];
     for (int j = 0; j < 2; j++) {
         const int q = 2 * wave + j, t = __builtin_amdgcn_readlane(tag, q);
         if (t < 0) continue;
@@ -240,7 +260,7 @@ static int wave_cu_count() {
 // The number of workspace planes a product of this shape needs (the most blocks that touch one tile), or 0 if
 // this kernel does not take it.
 int gemm_wave_slots(const GemmArgs& g, size_t workspace_bytes) {
-    if (g.M > 8 || g.K % 64 != 0 || g.lda >= (1 << 22) || g.ldw >= (1 << 22) || g.N < 32) return 0;
+    if (g.M > 16 || g.K % 64 != 0 || g.lda >= (1 << 22) || g.ldw >= (1 << 22) || g.N < 32) return 0;
     const long long nk = g.K / 64, tiles = (g.N + 31) / 32, U = tiles * nk;
     const int G = wave_cu_count() * WAVES;
     if (U < G) return 0;                                     // fewer units than waves: the tiled kernel's splits do as well
@@ -255,7 +275,7 @@ int gemm_wave_slots(const GemmArgs& g, size_t workspace_bytes) {
 
 template <int AR, int R>
 static int launch_wave(const GemmArgs& g, float* partial, int slots) {
-    constexpr int SMEM = WAVES * R * (4 + AR) * 1024 + WAVES * 2 * 4 * AR * WAVE * 4 + 4 * WAVES * 4;   // rings, records, their tags
+    constexpr int SMEM = WAVES * R * (4 + AR) * 1024 + 4 * WAVES * 4;   // rings, the records' tags
     static_assert(SMEM <= 160 * 1024, "the rings must fit into a CU's LDS");
     auto kernel = gemm_wave_kernel<AR, R>;
     static bool configured = false;
@@ -273,4 +293,6 @@ static int launch_wave(const GemmArgs& g, float* partial, int slots) {
     return 0;
 }
 
-int gemm_wave_launch(const GemmArgs& g, void* workspace, int slots) { return launch_wave<1, 3>(g, (float*)workspace, slots); }
+int gemm_wave_launch(const GemmArgs& g, void* workspace, int slots) {
+    return g.M <= 8 ? launch_wave<1, 3>(g, (float*)workspace, slots) : launch_wave<2, 3>(g, (float*)workspace, slots);
+}

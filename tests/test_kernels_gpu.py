@@ -747,9 +747,10 @@ def test_probes_of_the_device_peaks(ops16):
 
 @pytest.mark.parametrize("M,N,K", [(1, 4608, 3584), (8, 3584, 18944), (3, 2016, 896), (9, 37888, 3584), (16, 1000, 1024),
                                    (17, 4608, 3584), (32, 3584, 3584), (8, 152064, 3584), (5, 33, 8192), (32, 40, 16384),
-                                   (7, 37888, 3584), (2, 3584, 3584), (8, 9000, 1024), (4, 70000, 128), (6, 65530, 192)])
+                                   (7, 37888, 3584), (2, 3584, 3584), (8, 9000, 1024), (4, 70000, 128), (6, 65530, 192),
+                                   (12, 3584, 18944), (16, 4608, 3584), (13, 70000, 128)])
 def test_products_of_few_rows_streamed_wave_by_wave(ops16, M, N, K):
-    """The product for up to 8 rows in which every wave streams a run of the weights by itself (gemm_wave.hip),
+    """The product for up to 16 rows in which every wave streams a run of the weights by itself (gemm_wave.hip),
     and the tiled product that takes more rows, against a float64 product of the same bf16 operands: widths that are no multiple of the 32-column tiles (the last tile repeats its last row), runs of
     a few units and of hundreds, tiles that one wave covers whole, that the waves of one block share and that
     several blocks share, results stored, accumulated and left for the next kernel; and the same bits

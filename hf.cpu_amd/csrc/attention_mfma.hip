@@ -858,10 +858,12 @@ int attn_mfma_launch(const AttnArgs& a) {
     const long waves = (long)(a.max_q_len <= tpt ? a.n_seqs : (a.n_tokens + tpt - 1) / tpt) * a.n_kv_heads;
     const int span = a.window > 0 && a.window + a.max_q_len < a.max_seq_len ? a.window + a.max_q_len : a.max_seq_len;
     int n_chunks = 1, chunk_keys = a.max_seq_len;
-    // (512 waves in all: with 1,024 a step of the 7B shape took 1.3 % longer at 64 sequences and 4.5 % longer at
-    // 8 sequences of 16,384 tokens, with 256 more than that; 8 sequences of 2,048 tokens do not tell them apart.)
-    if (waves < 512 && span > 128 && a.workspace) {
-        int want = (int)((512 + waves - 1) / waves);
+    // How many waves in all is a measured choice. Head size 128 (7B shape): 512; with 1,024 a step took 1.3 % longer
+    // at 64 sequences and 4.5 % longer at 8 sequences of 16,384 tokens, with 256 more than that. Head size 64 (0.5B
+    // shape), where a wave has half the work per key: 1,024; with 512 a step of 64 sequences took 4.5 % longer.
+    const int fill = a.head_dim > 64 ? 512 : 1024;
+    if (waves < fill && span > 128 && a.workspace) {
+        int want = (int)((fill + waves - 1) / waves);
         const int most = (span + 63) / 64;
         if (want > most) want = most;
         chunk_keys = ((a.max_seq_len + want - 1) / want + KB - 1) / KB * KB;

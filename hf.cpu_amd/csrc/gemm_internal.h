@@ -31,7 +31,7 @@ int gemm_mode_of(const GemmArgs& g);
 // order is the product.
 int gemm_stream_slots(const GemmArgs& g, size_t workspace_bytes);
 int gemm_stream_launch(const GemmArgs& g, void* workspace, int slots);
-// bf16 x bf16 for M <= 8 as one stream of (tile of 32 columns, 64 columns of K) units cut evenly over all waves
+// bf16 x bf16 for M <= 16 as one stream of (tile of 32 columns, 64 columns of K) units cut evenly over all waves
 // of the machine, every wave streaming its run by itself (K a multiple of 64). gemm_wave_slots() says how many
 // [M][N] fp32 planes of the workspace the product will leave its partial sums in (0: not taken).
 int gemm_wave_slots(const GemmArgs& g, size_t workspace_bytes);

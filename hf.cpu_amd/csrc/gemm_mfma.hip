@@ -17,15 +17,15 @@
 // bias and the output mode. Nothing is accumulated with atomics: results are reproducible.
 //
 // Which kernel takes which shape (gemm_mfma_launch, at the end of this file):
-//   M <= 8           gemm_wave_kernel (gemm_wave.hip) if K is a multiple of 64 and there are as many units as waves; else as
+//   M <= 16          gemm_wave_kernel (gemm_wave.hip) if K is a multiple of 64 and there are as many units as waves; else as
 //   M <= 32          gemm_mfma_kernel, tiles of 32 x 128, K split, two register sets of loads in flight
 //   M in 33 .. 128   gemm_stream_kernel (gemm_stream.hip) if N is a multiple of 128 and K of 64, the output
 //                    has fewer than 512 tiles and a block gets 16 units or more; else gemm_mfma_kernel
 //                    with tiles of 64 x 128 or 128 x 128
 //   M > 64           gemm_dma_kernel (below) with tiles of 256 rows, if M wastes few of them and the
 //                    output has 128 tiles of 256 x 256 (tiles of 256 x 192 where those need fewer rounds
-//                    over the CUs; with fewer K is cut into parts that give every CU a block, or the tiles
-//                    are 256 x 128); else
+//                    over the CUs; with fewer K is cut into parts that give every CU a block, with tiles of
+//                    256 x 128 if M is at most 256; or the tiles are 256 x 128 without parts); else
 //                    gemm_mfma_kernel with tiles of 128 x 128
 #include <type_traits>
 

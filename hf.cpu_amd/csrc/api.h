@@ -64,13 +64,15 @@ int hfa_attention_prompt_rows(void);
 // bound the runs and the positions. bf16 with head_dim a multiple of 32, page_tokens a multiple
 // of 4 and at most 32 query heads per key/value head runs on the matrix cores, the key range
 // split over `workspace` when there are few queries; everything else, and everything when
-// `force_plain`, runs the plain kernel.
+// `force_plain`, runs the plain kernel. `slopes` (one fp32 per query head, or null) is the hook for a position
+// encoding that enters the scores rather than the queries and keys: the score of key j for the query at p
+// becomes dot * scale + slopes[h] * (j - p); with slopes the plain kernel runs.
 int hfa_paged_attention(const void* q, int dtype, int ldq, const void* k_cache, const void* v_cache,
                         int kv_width, const int* block_table, int max_blocks, const int* token_slot,
                         const int* positions, const int* q_start, int n_seqs, int max_q_len, int max_seq_len,
                         void* out, int ldo, int n_tokens, int n_heads, int n_kv_heads, int head_dim,
-                        int page_tokens, int window, float scale, void* workspace, size_t workspace_bytes,
-                        int force_plain, hipStream_t stream);
+                        int page_tokens, int window, float scale, const float* slopes, void* workspace,
+                        size_t workspace_bytes, int force_plain, hipStream_t stream);
 
 // out[t, i] = silu(gate_up[t, i]) * gate_up[t, width + i].  (src/model.c:532-538)
 int hfa_swiglu(const void* gate_up, void* out, int dtype, int n_tokens, int width, hipStream_t stream);

@@ -47,7 +47,7 @@ __global__ __launch_bounds__(WAVE) void attn_generic_kernel(
     const T* __restrict__ q, int ldq, const T* __restrict__ kc, const T* __restrict__ vc, int kvw,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ token_slot,
     const int* __restrict__ positions, T* __restrict__ out, int ldo, int H, int G, int D, int page_tokens,
-    int window, float scale) {
+    int window, float scale, const float* __restrict__ slopes) {
     __shared__ float q_s[ATT_MAX_D];
     __shared__ float p_s[WAVE];
     __shared__ int row_s[WAVE];
@@ -58,6 +58,7 @@ __global__ __launch_bounds__(WAVE) void attn_generic_kernel(
     for (int d = lane; d < D; d += WAVE) q_s[d] = to_f32(q[(size_t)t * ldq + h * D + d]);
     __syncthreads();
     const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+    const float slope = slopes ? slopes[h] : 0.f;           // a position encoding that enters the scores
     float m = -INFINITY, l = 0.f;
     float acc[ATT_MAX_D / WAVE];
 #pragma unroll
@@ -71,6 +72,7 @@ __global__ __launch_bounds__(WAVE) void attn_generic_kernel(
         if (valid) {
             row = bt[j / page_tokens] * page_tokens + j % page_tokens;
             s = dot_row(q_s, kc + (size_t)row * kvw + kvh * D, D) * scale;
+            if (slopes) s += slope * (float)(j - pos);
         }
         // every tile holds at least one visible key, so the maximum is finite
         const float mn = fmaxf(m, wave_max(s));
@@ -110,7 +112,7 @@ __global__ __launch_bounds__(WAVE) void attn_generic_kernel(
 int attn_generic_launch(const void* q, int dtype, int ldq, const void* k_cache, const void* v_cache, int kv_width,
                         const int* block_table, int max_blocks, const int* token_slot, const int* positions,
                         void* out, int ldo, int n_tokens, int n_heads, int n_kv_heads, int head_dim,
-                        int page_tokens, int window, float scale, hipStream_t stream) {
+                        int page_tokens, int window, float scale, const float* slopes, hipStream_t stream) {
     HFA_REQUIRE(head_dim <= ATT_MAX_D, "paged_attention: head_dim %d exceeds the kernel's limit %d", head_dim,
                 ATT_MAX_D);
     HFA_REQUIRE(n_heads <= 65535, "paged_attention: %d heads exceed the grid", n_heads);
@@ -118,11 +120,11 @@ int attn_generic_launch(const void* q, int dtype, int ldq, const void* k_cache, 
     if (dtype == HFA_F32)
         attn_generic_kernel<float><<<grid, WAVE, 0, stream>>>(
             (const float*)q, ldq, (const float*)k_cache, (const float*)v_cache, kv_width, block_table, max_blocks,
-            token_slot, positions, (float*)out, ldo, n_heads, n_kv_heads, head_dim, page_tokens, window, scale);
+            token_slot, positions, (float*)out, ldo, n_heads, n_kv_heads, head_dim, page_tokens, window, scale, slopes);
     else
         attn_generic_kernel<bf16><<<grid, WAVE, 0, stream>>>(
             (const bf16*)q, ldq, (const bf16*)k_cache, (const bf16*)v_cache, kv_width, block_table, max_blocks,
-            token_slot, positions, (bf16*)out, ldo, n_heads, n_kv_heads, head_dim, page_tokens, window, scale);
+            token_slot, positions, (bf16*)out, ldo, n_heads, n_kv_heads, head_dim, page_tokens, window, scale, slopes);
     HFA_LAUNCH_CHECK("paged_attention");
     return 0;
 }
@@ -131,8 +133,8 @@ extern "C" int hfa_paged_attention(const void* q, int dtype, int ldq, const void
                                    int kv_width, const int* block_table, int max_blocks, const int* token_slot,
                                    const int* positions, const int* q_start, int n_seqs, int max_q_len,
                                    int max_seq_len, void* out, int ldo, int n_tokens, int n_heads, int n_kv_heads,
-                                   int head_dim, int page_tokens, int window, float scale, void* workspace,
-                                   size_t workspace_bytes, int force_plain, hipStream_t stream) {
+                                   int head_dim, int page_tokens, int window, float scale, const float* slopes,
+                                   void* workspace, size_t workspace_bytes, int force_plain, hipStream_t stream) {
     HFA_REQUIRE(n_tokens > 0 && n_heads > 0 && n_kv_heads > 0 && head_dim > 0 && page_tokens > 0 && max_blocks > 0,
                 "paged_attention: bad sizes");
     HFA_REQUIRE(n_heads % n_kv_heads == 0, "paged_attention: %d heads are not a multiple of %d key/value heads",
@@ -144,8 +146,9 @@ extern "C" int hfa_paged_attention(const void* q, int dtype, int ldq, const void
     AttnArgs a = {q, ldq, k_cache, v_cache, kv_width, block_table, max_blocks, token_slot, positions, q_start,
                   n_seqs, max_q_len, max_seq_len, out, ldo, n_tokens, n_heads, n_kv_heads, head_dim, page_tokens,
                   window, scale, workspace, workspace_bytes, stream};
-    if (!force_plain && dtype == HFA_BF16 && attn_mfma_supports(a)) return attn_mfma_launch(a);
+    // the matrix-core kernels take no slopes: scores with a position term go the plain way
+    if (!force_plain && !slopes && dtype == HFA_BF16 && attn_mfma_supports(a)) return attn_mfma_launch(a);
     return attn_generic_launch(q, dtype, ldq, k_cache, v_cache, kv_width, block_table, max_blocks, token_slot,
                                positions, out, ldo, n_tokens, n_heads, n_kv_heads, head_dim, page_tokens, window,
-                               scale, stream);
+                               scale, slopes, stream);
 }

@@ -308,9 +308,14 @@ class Ops:
             0 if pend is None else pend.splits,
             None if pend is None or pend.bias is None else pend.bias.data_ptr(), self._stream()))
 
-    def paged_attention(self, q, n_heads, n_kv_heads, head_dim, cache, step, window, scale, out):
-        """Attention of the first ``n_heads * head_dim`` columns of ``q`` over ``cache``."""
+    def paged_attention(self, q, n_heads, n_kv_heads, head_dim, cache, step, window, scale, out, slopes=None):
+        """Attention of the first ``n_heads * head_dim`` columns of ``q`` over ``cache``. ``slopes``
+        (fp32, one per query head): the score of key j for the query at p gets ``slopes[h] * (j - p)``
+        added, for position encodings that enter the scores; the plain kernel then runs."""
         self.settle()
+        if slopes is not None and (slopes.dtype != torch.float32 or slopes.numel() != n_heads or not slopes.is_contiguous()
+                                   or slopes.device != q.device):
+            fail(EINVAL, "paged_attention: slopes must be contiguous fp32 on the device, one per query head")
         T = q.shape[0]
         ldq, ldo = _rows(q, "attention q"), _rows(out, "attention out")
         g = step.group(cache.group)
@@ -322,7 +327,7 @@ class Ops:
         _ints(step.positions, "positions", T)
         _ints(step.q_start, "q_start", step.n_seqs + 1)
         # the matrix-core kernels address the cache with 32-bit element offsets and 24-bit row numbers
-        plain = self.force_plain_attention or cache.k.numel() >= 1 << 32 or cache.k.shape[0] >= 1 << 24
+        plain = self.force_plain_attention or slopes is not None or cache.k.numel() >= 1 << 32 or cache.k.shape[0] >= 1 << 24
 
         def call(first, n_tokens, q_start, n_seqs, max_q_len):
             self._check(self.lib.hfa_paged_attention(
@@ -330,7 +335,8 @@ class Ops:
                 cache.k.shape[1], g.block_table.data_ptr(), g.block_table.shape[1],
                 step.token_slot.data_ptr() + 4 * first, step.positions.data_ptr() + 4 * first, q_start.data_ptr(), n_seqs,
                 max_q_len, step.max_seq_len, out.data_ptr() + first * ldo * out.element_size(), ldo, n_tokens, n_heads,
-                n_kv_heads, head_dim, cache.page_tokens, int(window), float(scale), self.attn_workspace.data_ptr(),
+                n_kv_heads, head_dim, cache.page_tokens, int(window), float(scale),
+                None if slopes is None else slopes.data_ptr(), self.attn_workspace.data_ptr(),
                 self.attn_workspace.numel(), 1 if plain else 0, self._stream()))
 
         # Decoded tokens beside prompt portions: one call would send all of them to the kernel for prompt

@@ -20,6 +20,10 @@ class Attention(Part):
 
     A key at ``pk`` is visible to a query at ``pq`` iff ``0 <= pq - pk`` and, when
     ``window > 0``, ``pq - pk < window``.
+
+    A position encoding that enters the scores instead of the queries and keys has an
+    attribute ``score_slopes`` (fp32 on the device, one per query head): the score then is
+    ``dot(q, k) * scale + score_slopes[h] * (pk - pq)``.
     """
     graph_safe = True
 
@@ -80,6 +84,7 @@ class Attention(Part):
         self.position.store(ops, step, qkv, self.H, self.G if write_cache else 0, cache, write_cache)
         att = ops.scratch("att", (T, self.QD), ops.act_dtype)
         with ops.section("attn"):
-            ops.paged_attention(qkv, self.H, self.G, self.D, cache, step, self.window, self.scale, att)
+            ops.paged_attention(qkv, self.H, self.G, self.D, cache, step, self.window, self.scale, att,
+                                slopes=getattr(self.position, "score_slopes", None))
         with ops.section("wo"):
             ops.gemm(att, self.w_o, x, bias=self.b_o, accumulate=True, defer=True)

@@ -340,6 +340,47 @@ def test_paged_attention(ops32, dtype, H, G, D, page, window):
         assert np.max(np.abs(other.float().cpu().numpy() - want)) <= tol
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,G,D,page,window", [(6, 2, 32, 8, 0), (4, 4, 48, 16, 30), (28, 4, 128, 16, 0)])
+def test_paged_attention_with_score_slopes(ops32, dtype, H, G, D, page, window):
+    """The hook for position encodings that enter the scores: slope_h * (j - p) added to the score of key j
+    for the query at p, against attention written out in float64 (also for a shape that would otherwise run on
+    the matrix cores)."""
+    rng = np.random.default_rng(H + D)
+    lengths, q_lens = [1, 77, 300], [1, 40, 2]
+    slopes = (2.0 ** -(1 + 6 * np.arange(H) / H)).astype(np.float32)
+    ks, vs, cache, table = paged_setup(rng, lengths, G, D, page, dtype)
+    qs, positions, slots, wants = [], [], [], []
+    for s, (n, ql) in enumerate(zip(lengths, q_lens)):
+        q_tail = rounded(rng.standard_normal((ql, H, D)).astype(np.float32), dtype).astype(np.float64)
+        k64, v64 = rounded(ks[s], dtype).astype(np.float64), rounded(vs[s], dtype).astype(np.float64)
+        want = np.empty((ql, H, D))
+        for i in range(ql):
+            p = n - ql + i
+            lo = max(0, p - window + 1) if window else 0
+            for h in range(H):
+                sc = k64[lo:p + 1, h // (H // G)] @ q_tail[i, h] / math.sqrt(D) + slopes[h] * (np.arange(lo, p + 1) - p)
+                e = np.exp(sc - sc.max())
+                want[i, h] = (e / e.sum()) @ v64[lo:p + 1, h // (H // G)]
+        qs.append(q_tail)
+        wants.append(want)
+        positions += list(range(n - ql, n))
+        slots += [s] * ql
+    q = np.concatenate(qs).reshape(-1, H * D)
+    want = np.concatenate(wants).reshape(-1, H * D)
+    out = torch.empty((q.shape[0], H * D), dtype=dtype, device="cuda")
+    step = FakeStep(ints(positions), ints(slots), table, None)
+    ops32.paged_attention(dev(q, dtype), H, G, D, cache, step, window, 1.0 / math.sqrt(D), out, slopes=dev(slopes))
+    err = np.max(np.abs(out.float().cpu().numpy() - want))
+    assert err <= (2e-5 if dtype == torch.float32 else 0.02), f"max |diff| {err:.3e}"
+    none = torch.empty_like(out)                                    # and the slopes do matter
+    ops32.paged_attention(dev(q, dtype), H, G, D, cache, step, window, 1.0 / math.sqrt(D), none)
+    assert np.max(np.abs(none.float().cpu().numpy() - want)) > 0.05
+    from hf_cpu_amd.status import EngineError
+    with pytest.raises(EngineError, match="slopes"):
+        ops32.paged_attention(dev(q, dtype), H, G, D, cache, step, window, 1.0 / math.sqrt(D), out, slopes=dev(slopes[:-1]))
+
+
 @pytest.mark.parametrize("H,G,D,page,window,lengths,q_lens", [
     (28, 4, 128, 16, 0, [2100, 700, 64, 1500], [1, 1, 1, 1]),          # decode: keys cut into chunks
     (28, 4, 128, 16, 0, [600], [600]),                                   # one prompt, whole

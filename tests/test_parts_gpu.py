@@ -497,8 +497,9 @@ def test_toy_blocks_with_four_norms_with_parallel_branches_and_without_a_feed_fo
 
 
 def routed_plan_factory():
-    """Registers a toy feed-forward with routing (top-1 of four experts, the router in fp32), a toy
-    position encoding (a learned vector per position added to queries and keys) and an
+    """Registers a toy feed-forward with routing (top-1 of four experts, the router in fp32), two toy
+    position encodings (a learned vector per position added to queries and keys; a slope per head times the
+    distance added to the scores) and an
     architecture that uses them in some layers and the package's parts in others. Nothing in
     the package is edited for this; the toy parts use the package's products and cache store
     and plain tensor arithmetic for the rest."""
@@ -522,6 +523,24 @@ def routed_plan_factory():
             add = self.table[step.positions.long()].to(qkv.dtype)
             for h in range(n_heads + n_kv_heads):              # queries, then keys
                 qkv[:, h * self.head_dim:(h + 1) * self.head_dim] += add
+            if write:
+                ops.rope_store(qkv, step.positions, None, 0, n_heads, n_kv_heads, self.head_dim, cache,
+                               step.group(cache.group).slot_map)
+
+    @register_part("position", "toy_slopes")
+    class ToySlopes(Part):
+        """Queries and keys as they are; the score of key j for the query at p gets slope_h * (j - p) added: an
+        encoding that enters the scores, through the attention part's ``score_slopes`` hook."""
+
+        def __init__(self, head_dim, slopes, prefix=""):
+            super().__init__(prefix)
+            self.head_dim, self.slopes = head_dim, tuple(slopes)
+
+        def bind(self, params, ops):
+            self.score_slopes = hf_cpu_amd.memory.to_device(torch.tensor(self.slopes, dtype=torch.float32), ops.device,
+                                                            "toy slopes")
+
+        def store(self, ops, step, qkv, n_heads, n_kv_heads, cache, write):
             if write:
                 ops.rope_store(qkv, step.positions, None, 0, n_heads, n_kv_heads, self.head_dim, cache,
                                step.group(cache.group).slot_map)
@@ -593,17 +612,23 @@ def routed_plan_factory():
                 norm2=PartSpec("rmsnorm", dict(size=E, eps=1e-6, prefix=pre + "norm2.")), feed_forward=ffn)
         learned = PartSpec("toy_learned", dict(head_dim=16, max_positions=cfg.max_positions, prefix="layers.0.attn."))
         rotary = PartSpec("rotary", dict(head_dim=16, rot_dim=8, theta=100.0))
+        slopes = PartSpec("toy_slopes", dict(head_dim=16, slopes=TOY_SLOPES))
         dense = PartSpec("gated_mlp", dict(hidden_size=E, intermediate_size=40, prefix="layers.0.mlp."))
+        dense2 = PartSpec("gated_mlp", dict(hidden_size=E, intermediate_size=24, prefix="layers.2.mlp."))
         routed = PartSpec("toy_routed", dict(hidden_size=E, intermediate_size=24, n_experts=cfg.n_experts,
                                              prefix="layers.1.moe."))
         return hf_cpu_amd.ModelPlan(
             hidden_size=E, vocab_size=cfg.vocab_size,
             embedding=PartSpec("lookup", dict(vocab_size=cfg.vocab_size, hidden_size=E, prefix="embed.")),
-            layers=(layer(0, attention(0, learned, 0), dense), layer(1, attention(1, rotary, 9), routed)),
-            schedule=(ScheduleEntry(0), ScheduleEntry(1)),
+            layers=(layer(0, attention(0, learned, 0), dense), layer(1, attention(1, rotary, 9), routed),
+                    layer(2, attention(2, slopes, 0), dense2)),
+            schedule=(ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(2)),
             final_norm=PartSpec("rmsnorm", dict(size=E, eps=1e-6, prefix="final.")),
             head=PartSpec("linear", dict(vocab_size=cfg.vocab_size, hidden_size=E, tied=False, prefix="head.")))
     register_architecture("ToyRoutedForCausalLM", RoutedConfig, routed_plan)
+
+
+TOY_SLOPES = (0.5, 0.125, 0.03125)
 
 
 def routed_reference(w, toks, n_experts):
@@ -620,8 +645,15 @@ def routed_reference(w, toks, n_experts):
         if l == 0:
             q = q + w[pre + "pos.weight"][:T, None, :]
             k = k + w[pre + "pos.weight"][:T, None, :]
-        else:
+        elif l == 1:
             q, k = plain.rope(q, range(T), 8, 100.0), plain.rope(k, range(T), 8, 100.0)
+        else:                                                  # scores with slope_h * (j - p), written out
+            att = np.empty_like(q)
+            dist = np.arange(T)[None, :] - np.arange(T)[:, None]
+            for h in range(3):
+                sc = (q[:, h, :] @ k[:, 0, :].T) / 4.0 + TOY_SLOPES[h] * dist
+                att[:, h, :] = plain.softmax(np.where(dist <= 0, sc, -np.inf)) @ v[:, 0, :]
+            return plain.linear(att.reshape(T, 48), w[pre + "o_proj.weight"])
         return plain.linear(plain.attention(q, k, v, window).reshape(T, 48), w[pre + "o_proj.weight"])
     x = x + attn(x, 0, 0)
     x = x + plain.swiglu_mlp(plain.rmsnorm(x, w["layers.0.norm2.weight"], 1e-6), w["layers.0.mlp.gate_proj.weight"],
@@ -636,14 +668,18 @@ def routed_reference(w, toks, n_experts):
         used.add(e)
         mid = np.maximum(w[f"layers.1.moe.experts.{e}.up.weight"] @ h[t], 0.0)
         x[t] = x[t] + prob[t, e] * (w[f"layers.1.moe.experts.{e}.down.weight"] @ mid)
+    x = x + attn(x, 2, 0)
+    x = x + plain.swiglu_mlp(plain.rmsnorm(x, w["layers.2.norm2.weight"], 1e-6), w["layers.2.mlp.gate_proj.weight"],
+                             w["layers.2.mlp.up_proj.weight"], w["layers.2.mlp.down_proj.weight"])
     out = plain.linear(plain.rmsnorm(x, w["final.weight"], 1e-6), w["head.weight"])
     return out, used
 
 
 def test_toy_routed_feed_forward_and_toy_position_encoding(gpu, tmp_path):
-    """Another feed-forward (with routing) and another position encoding, registered from
-    here, in a model whose two layers differ in position encoding, window and feed-forward:
-    whole, in portions and mixed with few pages, against the model written out directly."""
+    """Another feed-forward (with routing) and two other position encodings (one added to queries and
+    keys, one that enters the scores), registered from here, in a model whose three layers differ in
+    position encoding, window and feed-forward: whole, in portions and mixed with few pages, against the
+    model written out directly."""
     routed_plan_factory()
     cfg = {"architectures": ["ToyRoutedForCausalLM"], "vocab_size": 70, "hidden_size": 20, "n_experts": 4,
            "max_positions": 64}
@@ -653,7 +689,7 @@ def test_toy_routed_feed_forward_and_toy_position_encoding(gpu, tmp_path):
         json.dump(cfg, f)
     model = hf_cpu_amd.Model.from_config(hf_cpu_amd.config_from_dict(cfg))
     needs = model.cache_needs()
-    assert [type(n).__name__ for n in needs] == ["PagedKV", "PagedKV"] and (needs[0].window, needs[1].window) == (0, 9)
+    assert [type(n).__name__ for n in needs] == ["PagedKV"] * 3 and [n.window for n in needs] == [0, 9, 0]
     names = {s.name for s in model.param_specs()}
     assert "layers.1.moe.experts.3.down.weight" in names and "layers.0.attn.pos.weight" in names
     rng = np.random.default_rng(5)

@@ -27,6 +27,9 @@
 // way for the same LDS and the products are a little slower than the tiled kernel's, but the few planes make up for
 // it in the kernels that follow (a step of 16 rows 4.28 against 4.40 ms). With four requests (32 rows) a step
 // was slower (5.53 against 5.07 ms): those rows stay with the tiled kernel.
+#include <mutex>
+#include <unordered_map>
+
 #include "common.h"
 #include "gemm_internal.h"
 
@@ -264,10 +267,24 @@ int gemm_wave_slots(const GemmArgs& g, size_t workspace_bytes) {
     const long long nk = g.K / 64, tiles = (g.N + 31) / 32, U = tiles * nk;
     const int G = wave_cu_count() * WAVES;
     if (U < G) return 0;                                     // fewer units than waves: the tiled kernel's splits do as well
-    int slots = 1;
-    for (long long t = 0; t < tiles; t++) {
-        const int n = wave_of_unit(t * nk + nk - 1, U, G) / WAVES - wave_of_unit(t * nk, U, G) / WAVES + 1;
-        if (n > slots) slots = n;
+    // the walk over the tiles is remembered per shape (a decode step asks for the same few shapes every time)
+    static std::mutex lock;
+    static std::unordered_map<unsigned long long, int> known;
+    const unsigned long long key = ((unsigned long long)tiles << 32) | (unsigned long long)nk;
+    int slots = 0;
+    {
+        std::lock_guard<std::mutex> hold(lock);
+        auto it = known.find(key);
+        if (it != known.end()) slots = it->second;
+    }
+    if (slots == 0) {
+        slots = 1;
+        for (long long t = 0; t < tiles; t++) {
+            const int n = wave_of_unit(t * nk + nk - 1, U, G) / WAVES - wave_of_unit(t * nk, U, G) / WAVES + 1;
+            if (n > slots) slots = n;
+        }
+        std::lock_guard<std::mutex> hold(lock);
+        known[key] = slots;
     }
     if (slots > 64 || (size_t)slots * g.M * g.N * sizeof(float) > workspace_bytes) return 0;
     return slots;

@@ -481,6 +481,36 @@ def test_real_layer_sizes_at_the_batch_sizes_with_kernels_of_their_own(gpu, tmp_
         assert all(np.array_equal(again[key], row) for key, row in got.items())
 
 
+def test_real_layer_sizes_at_the_step_sizes_in_between(gpu, tmp_path):
+    """The 7B-shaped layer in bf16 at the step sizes between a handful of decoded tokens and a long prompt: 12
+    requests decoded together (9 to 16 rows: every wave streams by itself, two requests for the activations a
+    unit), prompt portions of 200 and 256 tokens (one row of 256 x 128 tiles, K cut into as many parts as a cost
+    picks) and of 500 (two rows of tiles), and a step that mixes a portion of 150 with the 12 decoded tokens:
+    against the plain implementation on weights rounded to bf16, and the same bits when run again."""
+    import hf_cpu_amd
+    cfg = dict(architectures=["Qwen2ForCausalLM"], num_hidden_layers=1, hidden_size=3584, num_attention_heads=28,
+               num_key_value_heads=4, head_dim=128, intermediate_size=18944, vocab_size=4096, rope_theta=1e6,
+               rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=4096)
+    d = helpers.make_model_dir(str(tmp_path / "m"), cfg, seed=5)
+    reqs = helpers.random_requests(cfg, [200, 756, 150] + [5 + i % 4 for i in range(12)], seed=3)
+    few = [f"r{i}" for i in range(3, 15)]
+    steps = [helpers._step(0, [("r0", reqs["r0"], [0, 100, 199])], ["r0"]),
+             helpers._step(1, [("r1", reqs["r1"][:256], [0, 255])]),
+             helpers._step(2, [("r1", reqs["r1"][256:], [0, 499])], ["r1"]),
+             helpers._step(3, [(r, reqs[r][:-3], []) for r in few])]
+    steps.append(helpers._step(4, [(r, [reqs[r][-3]], [0]) for r in few]))
+    steps.append(helpers._step(5, [("r2", reqs["r2"], [0, 149])] + [(r, [reqs[r][-2]], [0]) for r in few], ["r2"]))
+    steps.append(helpers._step(6, [(r, [reqs[r][-1]], [0]) for r in few], few))
+    want = helpers.plain_logits(d, reqs, round_weights_bf16=True)
+    engine = hf_cpu_amd.load_engine(d, dtype="bfloat16", page_tokens=16, max_tokens=1024 + 13 * 64, max_seqs=13)
+    got = helpers.run_trace_in_engine(engine, steps)
+    worst = helpers.compare(got, want, 2e-2, "7B layer, steps of 12 to 500 tokens")
+    print(f"7B-sized layer, steps of 12 to 500 tokens: worst relative difference {worst:.2e}")
+    assert not engine.manager.held
+    again = helpers.run_trace_in_engine(engine, steps)
+    assert all(np.array_equal(again[key], row) for key, row in got.items())
+
+
 FAMILY = {   # one layer of other members of the family: sizes from their published config.json files
     "0.5B": dict(hidden_size=896, num_attention_heads=14, num_key_value_heads=2, head_dim=64, intermediate_size=4864,
                  tie_word_embeddings=True),

@@ -171,3 +171,126 @@ def test_exponential_of_the_reference():
     rng = np.random.default_rng(0)
     more = (rng.standard_normal(20000) * 20).astype(np.float32)
     assert np.array_equal(hfc_expf(more), np.array([plain.expf(x) for x in more], dtype=np.float32))
+
+
+# ---- the arrangement of a layer (src/model.c:580-636) -----------------------------------------
+# Each case makes all but one path of the layer vanish, so that the logits have a closed form made
+# of parts that the tests above pin. A norm applied to the residual stream as well, a norm after
+# the branch instead of before it, a dropped final norm, a branch that replaces the stream
+# instead of adding to it, rotated values or a missing bias each fail at least one of them.
+
+def _f64(cfg, seed):
+    return {k: v.astype(np.float64) for k, v in helpers.make_weights(cfg, seed).items()}
+
+
+def _head_of(cfg, w, x):
+    head = w["lm_head.weight"] if "lm_head.weight" in w else w["model.embed_tokens.weight"]
+    return plain.linear(plain.rmsnorm(x, w["model.norm.weight"], cfg["rms_norm_eps"]), head)
+
+
+def _silence(w, cfg, keep=None):
+    """o_proj = down_proj = 0 in every layer but ``keep``: those layers add nothing to the stream."""
+    w = dict(w)
+    for l in range(cfg["num_hidden_layers"]):
+        if l != keep:
+            w[f"model.layers.{l}.self_attn.o_proj.weight"] = np.zeros_like(w[f"model.layers.{l}.self_attn.o_proj.weight"])
+            w[f"model.layers.{l}.mlp.down_proj.weight"] = np.zeros_like(w[f"model.layers.{l}.mlp.down_proj.weight"])
+    return w
+
+
+def test_layers_that_add_nothing_leave_head_of_norm_of_embedding():
+    """o_proj = down_proj = 0 everywhere: logits = head(norm(embed(tokens))) exactly (src/model.c:609, 623
+    add zeros; src/model.c:629-636). Fails if the final norm is missing, if a layer's norm also
+    replaces the stream, or if the stream is overwritten by a branch."""
+    for name, cfg in helpers.CONFIGS.items():
+        w = _silence(_f64(cfg, 11), cfg)
+        toks = helpers.random_requests(cfg, [9], 2)["r0"]
+        want = _head_of(cfg, w, plain.embed(w["model.embed_tokens.weight"], toks))
+        assert np.array_equal(plain.forward(cfg, w, toks), want), name
+        assert np.max(np.abs(want)) > 1e-3
+
+
+def test_a_zero_input_norm_leaves_the_biases_and_the_unnormed_stream():
+    """input_layernorm.weight = 0 in layer l: its attention sees h = 0, so q = bq, k = bk, v = bv at every
+    position; every visible value is bv, so the attention output is bv of the query head's key/value head
+    h // (H / G), and the stream grows by Wo times that, at every position alike (src/model.c:580-609).
+    With that layer's down_proj = 0 and the other layers silent, logits = head(norm(embed + Wo rep(bv))).
+    Fails if the norm sits behind the branch or on the stream, if values are rotated (bv would turn
+    with the position), if a bias is dropped, or if heads are grouped by h % G."""
+    for name, cfg in helpers.CONFIGS.items():
+        H, G, D = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+        for l in range(cfg["num_hidden_layers"]):
+            w = _silence(_f64(cfg, 12), cfg, keep=l)
+            p = f"model.layers.{l}."
+            w[p + "input_layernorm.weight"] = np.zeros(cfg["hidden_size"])
+            w[p + "mlp.down_proj.weight"] = np.zeros_like(w[p + "mlp.down_proj.weight"])
+            toks = helpers.random_requests(cfg, [40], 3)["r0"]            # beyond B's window of 32
+            bv = w[p + "self_attn.v_proj.bias"].reshape(G, D)
+            rep = np.concatenate([bv[h // (H // G)] for h in range(H)])
+            add = w[p + "self_attn.o_proj.weight"] @ rep
+            want = _head_of(cfg, w, plain.embed(w["model.embed_tokens.weight"], toks) + add[None, :])
+            got = plain.forward(cfg, w, toks, first_position=3)
+            assert np.allclose(got, want, rtol=0, atol=1e-11), (name, l)
+            assert np.max(np.abs(add)) > 1e-2
+            # the attention block alone, given h = 0
+            block = plain.attention_block(cfg, w, l, np.zeros((5, cfg["hidden_size"])), np.arange(4, 9))
+            assert np.allclose(block, np.tile(add, (5, 1)), rtol=0, atol=1e-12)
+
+
+def test_a_zero_post_attention_norm_silences_the_feed_forward():
+    """post_attention_layernorm.weight = 0: the feed-forward sees 0 and adds Wdown (silu(0) * 0) = 0
+    (src/model.c:611-623), so the logits are those of the model with that layer's down_proj = 0. Fails if
+    the feed-forward reads the stream without its norm, or the norm of the other branch."""
+    cfg = helpers.CONFIG_B
+    w = _f64(cfg, 13)
+    toks = helpers.random_requests(cfg, [21], 4)["r0"]
+    for l in range(cfg["num_hidden_layers"]):
+        p = f"model.layers.{l}."
+        a = dict(w, **{p + "post_attention_layernorm.weight": np.zeros(cfg["hidden_size"])})
+        b = dict(w, **{p + "mlp.down_proj.weight": np.zeros_like(w[p + "mlp.down_proj.weight"])})
+        full = plain.forward(cfg, w, toks)
+        assert np.array_equal(plain.forward(cfg, a, toks), plain.forward(cfg, b, toks))
+        assert np.max(np.abs(full - plain.forward(cfg, b, toks))) > 1e-3
+
+
+def test_one_layer_with_one_branch_is_that_branch_on_the_normed_stream():
+    """One layer alive. With its o_proj = 0: logits = head(norm(e + mlp(norm2(e)))) (the feed-forward reads
+    the norm of the stream as the attention left it, and adds to the un-normed stream). With its down_proj = 0
+    and a single token: attention over one key returns its value, so logits = head(norm(e + Wo rep(Wv norm1(e) + bv)))."""
+    for name, cfg in helpers.CONFIGS.items():
+        H, G, D = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+        eps = cfg["rms_norm_eps"]
+        l = cfg["num_hidden_layers"] - 1
+        p = f"model.layers.{l}."
+        base = _silence(_f64(cfg, 14), cfg, keep=l)
+        toks = helpers.random_requests(cfg, [6], 5)["r0"]
+        e = plain.embed(base["model.embed_tokens.weight"], toks)
+        w = dict(base, **{p + "self_attn.o_proj.weight": np.zeros_like(base[p + "self_attn.o_proj.weight"])})
+        mlp = plain.swiglu_mlp(plain.rmsnorm(e, w[p + "post_attention_layernorm.weight"], eps),
+                               w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+        assert np.allclose(plain.forward(cfg, w, toks), _head_of(cfg, w, e + mlp), rtol=0, atol=1e-11), name
+        w = dict(base, **{p + "mlp.down_proj.weight": np.zeros_like(base[p + "mlp.down_proj.weight"])})
+        for pos in (0, 7):                                      # one token: the output is its own value, not rotated
+            h1 = plain.rmsnorm(e[:1], w[p + "input_layernorm.weight"], eps)
+            v = plain.linear(h1, w[p + "self_attn.v_proj.weight"], w[p + "self_attn.v_proj.bias"]).reshape(G, D)
+            rep = np.concatenate([v[h // (H // G)] for h in range(H)])
+            want = _head_of(cfg, w, e[:1] + (w[p + "self_attn.o_proj.weight"] @ rep)[None, :])
+            assert np.allclose(plain.forward(cfg, w, toks[:1], first_position=pos), want, rtol=0, atol=1e-11), (name, pos)
+        # both branches alive, one token: the feed-forward reads the stream as the attention left it
+        w = base
+        h1 = plain.rmsnorm(e[:1], w[p + "input_layernorm.weight"], eps)
+        v = plain.linear(h1, w[p + "self_attn.v_proj.weight"], w[p + "self_attn.v_proj.bias"]).reshape(G, D)
+        x1 = e[:1] + (w[p + "self_attn.o_proj.weight"] @ np.concatenate([v[h // (H // G)] for h in range(H)]))[None, :]
+        x2 = x1 + plain.swiglu_mlp(plain.rmsnorm(x1, w[p + "post_attention_layernorm.weight"], eps),
+                                   w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+        assert np.allclose(plain.forward(cfg, w, toks[:1], first_position=3), _head_of(cfg, w, x2), rtol=0, atol=1e-11), name
+
+
+def test_positions_enter_only_through_distances():
+    """A shift of all positions changes nothing (rotary encodes distances; values and the stream carry no
+    position): the logits of a sequence that starts at position 1000 are those of one that starts at 0."""
+    for name, cfg in helpers.CONFIGS.items():
+        w = _f64(cfg, 15)
+        toks = helpers.random_requests(cfg, [45], 6)["r0"]
+        a, b = plain.forward(cfg, w, toks), plain.forward(cfg, w, toks, first_position=1000)
+        assert np.max(np.abs(a - b)) < 1e-8 * np.max(np.abs(a)), name

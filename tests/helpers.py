@@ -75,6 +75,8 @@ def write_safetensors(path, tensors, dtype="F32"):
         a = np.ascontiguousarray(a, dtype=np.float32)
         if dtype == "BF16":
             raw = (bf16_round(a).view(np.uint32) >> 16).astype("<u2").tobytes()
+        elif dtype == "F16":
+            raw = a.astype("<f2").tobytes()
         else:
             raw = a.astype("<f4").tobytes()
         header[name] = {"dtype": dtype, "shape": list(a.shape), "data_offsets": [off, off + len(raw)]}

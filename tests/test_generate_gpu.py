@@ -364,6 +364,54 @@ def test_generation_survives_a_cache_that_is_too_small(gpu, models):
     assert not tiny.engine.manager.held
 
 
+@pytest.mark.parametrize("name,dtype,temp", [("A", "float32", 0.0), ("B", "float32", 0.8), ("B", "bfloat16", 0.0)])
+def test_end_of_sequence_tokens_that_the_host_learns_a_step_late(gpu, models, name, dtype, temp):
+    """Ten requests, greedy or sampled, with end-of-sequence ids chosen so that several of them end by one at
+    different steps, in a cache too small for all of them: the host enqueues a step before it has read the
+    last one's tokens, so a request that drew an end-of-sequence token runs one step more into its own page,
+    and its pages go back while the next step is already enqueued (src/ops.c:849: the token is neither
+    reported nor fed). Every request ends with what it gives alone, cut before its first end-of-sequence
+    token, and the books balance."""
+    import hf_cpu_amd.session as S
+    from hf_cpu_amd.engine.scheduler import Request
+    from hf_cpu_amd.sampling import SamplerParams
+    cfg = helpers.CONFIGS[name]
+    P = helpers.PAGE[name]
+    rng = np.random.default_rng(17)
+    prompts = [[int(t) for t in rng.integers(0, cfg["vocab_size"], int(rng.integers(2, 40)))] for _ in range(10)]
+    new = 26
+    roomy = S.Session(models[name], dtype=dtype, ctx_max=128, batch=32, page_size=P, max_seqs=10)
+    free = [roomy.generate(p, temp=temp, seed=7 + i, max_tokens=new, eos_ids=())[0].tokens for i, p in enumerate(prompts)]
+    assert all(len(t) == new for t in free)
+    eos = {free[4][0]}
+    for i, at in ((0, 3), (1, 9), (2, 15), (3, 20)):          # a token that request i draws for the first time at step >= at
+        eos.add(next((t for j, t in enumerate(free[i]) if j >= at and t not in free[i][:j]), free[i][at]))
+    want, stops = [], []
+    for t in free:
+        cut = next((j for j, tok in enumerate(t) if tok in eos), None)
+        want.append(t if cut is None else t[:cut])
+        stops.append("length" if cut is None else "eos")
+    ends = {len(w) for w, s in zip(want, stops) if s == "eos"}
+    assert len(ends) >= 3 and max(ends) >= 8 and 0 in ends, ends            # ends at different steps, one at the first token
+    tight = S.Session(models[name], dtype=dtype, ctx_max=128, batch=32, page_size=P, max_seqs=10,
+                      kv_tokens=5 * 64)
+    sched = tight.scheduler()
+    reqs = [Request(i, list(p), SamplerParams(temp, 40, 0.95, 0.05), new, 7 + i, eos_ids=tuple(eos)) for i, p in enumerate(prompts)]
+    for r in reqs:
+        sched.submit(r)
+    sched.run()
+    assert sched.steps_ahead > 0
+    for i, r in enumerate(reqs):
+        assert r.error is None and r.stop == stops[i] and r.generated == want[i], \
+            f"request {i}: stop {r.stop} (want {stops[i]}), {len(r.generated)} tokens (want {len(want[i])})"
+    mgr = tight.engine.manager
+    mgr.check()
+    assert not mgr.held and all(p.n_held == 0 for p in mgr.pools) and mgr.pools[0].reused > 0
+    # and through the entry point, where the ids come as an argument
+    gens = tight.generate(prompts[:4], temp=temp, seed=7, max_tokens=new, eos_ids=sorted(eos))
+    assert gens[0].tokens == want[0] and gens[0].stop == stops[0]
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_twenty_requests_together_give_what_each_gives_alone(gpu, models, dtype):
     """More requests at once than the engine decodes without filling a step up (above 8 rows a
@@ -509,6 +557,46 @@ def test_real_layer_sizes_at_the_step_sizes_in_between(gpu, tmp_path):
     assert not engine.manager.held
     again = helpers.run_trace_in_engine(engine, steps)
     assert all(np.array_equal(again[key], row) for key, row in got.items())
+
+
+def test_real_layer_sizes_with_pages_of_64_tokens(gpu, tmp_path):
+    """The 7B-shaped layer in bf16 with the reference's page of 64 tokens (src/model.h:56): a block of 32 keys is
+    half a page, which the attention kernel for prompt portions addresses by other code than pages of up to
+    32. Three requests mixed (portions of some beside decoded tokens of others, two live at a time in a pool
+    that makes pages come back), and each with its tail decoded, against the plain implementation on weights
+    rounded to bf16."""
+    import hf_cpu_amd
+    cfg = dict(architectures=["Qwen2ForCausalLM"], num_hidden_layers=1, hidden_size=3584, num_attention_heads=28,
+               num_key_value_heads=4, head_dim=128, intermediate_size=18944, vocab_size=4096, rope_theta=1e6,
+               rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=512)
+    d = helpers.make_model_dir(str(tmp_path / "m"), cfg, seed=6)
+    reqs = helpers.random_requests(cfg, [150, 211, 97], seed=4)
+    want = helpers.plain_logits(d, reqs, round_weights_bf16=True)
+    for name, steps in (("mixed", helpers.trace_mixed(reqs, seed=9, max_live=2, decode_tail=6)),
+                        ("tail", helpers.trace_tail(reqs, tail=8)),
+                        ("whole", helpers.trace_whole(reqs))):
+        engine = hf_cpu_amd.load_engine(d, dtype="bfloat16", page_tokens=64, max_tokens=helpers.max_live_tokens(steps, 64),
+                                        max_seqs=2)
+        worst = helpers.compare(helpers.run_trace_in_engine(engine, steps), want, 2e-2, f"7B layer, pages of 64, {name}")
+        print(f"7B-sized layer, pages of 64 tokens, {name}: worst relative difference {worst:.2e}")
+        engine.manager.check()
+        assert not engine.manager.held
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", 1e-5), ("bfloat16", 2e-2)])
+def test_a_checkpoint_stored_in_half_precision(gpu, tmp_path, dtype, tol):
+    """A model folder whose tensors are stored as F16: the loader widens them (to fp32 for the 32-bit engine,
+    to bf16 after fp32 for the bf16 engine); against the plain implementation, which reads the same file with
+    its own reader."""
+    import hf_cpu_amd
+    cfg = helpers.CONFIG_B
+    d = helpers.make_model_dir(str(tmp_path / "m"), cfg, seed=8, dtype="F16")
+    reqs = helpers.random_requests(cfg, [50, 23], seed=2)
+    steps = helpers.trace_mixed(reqs, seed=1, max_live=2, decode_tail=5)
+    want = helpers.plain_logits(d, reqs, round_weights_bf16=dtype == "bfloat16")
+    engine = hf_cpu_amd.load_engine(d, dtype=dtype, page_tokens=8, max_tokens=128, max_seqs=2)
+    worst = helpers.compare(helpers.run_trace_in_engine(engine, steps), want, tol, f"F16 checkpoint, {dtype}")
+    print(f"F16 checkpoint, {dtype}: worst relative difference {worst:.2e}")
 
 
 FAMILY = {   # one layer of other members of the family: sizes from their published config.json files

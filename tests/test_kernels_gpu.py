@@ -392,6 +392,14 @@ def test_paged_attention_with_score_slopes(ops32, dtype, H, G, D, page, window):
     (6, 2, 96, 32, 0, [300], [37]),                                      # pages of 32 tokens
     (28, 4, 128, 16, 0, [1200], [1200]),                                 # one prompt whose 300 blocks are all resident: long tiles beside short ones
     (28, 4, 128, 16, 0, [1100], [1000]),                                 # the same for a portion late in a prompt
+    # pages of more than 32 tokens: a block of 32 keys is part of a page, and the prompt kernel addresses them otherwise
+    (28, 4, 128, 64, 0, [2100, 700, 64, 1500], [1, 1, 1, 1]),
+    (28, 4, 128, 128, 0, [600], [600]),
+    (14, 2, 64, 64, 300, [1000, 333], [1, 40]),                          # the window begins inside a page
+    (12, 4, 64, 128, 50, [400, 130], [130, 130]),
+    (28, 4, 128, 64, 0, [700, 90, 333, 64], [100, 90, 17, 1]),
+    (8, 1, 96, 128, 81, [657, 31], [9, 31]),
+    (28, 4, 128, 128, 0, [1100], [1000]),
 ])
 def test_paged_attention_on_matrix_cores(ops16, H, G, D, page, window, lengths, q_lens):
     """bf16 with head_dim a multiple of 32: long contexts (many key blocks, split into chunks when
@@ -419,15 +427,16 @@ def test_paged_attention_on_matrix_cores(ops16, H, G, D, page, window, lengths, 
     assert err <= 0.02, f"max |diff| {err:.3e}"
 
 
-def tail_attention(q_tail, k, v, window):
+def tail_attention(q_tail, k, v, window, rows=None):
     """Attention of the last queries of a sequence only (float64): q_tail [ql, H, D] stands at
     positions n-ql .. n-1 of k, v [n, G, D]; key j is visible to position p iff j <= p and,
-    with a window W, p - j < W. The mask is built per query, so that long sequences stay cheap."""
+    with a window W, p - j < W. The mask is built per query, so that long sequences stay cheap.
+    ``rows``: only these queries are computed (the others stay zero)."""
     ql, H, D = q_tail.shape
     n, G, _ = k.shape
-    out = np.empty((ql, H, D))
+    out = np.zeros((ql, H, D))
     k64, v64 = k.astype(np.float64), v.astype(np.float64)
-    for i in range(ql):
+    for i in (range(ql) if rows is None else rows):
         p = n - ql + i
         lo = max(0, p - window + 1) if window else 0
         for h in range(H):
@@ -482,6 +491,53 @@ def test_paged_attention_long_contexts(ops16, H, G, D, page, window, lengths, q_
     finally:
         ops16.force_plain_attention = False
     assert np.max(np.abs(other.float().cpu().numpy() - want)) <= 0.02
+
+
+@pytest.mark.parametrize("H,G,D,page,window,n,ql,cut", [
+    (8, 2, 64, 64, 0, 40000, 1, False),          # a decoded token whose one walk needs two windows of page ids
+    (8, 2, 64, 128, 0, 70000, 1, False),
+    (4, 4, 32, 64, 0, 40000, 900, False),        # a portion late in a prompt, every block walking all its keys
+    (4, 4, 32, 128, 0, 70000, 900, False),
+    (4, 2, 32, 64, 36000, 76109, 3, False),      # the window's first key lies inside a page: one page more than the keys fill
+    (4, 4, 32, 64, 36000, 76941, 900, False),
+    (8, 2, 64, 64, 0, 40000, 1, True),           # the same contexts with the keys cut into chunks
+    (4, 4, 32, 128, 0, 70000, 900, True),
+    (4, 2, 32, 64, 36000, 76109, 3, True),
+])
+def test_paged_attention_large_pages_long_walks(ops16, H, G, D, page, window, n, ql, cut):
+    """Pages of 64 and 128 tokens with more keys in one walk than one window of page ids covers (511 pages
+    when a walk may begin inside a page). Without ``cut`` the attention workspace is too small for partial
+    results, so the kernels do not cut the keys into chunks and one wave (or block) walks them all. A far
+    key in the first window and one in the second are made to matter."""
+    rng = np.random.default_rng(H + D + page + n)
+    dtype = torch.bfloat16
+    ks, vs, cache, table = paged_setup(rng, [n], G, D, page, dtype)
+    q_tail = rng.standard_normal((ql, H, D)).astype(np.float32)
+    lo = max(0, n - ql - window + 1) if window else 0
+    if window:
+        assert (lo // 32 * 32) % page >= 32                       # the walk begins inside a page
+    assert n - ql - lo > 511 * page
+    kc = cache.k.float().cpu().numpy()
+    for j, (far, score) in enumerate(((lo + 300, 12.0), (lo + 511 * page + 700, 13.0))):
+        ks[0][far, 0] = score * math.sqrt(D) * q_tail[j % ql, 0] / np.dot(q_tail[j % ql, 0], q_tail[j % ql, 0])
+        kc[int(table[0, far // page].item()) * page + far % page, :D] = ks[0][far, 0]
+    cache = FakeCache(group=0, k=dev(kc, dtype), v=cache.v, page_tokens=page, window=0)
+    rows = sorted({0, 1, ql // 2, ql - 2, ql - 1} & set(range(ql)))
+    want = tail_attention(rounded(q_tail, dtype), rounded(ks[0], dtype), rounded(vs[0], dtype), window, rows)[rows]
+    q = dev(q_tail.reshape(ql, H * D), dtype)
+    out = torch.empty((ql, H * D), dtype=dtype, device="cuda")
+    step = FakeStep(ints(list(range(n - ql, n))), ints([0] * ql), table, None)
+    whole = ops16.attn_workspace
+    if not cut:
+        ops16.attn_workspace = whole[:256]
+    try:
+        ops16.paged_attention(q, H, G, D, cache, step, window, 1.0 / math.sqrt(D), out)
+    finally:
+        ops16.attn_workspace = whole
+    got = out.float().cpu().numpy().reshape(ql, H, D)[rows]
+    err = np.max(np.abs(got - want))
+    assert err <= 0.02, f"max |diff| {err:.3e}"
+    assert np.max(np.abs(want[0, 0])) > 0.3                        # the far keys carry weight
 
 
 def test_attention_special_cases(ops32):

@@ -52,11 +52,8 @@ class Cli:
             return self.session
         self.session = None
         so = self.opts
-        over = None
-        if eff["window"] is not None:               # the window of config.json replaced (0: no window)
-            over = {"use_sliding_window": eff["window"] > 0}
-            if eff["window"] > 0:
-                over["sliding_window"] = eff["window"]
+        # the window of config.json replaced (0: no window); the architecture's configuration class knows its keys
+        over = None if eff["window"] is None else {"window": eff["window"]}
         if eff["random-weights"] is not None:
             from ..config import read_config
             model, seed = read_config(path, over), eff["random-weights"]
@@ -64,7 +61,7 @@ class Cli:
             model, seed = path, 0
         t0 = time.monotonic()
         s = Session(model, dtype=so["dtype"], ctx_max=so["ctx-max"], batch=so["batch"], page_size=so["page-size"],
-                    max_seqs=so["max-seqs"], kv_tokens=so["kv-tokens"] or None, seed=seed, config_overrides=over)
+                    max_seqs=so["max-seqs"], kv_tokens=so["kv-tokens"] or None, seed=seed, model_options=over)
         s.cli_identity = ident
         self.log("info", f"model={path} dtype={so['dtype']} load_ms={(time.monotonic() - t0) * 1e3:.0f} "
                          f"kv_bytes={s.engine.storage.nbytes()}")

@@ -62,6 +62,23 @@ class Qwen2Config:
             d["sliding_window"] = None
         return d
 
+    # ---- model options of a session ---------------------------------------
+    @classmethod
+    def apply_options(cls, obj, options):
+        """``obj`` (config.json's object) with the options a session gives in the engine's own words.
+        ``window`` = N replaces the file's window for the layers that may have one
+        (``use_sliding_window``, ``sliding_window``); 0 turns it off."""
+        obj = dict(obj)
+        for name, value in options.items():
+            if name == "window":
+                obj["use_sliding_window"] = int(value) > 0
+                if int(value) > 0:
+                    obj["sliding_window"] = int(value)
+                    obj.pop("layer_types", None)     # spelled from max_window_layers again when read
+            else:
+                fail(ENOTSUP, f"architecture '{(obj.get('architectures') or ['?'])[0]}' has no model option '{name}'")
+        return obj
+
     # ---- reading -------------------------------------------------------
     @classmethod
     def from_dict(cls, obj, origin="config.json"):

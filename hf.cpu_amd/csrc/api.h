@@ -41,14 +41,16 @@ int hfa_gemm_finish(const void* partial, int splits, const float* bias, void* ou
 // Rotary position encoding on the q (and k) heads inside qkv rows [q | k | v], split-half
 // pairing, and the store of k (rotated) and v into cache rows slot_map[t] (src/model.c:468-493,
 // 587-600). rot_dim 0: no rotation. n_kv_heads 0: the rows hold q only, nothing is stored.
-// Cache layout: row r = page * page_tokens + offset. Keys: k_cache[r * width + c]. Values lie
-// transposed inside their page, so that the keys of one value column are contiguous:
-// v_cache[page * page_tokens * width + c * page_tokens + offset].
+// Query and key heads have head_dim values, value heads v_head_dim (the same in most models; a
+// prompt-sized bf16 call with equal sizes takes a kernel of its own).
+// Cache layout: row r = page * page_tokens + offset. Keys: k_cache[r * width + c], width =
+// n_kv_heads * head_dim. Values (width n_kv_heads * v_head_dim) lie transposed inside their page, so that
+// the keys of one value column are contiguous: v_cache[page * page_tokens * width + c * page_tokens + offset].
 // With splits > 0 the input is not qkv but the partial sums of a deferred hfa_gemm
 // ([splits][n_tokens][(n_heads + 2 n_kv_heads) * head_dim] fp32) plus partial_bias; the rotated
 // queries are written into qkv.
 int hfa_rope_store(void* qkv, int dtype, int ld, const int* positions, const float* inv_freq, int rot_dim,
-                   int n_heads, int n_kv_heads, int head_dim, void* k_cache, void* v_cache,
+                   int n_heads, int n_kv_heads, int head_dim, int v_head_dim, void* k_cache, void* v_cache,
                    const int* slot_map, int page_tokens, int n_tokens, const float* partial, int splits,
                    const float* partial_bias, hipStream_t stream);
 
@@ -61,16 +63,18 @@ int hfa_attention_prompt_rows(void);
 // block_table[s, j / page_tokens] * page_tokens + j % page_tokens. A key is visible to the
 // query at position p iff j <= p and (window == 0 or p - j < window). q_start[n_seqs + 1] gives
 // each request's run of tokens (consecutive positions of one slot); max_q_len and max_seq_len
-// bound the runs and the positions. bf16 with head_dim a multiple of 32, page_tokens a multiple
-// of 4 and at most 32 query heads per key/value head runs on the matrix cores, the key range
+// bound the runs and the positions. Key rows are kv_width wide with head_dim values a head, value rows
+// v_width with v_head_dim a head; out has v_head_dim values per query head. bf16 with one head size for
+// both that is a multiple of 32, page_tokens a power of two from 4
+// and at most 32 query heads per key/value head runs on the matrix cores, the key range
 // split over `workspace` when there are few queries; everything else, and everything when
 // `force_plain`, runs the plain kernel. `slopes` (one fp32 per query head, or null) is the hook for a position
 // encoding that enters the scores rather than the queries and keys: the score of key j for the query at p
 // becomes dot * scale + slopes[h] * (j - p); with slopes the plain kernel runs.
 int hfa_paged_attention(const void* q, int dtype, int ldq, const void* k_cache, const void* v_cache,
-                        int kv_width, const int* block_table, int max_blocks, const int* token_slot,
+                        int kv_width, int v_width, const int* block_table, int max_blocks, const int* token_slot,
                         const int* positions, const int* q_start, int n_seqs, int max_q_len, int max_seq_len,
-                        void* out, int ldo, int n_tokens, int n_heads, int n_kv_heads, int head_dim,
+                        void* out, int ldo, int n_tokens, int n_heads, int n_kv_heads, int head_dim, int v_head_dim,
                         int page_tokens, int window, float scale, const float* slopes, void* workspace,
                         size_t workspace_bytes, int force_plain, hipStream_t stream);
 

@@ -44,9 +44,9 @@ __device__ __forceinline__ float dot_row(const float* __restrict__ q_s, const fl
 
 template <typename T>
 __global__ __launch_bounds__(WAVE) void attn_generic_kernel(
-    const T* __restrict__ q, int ldq, const T* __restrict__ kc, const T* __restrict__ vc, int kvw,
+    const T* __restrict__ q, int ldq, const T* __restrict__ kc, const T* __restrict__ vc, int kvw, int vw,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ token_slot,
-    const int* __restrict__ positions, T* __restrict__ out, int ldo, int H, int G, int D, int page_tokens,
+    const int* __restrict__ positions, T* __restrict__ out, int ldo, int H, int G, int D, int Dv, int page_tokens,
     int window, float scale, const float* __restrict__ slopes) {
     __shared__ float q_s[ATT_MAX_D];
     __shared__ float p_s[WAVE];
@@ -91,12 +91,12 @@ __global__ __launch_bounds__(WAVE) void attn_generic_kernel(
             const float pj = p_s[jj];
             // values lie transposed inside their page: [page][column][token]
             const int vr = row_s[jj];
-            const T* vp = vc + (size_t)(vr / page_tokens) * page_tokens * kvw + (size_t)(kvh * D) * page_tokens +
+            const T* vp = vc + (size_t)(vr / page_tokens) * page_tokens * vw + (size_t)(kvh * Dv) * page_tokens +
                           vr % page_tokens;
 #pragma unroll
             for (int i = 0; i < ATT_MAX_D / WAVE; i++) {
                 const int d = lane + WAVE * i;
-                if (d < D) acc[i] = fmaf(pj, to_f32(vp[(size_t)d * page_tokens]), acc[i]);
+                if (d < Dv) acc[i] = fmaf(pj, to_f32(vp[(size_t)d * page_tokens]), acc[i]);
             }
         }
         __syncthreads();
@@ -105,41 +105,42 @@ __global__ __launch_bounds__(WAVE) void attn_generic_kernel(
 #pragma unroll
     for (int i = 0; i < ATT_MAX_D / WAVE; i++) {
         const int d = lane + WAVE * i;
-        if (d < D) out[(size_t)t * ldo + h * D + d] = from_f32<T>(acc[i] * inv);
+        if (d < Dv) out[(size_t)t * ldo + h * Dv + d] = from_f32<T>(acc[i] * inv);
     }
 }
 
 int attn_generic_launch(const void* q, int dtype, int ldq, const void* k_cache, const void* v_cache, int kv_width,
-                        const int* block_table, int max_blocks, const int* token_slot, const int* positions,
-                        void* out, int ldo, int n_tokens, int n_heads, int n_kv_heads, int head_dim,
+                        int v_width, const int* block_table, int max_blocks, const int* token_slot, const int* positions,
+                        void* out, int ldo, int n_tokens, int n_heads, int n_kv_heads, int head_dim, int v_head_dim,
                         int page_tokens, int window, float scale, const float* slopes, hipStream_t stream) {
-    HFA_REQUIRE(head_dim <= ATT_MAX_D, "paged_attention: head_dim %d exceeds the kernel's limit %d", head_dim,
-                ATT_MAX_D);
+    HFA_REQUIRE(head_dim <= ATT_MAX_D && v_head_dim <= ATT_MAX_D, "paged_attention: head_dim %d (values: %d) exceeds the kernel's limit %d",
+                head_dim, v_head_dim, ATT_MAX_D);
     HFA_REQUIRE(n_heads <= 65535, "paged_attention: %d heads exceed the grid", n_heads);
     dim3 grid(n_tokens, n_heads);
     if (dtype == HFA_F32)
         attn_generic_kernel<float><<<grid, WAVE, 0, stream>>>(
-            (const float*)q, ldq, (const float*)k_cache, (const float*)v_cache, kv_width, block_table, max_blocks,
-            token_slot, positions, (float*)out, ldo, n_heads, n_kv_heads, head_dim, page_tokens, window, scale, slopes);
+            (const float*)q, ldq, (const float*)k_cache, (const float*)v_cache, kv_width, v_width, block_table, max_blocks,
+            token_slot, positions, (float*)out, ldo, n_heads, n_kv_heads, head_dim, v_head_dim, page_tokens, window, scale, slopes);
     else
         attn_generic_kernel<bf16><<<grid, WAVE, 0, stream>>>(
-            (const bf16*)q, ldq, (const bf16*)k_cache, (const bf16*)v_cache, kv_width, block_table, max_blocks,
-            token_slot, positions, (bf16*)out, ldo, n_heads, n_kv_heads, head_dim, page_tokens, window, scale, slopes);
+            (const bf16*)q, ldq, (const bf16*)k_cache, (const bf16*)v_cache, kv_width, v_width, block_table, max_blocks,
+            token_slot, positions, (bf16*)out, ldo, n_heads, n_kv_heads, head_dim, v_head_dim, page_tokens, window, scale, slopes);
     HFA_LAUNCH_CHECK("paged_attention");
     return 0;
 }
 
 extern "C" int hfa_paged_attention(const void* q, int dtype, int ldq, const void* k_cache, const void* v_cache,
-                                   int kv_width, const int* block_table, int max_blocks, const int* token_slot,
+                                   int kv_width, int v_width, const int* block_table, int max_blocks, const int* token_slot,
                                    const int* positions, const int* q_start, int n_seqs, int max_q_len,
                                    int max_seq_len, void* out, int ldo, int n_tokens, int n_heads, int n_kv_heads,
-                                   int head_dim, int page_tokens, int window, float scale, const float* slopes,
+                                   int head_dim, int v_head_dim, int page_tokens, int window, float scale, const float* slopes,
                                    void* workspace, size_t workspace_bytes, int force_plain, hipStream_t stream) {
-    HFA_REQUIRE(n_tokens > 0 && n_heads > 0 && n_kv_heads > 0 && head_dim > 0 && page_tokens > 0 && max_blocks > 0,
+    HFA_REQUIRE(n_tokens > 0 && n_heads > 0 && n_kv_heads > 0 && head_dim > 0 && v_head_dim > 0 && page_tokens > 0 && max_blocks > 0,
                 "paged_attention: bad sizes");
     HFA_REQUIRE(n_heads % n_kv_heads == 0, "paged_attention: %d heads are not a multiple of %d key/value heads",
                 n_heads, n_kv_heads);
-    HFA_REQUIRE(kv_width >= n_kv_heads * head_dim && ldq >= n_heads * head_dim && ldo >= n_heads * head_dim,
+    HFA_REQUIRE(kv_width >= n_kv_heads * head_dim && v_width >= n_kv_heads * v_head_dim && ldq >= n_heads * head_dim &&
+                    ldo >= n_heads * v_head_dim,
                 "paged_attention: a row stride is smaller than its row");
     HFA_REQUIRE(window >= 0, "paged_attention: negative window");
     HFA_REQUIRE(dtype == HFA_F32 || dtype == HFA_BF16, "paged_attention: unknown dtype %d", dtype);
@@ -147,8 +148,10 @@ extern "C" int hfa_paged_attention(const void* q, int dtype, int ldq, const void
                   n_seqs, max_q_len, max_seq_len, out, ldo, n_tokens, n_heads, n_kv_heads, head_dim, page_tokens,
                   window, scale, workspace, workspace_bytes, stream};
     // the matrix-core kernels take no slopes: scores with a position term go the plain way
-    if (!force_plain && !slopes && dtype == HFA_BF16 && attn_mfma_supports(a)) return attn_mfma_launch(a);
-    return attn_generic_launch(q, dtype, ldq, k_cache, v_cache, kv_width, block_table, max_blocks, token_slot,
-                               positions, out, ldo, n_tokens, n_heads, n_kv_heads, head_dim, page_tokens, window,
+    // and they know one head size and one row width for keys and values
+    if (!force_plain && !slopes && dtype == HFA_BF16 && v_head_dim == head_dim && v_width == kv_width && attn_mfma_supports(a))
+        return attn_mfma_launch(a);
+    return attn_generic_launch(q, dtype, ldq, k_cache, v_cache, kv_width, v_width, block_table, max_blocks, token_slot,
+                               positions, out, ldo, n_tokens, n_heads, n_kv_heads, head_dim, v_head_dim, page_tokens, window,
                                scale, slopes, stream);
 }

@@ -16,8 +16,8 @@ struct AttnArgs {
 };
 
 int attn_generic_launch(const void* q, int dtype, int ldq, const void* k_cache, const void* v_cache, int kv_width,
-                        const int* block_table, int max_blocks, const int* token_slot, const int* positions,
-                        void* out, int ldo, int n_tokens, int n_heads, int n_kv_heads, int head_dim,
+                        int v_width, const int* block_table, int max_blocks, const int* token_slot, const int* positions,
+                        void* out, int ldo, int n_tokens, int n_heads, int n_kv_heads, int head_dim, int v_head_dim,
                         int page_tokens, int window, float scale, const float* slopes, hipStream_t stream);
 
 // bf16 on the matrix cores; see attention_mfma.hip for what it needs.

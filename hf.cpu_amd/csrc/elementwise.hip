@@ -190,27 +190,27 @@ struct QkvSource {
 template <typename T>
 __global__ __launch_bounds__(128) void rope_store_kernel(
     T* __restrict__ qkv, int ld, const int* __restrict__ positions, const float* __restrict__ inv_freq, int rot_dim,
-    int H, int G, int D, T* __restrict__ k_cache, T* __restrict__ v_cache, const int* __restrict__ slot_map,
+    int H, int G, int D, int Dv, T* __restrict__ k_cache, T* __restrict__ v_cache, const int* __restrict__ slot_map,
     int page_tokens, const float* __restrict__ partial, int splits, const float* __restrict__ pbias, int n_tokens) {
     const int t = blockIdx.x, hs = blockIdx.y;
     const int half = rot_dim / 2, rest = D - rot_dim;
-    const int width = (H + 2 * G) * D;
+    const int width = (H + G) * D + G * Dv;                   // value heads may have a size of their own
     QkvSource<T> in = {qkv + (size_t)t * ld, partial + (size_t)t * width, pbias, (size_t)n_tokens * width, splits};
     T* row = qkv + (size_t)t * ld;
     const int slot = (G > 0 && slot_map) ? slot_map[t] : -1;
-    const int base = hs * D;                                  // first column of this head in the row
     if (hs >= H + G) {                                        // a value head: copy, transposed inside the page
+        const int c0 = (hs - H - G) * Dv, vbase = (H + G) * D + c0;
         if (slot < 0) {
             if (splits > 0)
-                for (int i = threadIdx.x; i < D; i += blockDim.x) row[base + i] = from_f32<T>(in.at(base + i));
+                for (int i = threadIdx.x; i < Dv; i += blockDim.x) row[vbase + i] = from_f32<T>(in.at(vbase + i));
             return;
         }
-        const int c0 = (hs - H - G) * D;
-        T* vdst = v_cache + (size_t)(slot / page_tokens) * page_tokens * (G * D) + slot % page_tokens;
-        for (int i = threadIdx.x; i < D; i += blockDim.x)
-            vdst[(size_t)(c0 + i) * page_tokens] = from_f32<T>(in.at(base + i));
+        T* vdst = v_cache + (size_t)(slot / page_tokens) * page_tokens * (G * Dv) + slot % page_tokens;
+        for (int i = threadIdx.x; i < Dv; i += blockDim.x)
+            vdst[(size_t)(c0 + i) * page_tokens] = from_f32<T>(in.at(vbase + i));
         return;
     }
+    const int base = hs * D;                                  // first column of this head in the row
     // a query or key head: rotate; keys go to the cache (or stay in the row if there is no cache row)
     const bool is_key = hs >= H;
     T* dst = (is_key && slot >= 0) ? k_cache + (size_t)slot * (G * D) + (hs - H) * D : row + base;
@@ -309,14 +309,14 @@ __global__ __launch_bounds__(256) void rope_store_rows_kernel(
 }
 
 extern "C" int hfa_rope_store(void* qkv, int dtype, int ld, const int* positions, const float* inv_freq, int rot_dim,
-                              int n_heads, int n_kv_heads, int head_dim, void* k_cache, void* v_cache,
+                              int n_heads, int n_kv_heads, int head_dim, int v_head_dim, void* k_cache, void* v_cache,
                               const int* slot_map, int page_tokens, int n_tokens, const float* partial, int splits,
                               const float* partial_bias, hipStream_t stream) {
-    HFA_REQUIRE(n_tokens > 0 && n_heads > 0 && n_kv_heads >= 0 && head_dim > 0, "rope_store: bad sizes");
+    HFA_REQUIRE(n_tokens > 0 && n_heads > 0 && n_kv_heads >= 0 && head_dim > 0 && v_head_dim > 0, "rope_store: bad sizes");
     HFA_REQUIRE(rot_dim >= 0 && rot_dim % 2 == 0 && rot_dim <= head_dim,
                 "rope_store: rot_dim %d must be even and at most head_dim %d", rot_dim, head_dim);
     HFA_REQUIRE(rot_dim == 0 || (positions && inv_freq), "rope_store: positions and inv_freq are needed");
-    HFA_REQUIRE(ld >= (n_heads + 2 * n_kv_heads) * head_dim, "rope_store: row stride %d is too small", ld);
+    HFA_REQUIRE(ld >= (n_heads + n_kv_heads) * head_dim + n_kv_heads * v_head_dim, "rope_store: row stride %d is too small", ld);
     HFA_REQUIRE(n_kv_heads == 0 || !slot_map || (k_cache && v_cache && page_tokens > 0),
                 "rope_store: no cache to store into");
     HFA_REQUIRE(dtype == HFA_F32 || dtype == HFA_BF16, "rope_store: unknown dtype %d", dtype);
@@ -324,7 +324,7 @@ extern "C" int hfa_rope_store(void* qkv, int dtype, int ld, const int* positions
     HFA_REQUIRE(n_heads + 2 * n_kv_heads <= 65535, "rope_store: too many heads for the grid");
     const int kd = n_kv_heads * head_dim;
     const size_t rows_lds = (size_t)ROPE_TOKENS * rot_dim * sizeof(float) + (size_t)ROPE_TOKENS * kd * 2 + ROPE_TOKENS * sizeof(int);
-    if (dtype == HFA_BF16 && splits == 0 && n_tokens >= ROPE_ROWS_FROM && rot_dim > 0 && rot_dim % 16 == 0 &&
+    if (dtype == HFA_BF16 && splits == 0 && n_tokens >= ROPE_ROWS_FROM && rot_dim > 0 && rot_dim % 16 == 0 && v_head_dim == head_dim &&
         head_dim % 8 == 0 && ld % 8 == 0 && ((uintptr_t)qkv & 15) == 0 && ((uintptr_t)k_cache & 15) == 0 &&
         ((uintptr_t)v_cache & 15) == 0 && rows_lds <= 48 * 1024) {
         rope_store_rows_kernel<<<(n_tokens + ROPE_TOKENS - 1) / ROPE_TOKENS, 256, rows_lds, stream>>>(
@@ -337,12 +337,12 @@ extern "C" int hfa_rope_store(void* qkv, int dtype, int ld, const int* positions
     const int threads = head_dim >= 128 ? 128 : 64;
     if (dtype == HFA_F32)
         rope_store_kernel<float><<<grid, threads, 0, stream>>>((float*)qkv, ld, positions, inv_freq, rot_dim, n_heads,
-                                                               n_kv_heads, head_dim, (float*)k_cache,
+                                                               n_kv_heads, head_dim, v_head_dim, (float*)k_cache,
                                                                (float*)v_cache, slot_map, page_tokens, partial,
                                                                splits, partial_bias, n_tokens);
     else
         rope_store_kernel<bf16><<<grid, threads, 0, stream>>>((bf16*)qkv, ld, positions, inv_freq, rot_dim, n_heads,
-                                                              n_kv_heads, head_dim, (bf16*)k_cache, (bf16*)v_cache,
+                                                              n_kv_heads, head_dim, v_head_dim, (bf16*)k_cache, (bf16*)v_cache,
                                                               slot_map, page_tokens, partial, splits, partial_bias,
                                                               n_tokens);
     HFA_LAUNCH_CHECK("rope_store");

@@ -18,8 +18,8 @@ _SIGNATURES = {
     "hfa_rmsnorm": [P, P, P, I, P, I, I, F, P, I, P, P],
     "hfa_gemm": [P, I, I, P, I, I, P, P, I, I, I, I, I, I, I, P, c_size_t, I, P, I, P],
     "hfa_gemm_finish": [P, I, P, P, I, I, I, I, I, I, P],
-    "hfa_rope_store": [P, I, I, P, P, I, I, I, I, P, P, P, I, I, P, I, P, P],
-    "hfa_paged_attention": [P, I, I, P, P, I, P, I, P, P, P, I, I, I, P, I, I, I, I, I, I, I, F, P, P, c_size_t, I, P],
+    "hfa_rope_store": [P, I, I, P, P, I, I, I, I, I, P, P, P, I, I, P, I, P, P],
+    "hfa_paged_attention": [P, I, I, P, P, I, I, P, I, P, P, P, I, I, I, P, I, I, I, I, I, I, I, I, F, P, P, c_size_t, I, P],
     "hfa_swiglu": [P, P, I, I, I, P],
     "hfa_scatter_i32": [P, P, P, I, P],
     "hfa_move_i32": [P, P, P, P, I, P],

@@ -271,13 +271,16 @@ class Ops:
         F, E = w_gate.shape
         return torch.stack([w_gate.view(F // 32, 32, E), w_up.view(F // 32, 32, E)], dim=1).reshape(2 * F, E).contiguous()
 
-    def rope_store(self, qkv, positions, inv_freq, rot_dim, n_heads, n_kv_heads, head_dim, cache, slot_map):
+    def rope_store(self, qkv, positions, inv_freq, rot_dim, n_heads, n_kv_heads, head_dim, cache, slot_map,
+                   v_head_dim=None):
         """Rotates q (and k) inside ``qkv`` and, if ``slot_map`` is given, stores k and v
         rows into ``cache.k`` / ``cache.v`` at the rows it names (values transposed inside
-        their page, see csrc/api.h)."""
+        their page, see csrc/api.h). ``v_head_dim``: the size of a value head if it is not ``head_dim``."""
+        v_head_dim = head_dim if v_head_dim is None else int(v_head_dim)
+        row_width = (n_heads + n_kv_heads) * head_dim + n_kv_heads * v_head_dim
         pend = self._pending
         if pend is not None and not pend.accumulate and pend.out.data_ptr() == qkv.data_ptr() \
-                and pend.out.shape == qkv.shape and qkv.shape[1] == (n_heads + 2 * n_kv_heads) * head_dim:
+                and pend.out.shape == qkv.shape and qkv.shape[1] == row_width:
             self._pending = None
             if qkv.dtype == torch.bfloat16 and qkv.shape[0] >= 512 and rot_dim > 0:
                 # A prompt portion: the kernel for many tokens does not add up partial sums; finishing
@@ -290,29 +293,31 @@ class Ops:
             self.settle()
         ld = _rows(qkv, "rope_store qkv")
         T = qkv.shape[0]
-        if qkv.shape[1] < (n_heads + 2 * n_kv_heads) * head_dim:
+        if qkv.shape[1] < row_width:
             fail(EINVAL, "rope_store: the rows are narrower than the heads they should hold")
         k_ptr = v_ptr = None
         if n_kv_heads and slot_map is not None:
-            width = n_kv_heads * head_dim
-            for c in (cache.k, cache.v):
+            for c, width in ((cache.k, n_kv_heads * head_dim), (cache.v, n_kv_heads * v_head_dim)):
                 if c.dtype != qkv.dtype or c.dim() != 2 or c.shape[1] != width or not c.is_contiguous():
                     fail(EINVAL, "rope_store: the cache must have the activations' dtype and one row of "
                                  f"{width} values per token")
             k_ptr, v_ptr = cache.k.data_ptr(), cache.v.data_ptr()
         self._check(self.lib.hfa_rope_store(
             qkv.data_ptr(), _code(qkv), ld, None if positions is None else _ints(positions, "positions", T),
-            None if inv_freq is None else inv_freq.data_ptr(), rot_dim, n_heads, n_kv_heads, head_dim,
+            None if inv_freq is None else inv_freq.data_ptr(), rot_dim, n_heads, n_kv_heads, head_dim, v_head_dim,
             k_ptr, v_ptr, None if slot_map is None else _ints(slot_map, "slot_map", T),
             getattr(cache, "page_tokens", 0) or 0, T, None if pend is None else self.workspace.data_ptr(),
             0 if pend is None else pend.splits,
             None if pend is None or pend.bias is None else pend.bias.data_ptr(), self._stream()))
 
-    def paged_attention(self, q, n_heads, n_kv_heads, head_dim, cache, step, window, scale, out, slopes=None):
+    def paged_attention(self, q, n_heads, n_kv_heads, head_dim, cache, step, window, scale, out, slopes=None,
+                        v_head_dim=None):
         """Attention of the first ``n_heads * head_dim`` columns of ``q`` over ``cache``. ``slopes``
         (fp32, one per query head): the score of key j for the query at p gets ``slopes[h] * (j - p)``
-        added, for position encodings that enter the scores; the plain kernel then runs."""
+        added, for position encodings that enter the scores; the plain kernel then runs, as it does when
+        value heads have a size of their own (``v_head_dim``; ``out`` then has that many columns a head)."""
         self.settle()
+        v_head_dim = head_dim if v_head_dim is None else int(v_head_dim)
         if slopes is not None and (slopes.dtype != torch.float32 or slopes.numel() != n_heads or not slopes.is_contiguous()
                                    or slopes.device != q.device):
             fail(EINVAL, "paged_attention: slopes must be contiguous fp32 on the device, one per query head")
@@ -321,8 +326,8 @@ class Ops:
         g = step.group(cache.group)
         if cache.k.dtype != q.dtype or out.dtype != q.dtype:
             fail(EINVAL, "paged_attention: queries, cache and output must share a dtype")
-        if cache.k.shape[1] != n_kv_heads * head_dim:
-            fail(EINVAL, "paged_attention: the cache rows do not hold n_kv_heads * head_dim values")
+        if cache.k.shape[1] != n_kv_heads * head_dim or cache.v.shape[1] != n_kv_heads * v_head_dim:
+            fail(EINVAL, "paged_attention: the cache rows do not hold n_kv_heads * head_dim keys and n_kv_heads * v_head_dim values")
         _ints(step.token_slot, "token_slot", T)
         _ints(step.positions, "positions", T)
         _ints(step.q_start, "q_start", step.n_seqs + 1)
@@ -332,10 +337,10 @@ class Ops:
         def call(first, n_tokens, q_start, n_seqs, max_q_len):
             self._check(self.lib.hfa_paged_attention(
                 q.data_ptr() + first * ldq * q.element_size(), _code(q), ldq, cache.k.data_ptr(), cache.v.data_ptr(),
-                cache.k.shape[1], g.block_table.data_ptr(), g.block_table.shape[1],
+                cache.k.shape[1], cache.v.shape[1], g.block_table.data_ptr(), g.block_table.shape[1],
                 step.token_slot.data_ptr() + 4 * first, step.positions.data_ptr() + 4 * first, q_start.data_ptr(), n_seqs,
                 max_q_len, step.max_seq_len, out.data_ptr() + first * ldo * out.element_size(), ldo, n_tokens, n_heads,
-                n_kv_heads, head_dim, cache.page_tokens, int(window), float(scale),
+                n_kv_heads, head_dim, v_head_dim, cache.page_tokens, int(window), float(scale),
                 None if slopes is None else slopes.data_ptr(), self.attn_workspace.data_ptr(),
                 self.attn_workspace.numel(), 1 if plain else 0, self._stream()))
 

@@ -65,8 +65,9 @@ class Model:
         return cls(plan_fn(config), config)
 
     @classmethod
-    def from_dir(cls, model_dir, dtype, ops, overrides=None):
-        model = cls.from_config(read_config(model_dir, overrides))
+    def from_dir(cls, model_dir, dtype, ops, options=None):
+        """``options``: model options of the session (``config.apply_model_options``)."""
+        model = cls.from_config(read_config(model_dir, options))
         dt = compute_dtype(dtype)
         model._bind(load_tensors(model_dir, model.param_specs(), dt, ops.device), dt, ops)
         return model

@@ -29,12 +29,17 @@ class Attention(Part):
 
 
     def __init__(self, hidden_size, n_heads, n_kv_heads, head_dim, qkv_bias, window, position,
-                 scale=None, out_bias=False, prefix=""):
+                 scale=None, out_bias=False, v_head_dim=None, prefix=""):
+        """``v_head_dim``: the size of a value head where it is not ``head_dim`` (key rows of the cache are
+        then ``n_kv_heads * head_dim`` wide, value rows ``n_kv_heads * v_head_dim``, and the output
+        projection reads ``n_heads * v_head_dim`` columns; such a mixer runs the plain kernels)."""
         super().__init__(prefix)
         if n_heads % n_kv_heads:
             fail(EINVAL, f"attention: {n_heads} heads are not a multiple of {n_kv_heads} key/value heads")
         self.E, self.H, self.G, self.D = hidden_size, n_heads, n_kv_heads, head_dim
+        self.Dv = head_dim if v_head_dim is None else int(v_head_dim)
         self.QD, self.KD = n_heads * head_dim, n_kv_heads * head_dim
+        self.VD, self.OD = n_kv_heads * self.Dv, n_heads * self.Dv
         self.qkv_bias = bool(qkv_bias)
         self.out_bias = bool(out_bias)
         self.window = int(window)
@@ -49,18 +54,18 @@ class Attention(Part):
         p = self.prefix
         specs = [ParamSpec(p + "q_proj.weight", (self.QD, self.E)),
                  ParamSpec(p + "k_proj.weight", (self.KD, self.E)),
-                 ParamSpec(p + "v_proj.weight", (self.KD, self.E)),
-                 ParamSpec(p + "o_proj.weight", (self.E, self.QD))]
+                 ParamSpec(p + "v_proj.weight", (self.VD, self.E)),
+                 ParamSpec(p + "o_proj.weight", (self.E, self.OD))]
         if self.qkv_bias:
             specs += [ParamSpec(p + "q_proj.bias", (self.QD,), "vector"),
                       ParamSpec(p + "k_proj.bias", (self.KD,), "vector"),
-                      ParamSpec(p + "v_proj.bias", (self.KD,), "vector")]
+                      ParamSpec(p + "v_proj.bias", (self.VD,), "vector")]
         if self.out_bias:
             specs.append(ParamSpec(p + "o_proj.bias", (self.E,), "vector"))
         return specs
 
     def cache_need(self):
-        return PagedKV(self.KD, self.KD, self.window)
+        return PagedKV(self.KD, self.VD, self.window)
 
     def bind(self, params, ops):
         p = self.prefix
@@ -76,15 +81,18 @@ class Attention(Part):
 
     def forward(self, ops, step, h, cache, x, write_cache=True):
         T = h.shape[0]
-        width = self.QD + 2 * self.KD if write_cache else self.QD
+        width = self.QD + self.KD + self.VD if write_cache else self.QD
         qkv = ops.scratch("qkv", (T, width), ops.act_dtype)
         # a product that split K is added up inside the next kernel (position.store, the next norm)
         with ops.section("qkv"):
             ops.gemm(h, self.w_qkv[:width], qkv, bias=None if self.b_qkv is None else self.b_qkv[:width], defer=True)
-        self.position.store(ops, step, qkv, self.H, self.G if write_cache else 0, cache, write_cache)
-        att = ops.scratch("att", (T, self.QD), ops.act_dtype)
+        if self.Dv == self.D:
+            self.position.store(ops, step, qkv, self.H, self.G if write_cache else 0, cache, write_cache)
+        else:                                   # only a position part that knows of value heads of another size can serve
+            self.position.store(ops, step, qkv, self.H, self.G if write_cache else 0, cache, write_cache, v_head_dim=self.Dv)
+        att = ops.scratch("att", (T, self.OD), ops.act_dtype)
         with ops.section("attn"):
             ops.paged_attention(qkv, self.H, self.G, self.D, cache, step, self.window, self.scale, att,
-                                slopes=getattr(self.position, "score_slopes", None))
+                                slopes=getattr(self.position, "score_slopes", None), v_head_dim=self.Dv)
         with ops.section("wo"):
             ops.gemm(att, self.w_o, x, bias=self.b_o, accumulate=True, defer=True)

@@ -9,7 +9,7 @@ Interfaces by role (``step`` is the engine's StepInputs, ``ops`` its kernels):
 
   embedding     forward(ops, step, out_x)                    tokens -> fp32 residual stream [T, E]
   norm          forward(ops, x, out, rows=None)              fp32 [T, E] -> activation dtype [T or R, E]
-  position      bind_tables(ops); store(ops, step, qkv, heads, kv_heads, head_dim, cache, write)
+  position      store(ops, step, qkv, heads, kv_heads, cache, write[, v_head_dim=...])    acts on packed q | k | v rows
   mixer         cache_need(); forward(ops, step, h, cache, x, write_cache=True)     x += mixer(h)
   feed_forward  forward(ops, step, h, x)                                             x += ffn(h)
   block         forward(ops, step, x, parts, caches, write_cache)    parts: {name: part} as the plan names them;

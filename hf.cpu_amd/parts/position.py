@@ -36,11 +36,12 @@ class Rotary(Part):
         inv = torch.pow(torch.tensor(self.theta, dtype=torch.float64), -2.0 * i / self.rot_dim)
         self.inv_freq = memory.to_device(inv.to(torch.float32), ops.device, "rotary frequencies")
 
-    def store(self, ops, step, qkv, n_heads, n_kv_heads, cache, write):
+    def store(self, ops, step, qkv, n_heads, n_kv_heads, cache, write, v_head_dim=None):
         """Rotates the queries (and keys) inside ``qkv`` at each token's position;
-        if ``write``, puts each token's rotated key and its value into its cache row."""
+        if ``write``, puts each token's rotated key and its value into its cache row.
+        ``v_head_dim``: the size of a value head where it is not the keys'."""
         ops.rope_store(qkv, step.positions, self.inv_freq, self.rot_dim, n_heads, n_kv_heads,
-                       self.head_dim, cache, step.group(cache.group).slot_map if write else None)
+                       self.head_dim, cache, step.group(cache.group).slot_map if write else None, v_head_dim=v_head_dim)
 
 
 @register_part("position", "none")
@@ -53,7 +54,7 @@ class NoPosition(Part):
         super().__init__(prefix)
         self.head_dim = head_dim
 
-    def store(self, ops, step, qkv, n_heads, n_kv_heads, cache, write):
+    def store(self, ops, step, qkv, n_heads, n_kv_heads, cache, write, v_head_dim=None):
         if write:
             ops.rope_store(qkv, step.positions, None, 0, n_heads, n_kv_heads, self.head_dim,
-                           cache, step.group(cache.group).slot_map)
+                           cache, step.group(cache.group).slot_map, v_head_dim=v_head_dim)

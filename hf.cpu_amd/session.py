@@ -49,19 +49,20 @@ def state_bytes_per_request(model):
 
 class Session:
     def __init__(self, model, dtype="bfloat16", ctx_max=32768, batch=64, page_size=16, max_seqs=64,
-                 kv_tokens=None, device="cuda:0", seed=0, config_overrides=None):
+                 kv_tokens=None, device="cuda:0", seed=0, model_options=None):
         """``model``: a folder with config.json and model.safetensors, or a typed
         configuration (random weights from ``seed`` are then made on the device).
         ``ctx_max``: most tokens per request. ``batch``: tokens per step. ``kv_tokens``:
         tokens the page pools hold (default: ``ctx_max * max_seqs``, but no more than
-        most of the free memory allows). ``config_overrides``: keys that replace those of the folder's
-        config.json (``--window``)."""
+        most of the free memory allows). ``model_options``: options that change the folder's
+        configuration in the engine's own words, e.g. ``{"window": 4096}`` (``--window``); the architecture's
+        configuration class turns them into its config.json keys."""
         self.ops = Ops(compute_dtype(dtype), device)
         if isinstance(model, (str, os.PathLike)):
             self.model_dir = os.fspath(model)
             stat = os.stat(os.path.join(self.model_dir, "config.json"))
             self.identity = (os.path.abspath(self.model_dir), stat.st_size, stat.st_mtime)     # src/ops.c:538-545
-            self.model = Model.from_dir(self.model_dir, dtype, self.ops, config_overrides)
+            self.model = Model.from_dir(self.model_dir, dtype, self.ops, model_options)
         else:
             self.model_dir, self.identity = None, ("random", id(model), seed)
             self.model = Model.from_random(model, seed, dtype, self.ops)

@@ -125,3 +125,34 @@ def test_allocation_counter_fails_the_nth_once():
     assert memory.allocations() == base + 8
     memory.fail_after(0)
     memory.note("none fails")
+
+
+def test_model_options_are_spelled_by_the_configuration_class(tmp_path):
+    """A session's model options come in the engine's words (``window``); the architecture's configuration
+    class turns them into its own config.json keys, so nothing above it names a key of Qwen2's. An
+    architecture whose class has no such method, or does not know the option, refuses it by name."""
+    import json
+    import hf_cpu_amd
+    from hf_cpu_amd.config import apply_model_options, read_config
+    from hf_cpu_amd.status import EngineError
+    assert apply_model_options(dict(helpers.CONFIG_A), None) == helpers.CONFIG_A
+    assert apply_model_options(dict(helpers.CONFIG_A), {"window": None}) == helpers.CONFIG_A
+    on = config_from_dict(apply_model_options(dict(helpers.CONFIG_A, max_window_layers=1), {"window": 9}))
+    assert [on.layer_window(l) for l in range(2)] == [0, 9]
+    off = config_from_dict(apply_model_options(dict(helpers.CONFIG_B), {"window": 0}))
+    assert [off.layer_window(l) for l in range(3)] == [0, 0, 0]
+    (tmp_path / "config.json").write_text(json.dumps(dict(helpers.CONFIG_B, layer_types=["full_attention"] + 2 * ["sliding_attention"])))
+    assert [read_config(str(tmp_path), {"window": 5}).layer_window(l) for l in range(3)] == [0, 5, 5]
+    with pytest.raises(EngineError) as e:
+        apply_model_options(dict(helpers.CONFIG_A), {"experts": 4})
+    assert e.value.code == "ENOTSUP" and "experts" in e.value.msg and "Qwen2ForCausalLM" in e.value.msg
+
+    class Bare:                                 # a configuration class without model options
+        @classmethod
+        def from_dict(cls, obj, origin="config.json"):
+            return cls()
+    hf_cpu_amd.register_architecture("BareForTest", Bare, lambda cfg: None)
+    assert isinstance(config_from_dict(apply_model_options({"architectures": ["BareForTest"]}, {})), Bare)
+    with pytest.raises(EngineError) as e:
+        apply_model_options({"architectures": ["BareForTest"]}, {"window": 8})
+    assert e.value.code == "ENOTSUP" and "BareForTest" in e.value.msg and "window" in e.value.msg

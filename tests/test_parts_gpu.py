@@ -84,33 +84,45 @@ def test_feed_forward_part(ops32):
     assert np.max(np.abs(tx.cpu().numpy() - want)) < 2e-5
 
 
-def attention_reference(p, prefix, h, positions, H, G, D, theta, window, rot=None):
+def attention_reference(p, prefix, h, positions, H, G, D, theta, window, rot=None, Dv=None):
     T = h.shape[0]
+    Dv = Dv or D
     q = plain.linear(h, p[prefix + "q_proj.weight"], p[prefix + "q_proj.bias"]).reshape(T, H, D)
     k = plain.linear(h, p[prefix + "k_proj.weight"], p[prefix + "k_proj.bias"]).reshape(T, G, D)
-    v = plain.linear(h, p[prefix + "v_proj.weight"], p[prefix + "v_proj.bias"]).reshape(T, G, D)
+    v = plain.linear(h, p[prefix + "v_proj.weight"], p[prefix + "v_proj.bias"]).reshape(T, G, Dv)
     q, k = plain.rope(q, positions, rot or D, theta), plain.rope(k, positions, rot or D, theta)
-    return plain.linear(plain.attention(q, k, v, window).reshape(T, H * D), p[prefix + "o_proj.weight"])
+    if Dv == D:
+        att = plain.attention(q, k, v, window)
+    else:       # value heads of their own size: the same weights on other values (scores do not see the values)
+        att = np.zeros((T, H, Dv))
+        for lo in range(0, Dv, D):
+            part = np.zeros((T, G, D))
+            part[..., :min(D, Dv - lo)] = v[..., lo:lo + D]
+            att[..., lo:lo + D] = plain.attention(q, k, part, window)[..., :min(D, Dv - lo)]
+    return plain.linear(att.reshape(T, H * Dv), p[prefix + "o_proj.weight"])
 
 
-@pytest.mark.parametrize("H,G,D,window,rot", [(4, 2, 16, 0, 16), (6, 3, 32, 9, 32), (2, 2, 48, 0, 32)])
-def test_attention_part_alone(ops32, H, G, D, window, rot):
+@pytest.mark.parametrize("H,G,D,window,rot,Dv", [(4, 2, 16, 0, 16, None), (6, 3, 32, 9, 32, None), (2, 2, 48, 0, 32, None),
+                                                 (4, 2, 16, 0, 16, 24), (6, 2, 32, 11, 32, 8)])
+def test_attention_part_alone(ops32, ops16, H, G, D, window, rot, Dv):
     """One attention mixer with its cache: a prompt in two portions, then single tokens; two
     requests side by side. The reference is attention over each whole sequence. The third
-    case rotates only part of each head and has a width that is no multiple of 64."""
+    case rotates only part of each head and has a width that is no multiple of 64; the last two have
+    value heads of another size than the keys' (the cache's value rows are then narrower or wider than
+    its key rows: a group of its own in the manager, the plain kernels on the device), also in bf16."""
     rng = np.random.default_rng(H * D)
     E, theta = 56, 5e4
     spec = PartSpec("attention", dict(hidden_size=E, n_heads=H, n_kv_heads=G, head_dim=D, qkv_bias=True,
-                                      window=window, prefix="a.",
+                                      window=window, prefix="a.", **({} if Dv is None else {"v_head_dim": Dv}),
                                       position=PartSpec("rotary", dict(head_dim=D, rot_dim=rot, theta=theta))))
     part = make_part("mixer", spec)
-    assert part.cache_need() == PagedKV(G * D, G * D, window)
+    assert part.cache_need() == PagedKV(G * D, G * (Dv or D), window)
     p = {s.name: (rng.standard_normal(s.shape) * (0.3 if s.kind == "vector" else 1.2 / math.sqrt(s.shape[1])))
          .astype(np.float32) for s in part.all_param_specs()}
     bind(part, p, ops32)
     p64 = {k: v.astype(np.float64) for k, v in p.items()}
     hs = {r: rng.standard_normal((n, E)).astype(np.float32) for r, n in (("a", 21), ("b", 13))}
-    want = {r: attention_reference(p64, "a.", h.astype(np.float64), range(len(h)), H, G, D, theta, window, rot)
+    want = {r: attention_reference(p64, "a.", h.astype(np.float64), range(len(h)), H, G, D, theta, window, rot, Dv)
             for r, h in hs.items()}
     har = Harness(ops32, [part.cache_need()])
     cuts = [[("a", 0, 9)], [("a", 9, 19), ("b", 0, 12)], [("a", 19, 20), ("b", 12, 13)], [("a", 20, 21)]]
@@ -122,6 +134,23 @@ def test_attention_part_alone(ops32, H, G, D, window, rot):
         ref = np.concatenate([want[r][s:e] for r, s, e in cut])
         err = np.max(np.abs(x.cpu().numpy() - ref))
         assert err < 5e-5, f"cut {cut}: {err:.3e}"
+    if Dv is None:
+        return
+    part16 = make_part("mixer", spec)
+    part16.bind_all({k: dev(v, torch.float32 if v.ndim == 1 else torch.bfloat16) for k, v in p.items()}, ops16)
+    r64 = {k: (helpers.bf16_round(v).astype(np.float64) if v.ndim == 2 else v.astype(np.float64)) for k, v in p.items()}
+    har = Harness(ops16, [part16.cache_need()])
+    for cut in cuts:
+        step = har.inputs([(r, [0] * (e - s)) for r, s, e in cut])
+        h = helpers.bf16_round(np.concatenate([hs[r][s:e] for r, s, e in cut]))
+        x = torch.zeros((h.shape[0], E), device="cuda")
+        part16.forward(ops16, step, dev(h, torch.bfloat16), har.views[0], x)
+        ops16.settle()
+        whole = {r: attention_reference(r64, "a.", helpers.bf16_round(hh).astype(np.float64), range(len(hh)), H, G, D, theta, window, rot, Dv)
+                 for r, hh in hs.items()}
+        ref = np.concatenate([whole[r][s:e] for r, s, e in cut])
+        err = np.max(np.abs(x.cpu().numpy() - ref)) / np.max(np.abs(ref))
+        assert err < 2e-2, f"bf16, cut {cut}: {err:.3e}"
 
 
 def toy_plan_factory():

@@ -98,6 +98,9 @@ int hfa_argmax(const float* logits, int ld, int* out, int n_rows, int vocab, voi
 // GPU it runs on, until the process ends), so the call allocates nothing; the caller still passes
 // logits and out. At most HFA_ARGMAX_STATIC_ROWS rows; more are refused. Calls that overlap on one
 // GPU share that array and race; nothing needs clearing between calls that follow each other.
+// The first call on a device asks the runtime for the array's address there, which is no stream
+// operation: it must be an eager call (one made while the stream is being captured is refused with
+// a message that says so); every later call on that device may be captured.
 #define HFA_ARGMAX_STATIC_ROWS 256
 int hfa_argmax_static(const float* logits, int ld, int* out, int n_rows, int vocab, hipStream_t stream);
 

@@ -101,7 +101,7 @@ static __device__ __align__(256) unsigned char scratch[(size_t)HFA_ARGMAX_STATIC
 static void* scratch_of_device[HFA_MAX_DEVICES];      // device address of `scratch` per GPU, null = not asked yet
 static std::mutex scratch_lock;
 
-static int scratch_address(void** out) {
+static int scratch_address(void** out, hipStream_t stream) {
     int dev = -1;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess || dev < 0 || dev >= HFA_MAX_DEVICES) {
@@ -110,6 +110,15 @@ static int scratch_address(void** out) {
     }
     std::lock_guard<std::mutex> hold(scratch_lock);
     if (scratch_of_device[dev] == nullptr) {
+        // Asking for the address may load the code object and is no stream operation: under a capture it
+        // could fail or break the capture. The first call on a device therefore has to be an eager one.
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        e = hipStreamIsCapturing(stream, &capturing);
+        if (e != hipSuccess || capturing != hipStreamCaptureStatusNone) {
+            hfa_set_error("argmax_static: the first call on device %d came while its stream is being captured; call it "
+                          "once eagerly on this device before capturing it into a graph", dev);
+            return 1;
+        }
         void* ptr = nullptr;
         e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));       // for the current device
         if (e != hipSuccess || ptr == nullptr) {
@@ -129,7 +138,7 @@ extern "C" int hfa_argmax_static(const float* logits, int ld, int* out, int n_ro
                 "workspace for more)", n_rows, HFA_ARGMAX_STATIC_ROWS);
     HFA_REQUIRE(logits != nullptr && out != nullptr, "argmax_static: null logits or output");
     void* ptr = nullptr;
-    if (int rc = scratch_address(&ptr)) return rc;
+    if (int rc = scratch_address(&ptr, stream)) return rc;
     float* part_v = (float*)ptr;
     int* part_i = (int*)(part_v + (size_t)n_rows * ARGMAX_PARTS);
     argmax_part_kernel<<<dim3(n_rows, ARGMAX_PARTS), 256, 0, stream>>>(logits, ld, vocab, part_v, part_i);

@@ -73,6 +73,8 @@ class Sampler:
         self.ops = ops
         self._landing = []            # pinned host buffers that chosen tokens are copied to, used in turn
         self._turn = 0
+        self._outbox = []             # pinned host buffers that the draws' numbers leave from: [tensor, event of its last copy]
+        self._out_turn = 0
 
     def _to_host_later(self, tokens):
         """Enqueues the copy of ``tokens`` (int32 on the device) to pinned host memory right behind the
@@ -97,12 +99,32 @@ class Sampler:
     def _draw(self, ids, vals, numbers, cuts, on_device=False):
         """The device's draw for rows of candidates in order; the rows' numbers and cuts travel as one copy."""
         n = len(cuts)
-        both = np.empty(5 * n, dtype=f32)
-        both[:4 * n] = numbers.reshape(-1)
-        both[4 * n:].view(np.int32)[:] = cuts
-        sent = memory.to_device(torch.from_numpy(both), vals.device, "the draws' numbers")
+        sent = self._send(numbers, cuts, vals.device)
         drawn = self.ops.draw_rows(ids, vals, sent[:4 * n].view(n, 4), sent[4 * n:].view(torch.int32))
         return drawn if on_device else drawn.cpu().numpy()
+
+    def _send(self, numbers, cuts, device):
+        """The rows' numbers ([n, 4] fp32) and cuts ([n] int32) on the device as one fp32 tensor of 5 n, by a
+        copy from pinned memory that only enqueues: a copy from pageable memory makes the host wait for
+        everything the stream holds, the step that was just enqueued included. Four host buffers take turns;
+        one is written again only after the copy that last read it is done."""
+        n = len(cuts)
+        if len(self._outbox) < 4:
+            self._outbox.append([memory.empty(max(5 * n, 1280), torch.float32, None, "pinned buffer for the draws' numbers", pin=True), None])
+        self._out_turn = (self._out_turn + 1) % len(self._outbox)
+        box = self._outbox[self._out_turn]
+        if box[1] is not None:
+            box[1].synchronize()
+        if box[0].numel() < 5 * n:
+            box[0] = memory.empty(10 * n, torch.float32, None, "pinned buffer for the draws' numbers", pin=True)
+        flat = box[0].numpy()
+        flat[:4 * n] = np.asarray(numbers, dtype=f32).reshape(-1)
+        flat[4 * n:5 * n].view(np.int32)[:] = cuts
+        sent = memory.empty(5 * n, torch.float32, device, "the draws' numbers")
+        sent.copy_(box[0][:5 * n], non_blocking=True)
+        box[1] = torch.cuda.Event()
+        box[1].record()
+        return sent
 
     def sample_start(self, logits, wants):
         """Begins the sampling of a step's rows and returns a ``Started``: ``device_tokens`` is the int32

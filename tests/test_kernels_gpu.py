@@ -811,6 +811,39 @@ def test_sampler_with_rows_of_every_kind_in_one_step(ops32):
         assert [t for t, _ in got[4].top] == [int(t) for t in np.argsort(-logits[4], kind="stable")[:2]]
 
 
+@pytest.mark.parametrize("greedy", [True, False])
+def test_sampling_starts_without_waiting_for_the_stream(ops32, greedy):
+    """``sample_start`` only enqueues: with a long piece of work on the stream before it (the step that the
+    scheduler has just enqueued), it returns while that work still runs, for greedy rows and for rows drawn
+    from their best k with the reference's defaults (the rows' numbers travel from pinned memory; from
+    pageable memory the copy would make the host wait for the whole stream). The tokens are the plain
+    sampler's all the same."""
+    from hf_cpu_amd.sampling import Rng, Sampler, SamplerParams
+    rng = np.random.default_rng(5)
+    V, R = 4099, 6
+    params = (0.0, 40, 0.95, 0.05) if greedy else (0.8, 40, 0.95, 0.05)
+    sampler = Sampler(ops32)
+    big = torch.randn((4096, 4096), device="cuda")
+    junk = torch.empty_like(big)
+    for trial in range(3):                      # the first trial also allocates the pinned buffers
+        logits = (rng.standard_normal((R, V)) * 3).astype(np.float32)
+        dl = torch.from_numpy(logits).cuda()
+        wants = [(SamplerParams(*params), Rng(50 + trial * R + i), 0) for i in range(R)]
+        torch.cuda.synchronize()
+        for _ in range(60):                     # about a quarter of a second of fp32 products
+            torch.mm(big, big, out=junk)
+        busy = torch.cuda.Event()
+        busy.record()
+        started = sampler.sample_start(dl, wants)
+        still_running = not busy.query()
+        assert started.device_tokens is not None
+        if trial:
+            assert still_running, "sample_start waited for the work enqueued before it"
+        got = [c.token for c in started.finish()]
+        theirs = [plain.Rng(50 + trial * R + i) for i in range(R)]
+        assert got == [plain.sample(logits[i], *params, theirs[i]) for i in range(R)]
+
+
 def test_kernels_refuse_what_they_cannot_do(ops32):
     from hf_cpu_amd.status import EngineError
     with pytest.raises(EngineError, match="head_dim"):

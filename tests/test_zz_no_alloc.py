@@ -23,6 +23,51 @@ def _both(lib, ops, logits):
     return out.cpu().numpy(), want.cpu().numpy()
 
 
+def _static(lib, logits, out):
+    return lib.hfa_argmax_static(ctypes.c_void_p(logits.data_ptr()), logits.stride(0), ctypes.c_void_p(out.data_ptr()),
+                                 logits.shape[0], logits.shape[1], ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+
+
+def test_argmax_static_inside_a_captured_graph():
+    """The first call on a device resolves the address of the library's own buffer, which is no stream
+    operation: made under a capture it is refused with a message that says what to do (in a process that
+    has already called it eagerly the address is known and the call is simply recorded). After one eager
+    call the entry point is captured into a graph, and the graph is replayed on changed logits with eager
+    work of the program between the replays; every replay gives what hfa_argmax gives."""
+    from hf_cpu_amd.kernels import Ops
+    from hf_cpu_amd.kernels.lib import library
+    ops = Ops(torch.float32)
+    lib = library()
+    g = torch.Generator(device="cpu").manual_seed(5)
+    logits = torch.randn((12, 5001), generator=g).cuda()
+    out = torch.full((12,), -7, dtype=torch.int32, device="cuda")
+    torch.cuda.synchronize()
+    cold = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(cold):
+        rc = _static(lib, logits, out)
+    if rc != 0:
+        msg = lib.hfa_last_error().decode()
+        assert "eagerly" in msg and "captured" in msg
+    del cold
+    assert _static(lib, logits, out) == 0, lib.hfa_last_error().decode()          # the eager call
+    torch.cuda.synchronize()
+    assert np.array_equal(out.cpu().numpy(), logits.cpu().numpy().argmax(axis=1))
+    graph = torch.cuda.CUDAGraph()
+    out.fill_(-7)
+    with torch.cuda.graph(graph):
+        rc = _static(lib, logits, out)
+    assert rc == 0, lib.hfa_last_error().decode()
+    for i in range(3):
+        fresh = torch.randn((12, 5001), generator=g)
+        fresh[i, 4000 + i] = 50.0
+        logits.copy_(fresh.cuda())
+        want = ops.argmax(logits).cpu().numpy()            # eager work and a synchronisation between the replays
+        graph.replay()
+        torch.cuda.synchronize()
+        got = out.cpu().numpy()
+        assert np.array_equal(got, want) and got[i] == 4000 + i, f"replay {i}"
+
+
 def test_argmax_static_matches_argmax_on_two_calls_in_a_row():
     from hf_cpu_amd.kernels import Ops
     from hf_cpu_amd.kernels.lib import library

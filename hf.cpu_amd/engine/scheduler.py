@@ -190,12 +190,8 @@ class Scheduler:
         """The entries of a step under the budget and the pages at hand, or None if not even
         the decoded tokens fit."""
         mgr = self.manager
-        decode = [r for r in self.running if r.unfed == 1 and r.n_fed > 0]
+        decode = self._decoders()
         budget = self.token_budget
-        if len(decode) > budget:
-            # More requests decode than a step may hold tokens (the reference refuses --n above --batch,
-            # src/ops.c:810): they take turns, those that waited longest first, so every one advances.
-            decode = sorted(decode, key=lambda r: r.last_ran)[:budget]
         if not mgr.can_reserve([(r.req_id, 1) for r in decode]):      # only for those that run
             return None
         entries = [(r, 1, True) for r in decode]
@@ -228,6 +224,15 @@ class Scheduler:
                 live += 1
                 free_slots -= 1
         return entries
+
+    def _decoders(self):
+        """The running requests that bring one decoded token to the next step."""
+        decode = [r for r in self.running if r.unfed == 1 and r.n_fed > 0]
+        if len(decode) > self.token_budget:
+            # More requests decode than a step may hold tokens (the reference refuses --n above --batch,
+            # src/ops.c:810): they take turns, those that waited longest first, so every one advances.
+            decode = sorted(decode, key=lambda r: r.last_ran)[:self.token_budget]
+        return decode
 
     def _shrink(self, r, n):
         """The next smaller portion worth trying: one page less."""
@@ -280,9 +285,8 @@ class Scheduler:
             # Tokens are read before the plan where the plan turns on them: a request that is about to end
             # by its length holds pages until its last token is booked; short pages may be freed by an
             # end-of-sequence token that the host has not seen.
-            decoders = [r for r in self.running if r.unfed == 1 and r.n_fed > 0][:self.token_budget]
             if not self.running or any(r.unfed == 0 for r in self.running) \
-                    or not self.manager.can_reserve([(r.req_id, 1) for r in decoders]):
+                    or not self.manager.can_reserve([(r.req_id, 1) for r in self._decoders()]):
                 self._land()
         if self.idle:
             return None

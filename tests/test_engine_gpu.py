@@ -412,3 +412,67 @@ def test_what_a_page_held_before_does_not_matter(gpu, tiny, dtype):
                         view.k[p * P:(p + 1) * P] = keep_k[p]
                         view.v[p * P:(p + 1) * P] = keep_v[p]
     helpers.compare(got, {"r2": want["r2"]}, TOL[dtype], f"{name} {dtype} decoding beside poisoned pages")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_tokens_taken_from_the_device(gpu, tiny, dtype):
+    """``Engine.step(fed=...)``: the single token of some entries comes from an int32 tensor on the device,
+    at rows the caller names, instead of from the host. A mixed step whose entries are ordered long portion,
+    fed decoder, short portion, fed decoder (inside the step requests with few tokens are laid first, so the
+    places the tokens go to are not the entries' order), with rows taken from a shuffled tensor; then a plain
+    decode step of more requests than the engine decodes without filling the batch up, replayed from a graph.
+    Each gives the bits of the same step with the tokens given by the host. Rows outside the tensor and
+    entries with two tokens are refused."""
+    import torch
+    from hf_cpu_amd.status import EngineError
+    name, cfg, d, reqs, _ = tiny
+    V = cfg["vocab_size"]
+    rng = np.random.default_rng(9)
+    prompts = {f"q{i}": [int(t) for t in rng.integers(0, V, n)] for i, n in enumerate([5, 9, 3, 12, 6, 7, 4, 8, 10, 11, 2])}
+    many = list(prompts)
+    junk = 10 ** 6
+
+    def run(feed):
+        eng = engine_for(d, dtype, name, 64 * 16, max_seqs=13)
+        eng.step([(r, prompts[r], []) for r in many])
+        long_a, short_b = [int(t) for t in rng0.integers(0, V, 30)], [int(t) for t in rng0.integers(0, V, 4)]
+        tok = {r: int(rng0.integers(0, V)) for r in many}
+        pool = torch.full((64,), junk, dtype=torch.int32, device="cuda")
+        where = {r: int(p) for r, p in zip(many, rng0.permutation(64))}
+        for r in many:
+            pool[where[r]] = tok[r]
+        out = []
+        # long portion, fed decoder, short portion, fed decoder
+        entries = [("A", long_a, [0, 29]), ("q0", [tok["q0"]], [0]), ("B", short_b, [3]), ("q1", [tok["q1"]], [0])]
+        if feed:
+            entries[1] = ("q0", [junk], [0])
+            entries[3] = ("q1", [junk], [0])
+            out.append(eng.step(entries, fed=(pool, {1: where["q0"], 3: where["q1"]})).float().cpu().numpy().copy())
+        else:
+            out.append(eng.step(entries).float().cpu().numpy().copy())
+        # plain decode steps of eleven requests (filled up to sixteen rows), several so that a graph replays
+        for _ in range(4):
+            tok = {r: int(rng0.integers(0, V)) for r in many}
+            for r in many:
+                pool[where[r]] = tok[r]
+            if feed:
+                got = eng.step([(r, [junk], [0]) for r in many], fed=(pool, {i: where[r] for i, r in enumerate(many)}))
+            else:
+                got = eng.step([(r, [tok[r]], [0]) for r in many])
+            out.append(got.float().cpu().numpy().copy())
+        return eng, out, pool
+
+    rng0 = np.random.default_rng(4)
+    _, by_host, _ = run(False)
+    rng0 = np.random.default_rng(4)
+    eng, by_device, pool = run(True)
+    for i, (a, b) in enumerate(zip(by_host, by_device)):
+        assert a.shape == b.shape and np.array_equal(a, b), f"step {i}"
+    assert eng.graph_replays > 0
+    with pytest.raises(EngineError):
+        eng.step([("q0", [1], [0])], fed=(pool, {0: 64}))
+    with pytest.raises(EngineError):
+        eng.step([("q0", [1, 2], [1])], fed=(pool, {0: 3}))
+    with pytest.raises(EngineError):
+        eng.step([("q0", [1], [0])], fed=(pool.long(), {0: 3}))
+    eng.manager.check()

@@ -366,3 +366,26 @@ def test_steps_enqueued_ahead_give_what_steps_in_turn_give(seed):
             ran_ahead = sch.steps_ahead
     assert outcomes[0] == outcomes[1]
     assert ran_ahead > 0 or all(len(g) <= 1 for _, g, _, _ in outcomes[0])
+
+
+def test_the_early_read_looks_at_the_decoders_that_will_run():
+    """More decoders than the budget, a pool that is almost full, and an end-of-sequence token that the host
+    has not read yet: whether the tokens in flight must be read before planning is decided on the decoders
+    that the plan will pick (those that waited longest), not on the first ones in running order. Otherwise
+    the plan finds its own set short of a page and throws the newest request out, although the token in
+    flight frees the pages that are missing."""
+    for la, lb, lc, n_pages, low_at, eos_at, who in ((1, 1, 1, 5, 2, 4, 1), (1, 1, 3, 4, 1, 2, 1), (1, 1, 1, 5, 3, 5, 0)):
+        eng = FakeEngine(n_pages=n_pages, page=4, slots=3, ctx=32)
+        script = {f"r{i}": [10 + j for j in range(12)] for i in range(3)}
+        script[f"r{who}"][eos_at] = 99
+        sch = Scheduler(eng, AheadSampler(script), token_budget=16)
+        reqs = [sch.submit(Request(f"r{i}", list(range(1, n + 1)), greedy(), max_tokens=8, eos_ids=(99,)))
+                for i, n in enumerate((la, lb, lc))]
+        for _ in range(low_at):
+            sch.step()
+        sch.token_budget = 2
+        sch.run()
+        assert all(r.error is None for r in reqs) and sum(r.preemptions for r in reqs) == 0
+        assert reqs[who].stop == "eos" and len(reqs[who].generated) == eos_at
+        assert all(r.stop == "length" and r.generated == [10 + j for j in range(8)] for r in reqs if r is not reqs[who])
+        assert sch.steps_ahead > 0 and not eng.manager.held

@@ -38,6 +38,26 @@ int hfa_gemm(const void* a, int a_dtype, int lda, const void* w, int w_dtype, in
 int hfa_gemm_finish(const void* partial, int splits, const float* bias, void* out, int out_dtype, int ldo,
                     int accumulate, int epilogue, int M, int N, hipStream_t stream);
 
+// The product for up to 16 rows in which every block owns a range of outputs and finishes them itself (bf16
+// operands, K a multiple of 128; see gemm_rows.hip), with what follows a product in a decode step in its last lines:
+//   HFA_ROWS_OUT     out[m, n] = r[m] * sum + bias[n], fp32 or bf16 (out_dtype)
+//   HFA_ROWS_RESID   x[m, n] += sum + bias[n] (fp32, in place); ssq_out[b][m] = block b's share of sum_n x[m, n]^2
+//                    ([hfa_gemm_rows_parts()][16] floats); xg[m, n] = bf16(x[m, n] * g[n]) if xg is given
+//   HFA_ROWS_SWIGLU  act[m, f] = bf16(silu(r[m] * sum_gate) * (r[m] * sum_up)), N features, w's 2 N rows in blocks of
+//                    32 gate rows, 32 up rows (src/model.c:537)
+// r[m] = rsqrt(sum over the parts_in shares ssq_in[.][m] * inv_width + eps), or 1 without ssq_in: the RMS norm of the
+// tensor whose product with the norm's weight is `a` (src/mathx.c:65-75), applied to the sums instead of the operand.
+// hfa_gemm_rows_supports says whether a shape is taken (1 to 16 rows, K a multiple of 128, strides multiples of 8).
+#define HFA_ROWS_OUT 0
+#define HFA_ROWS_RESID 1
+#define HFA_ROWS_SWIGLU 2
+int hfa_gemm_rows_parts(void);
+int hfa_gemm_rows_supports(int mode, int M, int N, int K, int lda, int ldw);
+int hfa_gemm_rows(int mode, const void* a, int lda, const void* w, int ldw, int M, int N, int K, const float* bias,
+                  const float* ssq_in, int parts_in, float inv_width, float eps, void* out, int ldo, int out_dtype,
+                  float* x, int ldx, float* ssq_out, const float* g, void* xg, int ldxg, void* act, int ldact,
+                  hipStream_t stream);
+
 // Rotary position encoding on the q (and k) heads inside qkv rows [q | k | v], split-half
 // pairing, and the store of k (rotated) and v into cache rows slot_map[t] (src/model.c:468-493,
 // 587-600). rot_dim 0: no rotation. n_kv_heads 0: the rows hold q only, nothing is stored.

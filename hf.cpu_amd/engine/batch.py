@@ -50,6 +50,7 @@ class StepInputs:
         self.n_short_seqs = self.n_short_tokens = self.max_short_q_len = 0
         self.q_start_long = None
         self.host = None          # dict of the numpy arrays the device views were copied from
+        self.rows_in_order = False    # logits are wanted for every token, in the tokens' order (a decode step)
 
     def group(self, index):
         return self.groups[index]

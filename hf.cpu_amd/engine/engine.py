@@ -363,6 +363,7 @@ class Engine:
         step.max_q_len, step.max_seq_len = max_q, max_len
         step.n_short_seqs, step.n_short_tokens, step.max_short_q_len = short
         step.host = host
+        step.rows_in_order = R == T and bool(np.array_equal(host["logit_rows"], np.arange(T)))
         for g in range(G):
             slot_map = views[8 + g]
             idx, val = views[8 + G + 2 * g:10 + G + 2 * g]

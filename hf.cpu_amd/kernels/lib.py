@@ -18,6 +18,8 @@ _SIGNATURES = {
     "hfa_rmsnorm": [P, P, P, I, P, I, I, F, P, I, P, P],
     "hfa_gemm": [P, I, I, P, I, I, P, P, I, I, I, I, I, I, I, P, c_size_t, I, P, I, P],
     "hfa_gemm_finish": [P, I, P, P, I, I, I, I, I, I, P],
+    "hfa_gemm_rows": [I, P, I, P, I, I, I, I, P, P, I, F, F, P, I, I, P, I, P, P, P, I, P, I, P],
+    "hfa_gemm_rows_supports": [I, I, I, I, I, I],
     "hfa_rope_store": [P, I, I, P, P, I, I, I, I, I, P, P, P, I, I, P, I, P, P],
     "hfa_paged_attention": [P, I, I, P, P, I, I, P, I, P, P, P, I, I, I, P, I, I, I, I, I, I, I, I, F, P, P, c_size_t, I, P],
     "hfa_swiglu": [P, P, I, I, I, P],
@@ -50,6 +52,8 @@ def library():
             lib.hfa_version.restype = c_int
             lib.hfa_order_rows_scratch.restype = c_size_t
             lib.hfa_order_rows_scratch.argtypes = [c_int, c_int]
+            lib.hfa_gemm_rows_parts.restype = c_int
+            lib.hfa_gemm_rows_parts.argtypes = []
             lib.hfa_probe_barrier_blocks.restype = c_int
             lib.hfa_probe_barrier_blocks.argtypes = []
             lib.hfa_probe_mfma_threads.restype = c_int

@@ -58,6 +58,28 @@ class Pending:
     accumulate: bool
 
 
+@dataclass
+class LazyProduct:
+    """A product into the residual stream that has not been launched yet: ``x += a @ w.T + bias``. If the next
+    thing asked for is the norm of ``x``, product, residual sum and the norm's weight go into one kernel."""
+    a: torch.Tensor
+    w: torch.Tensor
+    x: torch.Tensor
+    bias: object
+
+
+@dataclass
+class Scaled:
+    """A norm's output that holds ``x * weight`` only, not yet divided by the root mean square: the products that
+    read it scale their sums by ``rsqrt(sum(ssq) / width + eps)`` instead. ``x``, ``weight`` and ``eps`` make it whole
+    again (the plain norm kernel) if something else wants to read it."""
+    out: torch.Tensor
+    x: torch.Tensor
+    weight: torch.Tensor
+    eps: float
+    ssq: torch.Tensor
+
+
 class _NoSection:
     def __enter__(self):
         return self
@@ -104,6 +126,10 @@ class Ops:
         self.workspace = memory.empty(WORKSPACE_BYTES, torch.uint8, self.device, "workspace of the matrix products")
         self.attn_workspace = memory.empty(WORKSPACE_BYTES, torch.uint8, self.device, "workspace of attention")
         self._pending = None
+        self._lazy = None                    # a LazyProduct
+        self._scaled = {}                    # data_ptr of a norm's output -> Scaled
+        self.rows_parts = int(self.lib.hfa_gemm_rows_parts())
+        self.fuse_rows = True                # tests switch it off to compare with the chain of separate kernels
         self._splits_out = ctypes.c_int(0)
         self._sections = None                # while timing: (name, start event, end event) of every section left
         self.force_plain_gemm = False        # tests set these to compare the matrix-core paths with the plain ones
@@ -139,6 +165,7 @@ class Ops:
         instead of once per kernel (a forward pass enqueues hundreds)."""
         before = self._stream_handle
         self._stream_handle = torch.cuda.current_stream(self.device).cuda_stream
+        self._scaled.clear()                 # what an earlier pass left in its work buffers is of no use to this one
         try:
             yield self
         finally:
@@ -185,6 +212,7 @@ class Ops:
     # ---- kernels -----------------------------------------------------------
     def embed(self, table, tokens, out_x):
         self.settle()
+        self._source_changes(out_x)
         T = out_x.shape[0]
         if out_x.dtype != torch.float32 or not out_x.is_contiguous() or not table.is_contiguous() \
                 or table.shape[1] != out_x.shape[1]:
@@ -192,7 +220,11 @@ class Ops:
         self._check(self.lib.hfa_embed(table.data_ptr(), _code(table), _ints(tokens, "embed tokens", T),
                                        out_x.data_ptr(), T, table.shape[1], table.shape[0], self._stream()))
 
-    def rmsnorm(self, x, weight, eps, out, rows=None):
+    def rmsnorm(self, x, weight, eps, out, rows=None, lazy=False):
+        """``out[r] = norm(x[rows[r]])``. ``lazy``: the caller promises that ``out`` is read by ``gemm`` alone. Then,
+        if the product that completes ``x`` waits to be launched (``gemm(..., accumulate=True, defer=True)`` of few rows),
+        one kernel does product, residual sum and ``out = x * weight``, and the division by the root mean square is
+        left to the products that read ``out`` (see ``Scaled``)."""
         R = out.shape[0]
         E = x.shape[1]
         if x.dtype != torch.float32 or weight.dtype != torch.float32 or not x.is_contiguous() \
@@ -200,6 +232,16 @@ class Ops:
             fail(EINVAL, "rmsnorm: x and weight must be fp32, contiguous, and of one width with out")
         if rows is None and R != x.shape[0]:
             fail(EINVAL, "rmsnorm: without row indices the output must have x's rows")
+        z = self._lazy
+        if lazy and rows is None and z is not None and z.x.data_ptr() == x.data_ptr() and z.x.shape == x.shape \
+                and out.dtype == torch.bfloat16:
+            self._lazy = None
+            self._source_changes(x, keep=out)
+            ssq = self.scratch(f"ssq@{out.data_ptr()}", (self.rows_parts * 16,), torch.float32)
+            self._rows_resid(z, weight, out, ssq)
+            self._scaled[out.data_ptr()] = Scaled(out, x, weight, float(eps), ssq)
+            return
+        self._scaled.pop(out.data_ptr(), None)
         pend = self._take_pending(x) if rows is None else None
         if pend is None:
             self.settle()
@@ -222,10 +264,74 @@ class Ops:
     def abandon(self):
         """Forgets a deferred product (after a step that failed: its partial sums are of no use)."""
         self._pending = None
+        self._lazy = None
+        self._scaled.clear()
+
+    # ---- products of few rows that finish their outputs themselves (csrc/gemm_rows.hip) -----------------------
+    def _rows_mode(self, a, w, out, bias, accumulate, swiglu):
+        """The mode in which ``hfa_gemm_rows`` takes this product, or None."""
+        if not self.fuse_rows or self.force_plain_gemm or a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 \
+                or a.dim() != 2 or w.dim() != 2 or a.stride(1) != 1 or w.stride(1) != 1 or out.stride(1) != 1:
+            return None
+        M, K = a.shape
+        mode = 1 if accumulate else 2 if swiglu else 0
+        N = w.shape[0] // 2 if swiglu else w.shape[0]
+        if (a.data_ptr() | w.data_ptr()) & 15 or not self.lib.hfa_gemm_rows_supports(
+                mode, M, N, K, _rows(a, "gemm a"), _rows(w, "gemm w")):
+            return None
+        if accumulate:
+            return mode if out.dtype == torch.float32 else None
+        if swiglu:
+            return mode if out.dtype == torch.bfloat16 and bias is None else None
+        return mode
+
+    def _rows_call(self, mode, a, w, N, bias, scaled=None, out=None, x=None, ssq_out=None, g=None, xg=None, act=None):
+        M, K = a.shape
+        null = ctypes.c_void_p(None)
+
+        def ptr(t):
+            return null if t is None else t.data_ptr()
+        self._check(self.lib.hfa_gemm_rows(
+            mode, a.data_ptr(), _rows(a, "gemm a"), w.data_ptr(), _rows(w, "gemm w"), M, N, K, ptr(bias),
+            ptr(None if scaled is None else scaled.ssq), self.rows_parts, 1.0 / K, 0.0 if scaled is None else scaled.eps,
+            ptr(out), 0 if out is None else _rows(out, "gemm out"), 0 if out is None else _code(out),
+            ptr(x), 0 if x is None else _rows(x, "gemm out"), ptr(ssq_out), ptr(g),
+            ptr(xg), 0 if xg is None else _rows(xg, "norm out"), ptr(act), 0 if act is None else _rows(act, "gemm out"),
+            self._stream()))
+
+    def _rows_resid(self, z, g=None, xg=None, ssq=None):
+        """Launches a LazyProduct; with ``g`` and ``xg`` the kernel also leaves ``xg = x * g`` and the sums of squares."""
+        if ssq is None:
+            ssq = self.scratch("ssq@none", (self.rows_parts * 16,), torch.float32)
+        self._rows_call(1, z.a, z.w, z.w.shape[0], z.bias, x=z.x, ssq_out=ssq, g=g, xg=xg)
+
+    def _whole(self, t):
+        """Makes a norm's output that was left undivided (``Scaled``) whole before something other than ``gemm`` reads it."""
+        sc = self._scaled.pop(t.data_ptr(), None)
+        if sc is not None:
+            self._check(self.lib.hfa_rmsnorm(sc.x.data_ptr(), sc.weight.data_ptr(), sc.out.data_ptr(), _code(sc.out), None,
+                                             sc.out.shape[0], sc.out.shape[1], sc.eps, None, 0, None, self._stream()))
+
+    def _source_changes(self, x, keep=None):
+        """``x`` is about to change: norm outputs that could only be made whole from it are made whole now (``keep``:
+        one that is about to be overwritten anyway is dropped instead)."""
+        for key, sc in list(self._scaled.items()):
+            if sc.x.data_ptr() == x.data_ptr():
+                if keep is not None and key == keep.data_ptr():
+                    del self._scaled[key]
+                else:
+                    self._whole(sc.out)
 
     def settle(self, tensor=None):
         """Adds up a deferred product now (all of them if ``tensor`` is None, else only one that
-        writes ``tensor``)."""
+        writes ``tensor``), and makes ``tensor`` whole if it is a norm's output that was left undivided."""
+        z = self._lazy
+        if z is not None and (tensor is None or z.x.data_ptr() == tensor.data_ptr()):
+            self._lazy = None
+            self._source_changes(z.x)
+            self._rows_resid(z)
+        if tensor is not None:
+            self._whole(tensor)
         p = self._pending
         if p is None or (tensor is not None and p.out.data_ptr() != tensor.data_ptr()):
             return
@@ -249,6 +355,34 @@ class Ops:
             fail(EINVAL, f"gemm: shapes a{tuple(a.shape)} w{tuple(w.shape)} out{tuple(out.shape)} do not fit")
         if bias is not None and (bias.dtype != torch.float32 or bias.numel() != N or not bias.is_contiguous()):
             fail(EINVAL, "gemm: the bias must be contiguous fp32 with one value per output column")
+        scaled = self._scaled.get(a.data_ptr())
+        if scaled is not None and scaled.out.shape != a.shape:
+            scaled = None
+        mode = self._rows_mode(a, w, out, bias, accumulate, swiglu)
+        if mode is not None and not (mode == 1 and scaled is not None):
+            self._scaled.pop(out.data_ptr(), None)
+            if mode == 1:                            # into the residual stream
+                z = LazyProduct(a, w, out, bias)
+                if defer:
+                    self._lazy = z                   # the next norm of `out` may take it along
+                else:
+                    self._source_changes(out)
+                    self._rows_resid(z)
+            elif mode == 2:
+                self._rows_call(2, a, w, N // 2, None, scaled=scaled, act=out)
+            elif defer and out.dtype == torch.bfloat16 and M * N * 4 <= self.workspace.numel():
+                # 32-bit sums for the kernel that follows (the rotation of queries and keys): one plane of the workspace
+                plane = self.workspace[:M * N * 4].view(torch.float32).view(M, N)
+                self._rows_call(0, a, w, N, bias, scaled=scaled, out=plane)
+                self._pending = Pending(out, 1, None, False)
+            else:
+                self._rows_call(0, a, w, N, bias, scaled=scaled, out=out)
+            return
+        if scaled is not None:
+            self._whole(a)
+        self._scaled.pop(out.data_ptr(), None)
+        if accumulate:
+            self._source_changes(out)
         self._splits_out.value = 0
         self._check(self.lib.hfa_gemm(a.data_ptr(), _code(a), lda, w.data_ptr(), _code(w), ldw,
                                       None if bias is None else bias.data_ptr(), out.data_ptr(), _code(out), ldo,

@@ -8,6 +8,7 @@ import torch
 
 from .config import config_from_dict, read_config
 from .parts.base import FixedState, PagedKV
+from .parts.block import norm_for
 from .registry import architecture, make_part
 from .status import EINVAL, fail
 from .weights.loader import load_tensors
@@ -146,9 +147,12 @@ class Model:
             own = e.cache_of is None
             mine = {name: caches[k] for name, k in self.cache_slots[i if own else e.cache_of].items()}
             layer.block.forward(ops, step, x, layer.named, mine, write_cache=own)
-        ops.settle()
         R = step.n_logit_rows
         if R:
             h = ops.scratch("head_in", (R, self.hidden_size), ops.act_dtype)
-            self.final_norm.forward(ops, x, h, rows=step.logit_rows)      # src/model.c:629-636
+            if getattr(step, "rows_in_order", False):         # every token's logits, in order: no rows to gather
+                norm_for(ops, self.final_norm, self.head, x, h)
+            else:
+                self.final_norm.forward(ops, x, h, rows=step.logit_rows)      # src/model.c:629-636
             self.head.forward(ops, h, logits_out)
+        ops.settle()

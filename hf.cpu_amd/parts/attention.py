@@ -26,6 +26,7 @@ class Attention(Part):
     ``dot(q, k) * scale + score_slopes[h] * (pk - pq)``.
     """
     graph_safe = True
+    lazy_input_ok = True
 
 
     def __init__(self, hidden_size, n_heads, n_kv_heads, head_dim, qkv_bias, window, position,

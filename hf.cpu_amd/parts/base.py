@@ -56,6 +56,9 @@ class Part:
     # on its values (no host-side loop over the step's tokens, no read-back): only then may the
     # engine capture a step into a graph and replay it. Parts say so themselves; the default is no.
     graph_safe = False
+    # True if forward() reads its input activations (the norm's output it is handed) through ``ops.gemm`` alone: the
+    # block may then ask the norm in front of it to be lazy (``Ops.rmsnorm``), which saves a kernel in decode steps.
+    lazy_input_ok = False
 
     def __init__(self, prefix=""):
         self.prefix = prefix

@@ -17,9 +17,18 @@ class PreNormBlock(Part):
     def forward(self, ops, step, x, parts, caches, write_cache=True):
         """``parts``: norm1, mixer, norm2, feed_forward; ``caches``: the mixer's, under its name."""
         h = ops.scratch("normed", (x.shape[0], self.E), ops.act_dtype)
-        parts["norm1"].forward(ops, x, h)      # also adds up a product the previous part deferred into x
+        norm_for(ops, parts["norm1"], parts["mixer"], x, h)      # also adds up a product the previous part deferred into x
         ops.settle(x)                          # (nothing left to do unless the norm could not)
         parts["mixer"].forward(ops, step, h, caches.get("mixer"), x, write_cache)
-        parts["norm2"].forward(ops, x, h)
+        norm_for(ops, parts["norm2"], parts["feed_forward"], x, h)
         ops.settle(x)
         parts["feed_forward"].forward(ops, step, h, x)
+
+
+def norm_for(ops, norm, reader, x, out, rows=None):
+    """``out = norm(x)`` for the part ``reader``: lazily if the norm can be and the reader reads ``out`` through
+    ``ops.gemm`` alone."""
+    if getattr(norm, "can_be_lazy", False) and getattr(reader, "lazy_input_ok", False):
+        norm.forward(ops, x, out, rows, lazy=True)
+    else:
+        norm.forward(ops, x, out, rows)

@@ -31,6 +31,7 @@ class LinearHead(Part):
     matrix is the embedding table unless the checkpoint holds one of its own, which
     then wins (src/model.c:156-158)."""
     graph_safe = True
+    lazy_input_ok = True
 
 
     def __init__(self, vocab_size, hidden_size, tied, tied_to="", prefix=""):

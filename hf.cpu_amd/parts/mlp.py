@@ -14,6 +14,7 @@ class GatedMLP(Part):
     (src/model.c:612-623, src/mathx.c:34). Gate and up share their input and are held
     as one matrix, gate rows first."""
     graph_safe = True
+    lazy_input_ok = True
 
 
     def __init__(self, hidden_size, intermediate_size, activation="silu", prefix=""):

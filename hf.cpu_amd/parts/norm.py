@@ -8,6 +8,7 @@ class RMSNorm(Part):
     """``y_i = x_i * (1 / sqrt(mean(x^2) + eps)) * w_i`` with the mean of squares in
     fp32 (src/mathx.c:65-75; the reference sums in fp64)."""
     graph_safe = True
+    can_be_lazy = True          # forward(..., lazy=True) may leave the division to the products that read the output
 
 
     def __init__(self, size, eps, prefix=""):
@@ -22,6 +23,7 @@ class RMSNorm(Part):
     def bind(self, params, ops):
         self.weight = params[self.prefix + "weight"]
 
-    def forward(self, ops, x, out, rows=None):
-        """``out[r] = norm(x[rows[r]])`` (``rows`` None: every row in order)."""
-        ops.rmsnorm(x, self.weight, self.eps, out, rows)
+    def forward(self, ops, x, out, rows=None, lazy=False):
+        """``out[r] = norm(x[rows[r]])`` (``rows`` None: every row in order). ``lazy``: the caller promises that
+        ``out`` is read through ``ops.gemm`` alone (a part that says ``lazy_input_ok``); see ``Ops.rmsnorm``."""
+        ops.rmsnorm(x, self.weight, self.eps, out, rows, lazy=lazy)

@@ -183,6 +183,14 @@ def test_deferred_products_are_finished_by_the_next_kernel(ops16, M, K, E):
     """A product with few rows and a long K leaves partial sums (for 40 rows: the planes of the
     streamed product); the norm that follows adds them into the residual stream and norms the
     result; rope_store does the same for q, k and v."""
+    ops16.fuse_rows = False        # the chain of separate kernels (few rows otherwise take products that finish their outputs)
+    try:
+        _deferred_products(ops16, M, K, E)
+    finally:
+        ops16.fuse_rows = True
+
+
+def _deferred_products(ops16, M, K, E):
     rng = np.random.default_rng(0)
     a = rng.standard_normal((M, K)).astype(np.float32)
     w = (rng.standard_normal((E, K)) / 64).astype(np.float32)
@@ -226,6 +234,78 @@ def test_deferred_products_are_finished_by_the_next_kernel(ops16, M, K, E):
     assert np.max(np.abs(cache.k.float().cpu().numpy()[slot_map] - k_want)) < 0.05
     vc = from_value_layout(cache.v.float().cpu().numpy(), 4)
     assert np.max(np.abs(vc[slot_map] - full[:, (H + G) * D:])) < 0.05
+
+
+@pytest.mark.parametrize("M,K,E,N", [(1, 256, 128, 1000), (5, 4096, 896, 1152), (8, 18944, 3584, 4608), (16, 3584, 3584, 4100),
+                                     (11, 640, 2176, 77), (16, 1536, 8960, 333)])
+def test_products_of_few_rows_that_finish_their_outputs(ops16, M, K, E, N):
+    """Up to 16 rows: a product into the residual stream waits for the norm that follows; one kernel then does product,
+    residual sum, the sums of squares and x * weight, and the product that reads the norm's output scales its sums
+    (``Ops.rmsnorm(..., lazy=True)``). Against the same in float64: the residual stream, the product behind the
+    norm (into fp32, into bf16, and as the 32-bit plane that the rotation of queries and keys takes), gate and up
+    with the activation, and the norm's output made whole when something else asks for it."""
+    rng = np.random.default_rng(M + K)
+    bf = torch.bfloat16
+    a = rng.standard_normal((M, K)).astype(np.float32)
+    w = (rng.standard_normal((E, K)) / math.sqrt(K)).astype(np.float32)
+    b = rng.standard_normal(E).astype(np.float32)
+    x0 = rng.standard_normal((M, E)).astype(np.float32)
+    g = (1 + 0.1 * rng.standard_normal(E)).astype(np.float32)
+    w2 = (rng.standard_normal((N, E)) / math.sqrt(E)).astype(np.float32)
+    b2 = rng.standard_normal(N).astype(np.float32)
+    x_want = x0 + rounded(a, bf) @ rounded(w, bf).T + b
+    h_want = plain.rmsnorm(x_want, g, 1e-5)
+    out_want = h_want @ rounded(w2, bf).T + b2
+
+    def lazily():
+        x, h = dev(x0), torch.empty((M, E), dtype=bf, device="cuda")
+        ops16.gemm(dev(a, bf), dev(w, bf), x, bias=dev(b), accumulate=True, defer=True)
+        assert ops16._lazy is not None and ops16._pending is None
+        ops16.rmsnorm(x, dev(g), 1e-5, h, lazy=True)
+        assert ops16._lazy is None and h.data_ptr() in ops16._scaled
+        return x, h
+    x, h = lazily()
+    assert np.max(np.abs(x.cpu().numpy() - x_want)) < 2e-5 * max(1.0, np.max(np.abs(x_want)))
+    scale = np.max(np.abs(out_want))
+    for odt, tol in ((torch.float32, 6e-3), (bf, 1.2e-2)):
+        out = torch.empty((M, N), dtype=odt, device="cuda")
+        ops16.gemm(h, dev(w2, bf), out, bias=dev(b2))
+        assert np.max(np.abs(out.float().cpu().numpy() - out_want)) < tol * scale, str(odt)
+    if N % 8 == 0:                                         # deferred: a 32-bit plane for the kernel that follows
+        out = torch.empty((M, N), dtype=bf, device="cuda")
+        ops16.gemm(h, dev(w2, bf), out, bias=dev(b2), defer=True)
+        assert ops16._pending is not None and ops16._pending.splits == 1
+        ops16.settle()
+        assert np.max(np.abs(out.float().cpu().numpy() - out_want)) < 1.2e-2 * scale
+    # the norm's output made whole: what the plain norm kernel gives
+    ops16.settle(h)
+    assert h.data_ptr() not in ops16._scaled
+    assert np.max(np.abs(h.float().cpu().numpy() - h_want)) < 0.02 * np.max(np.abs(h_want))
+    # without the norm: the product alone (settled), the same residual stream bit for bit
+    x2 = dev(x0)
+    ops16.gemm(dev(a, bf), dev(w, bf), x2, bias=dev(b), accumulate=True, defer=True)
+    ops16.settle(x2)
+    assert torch.equal(x2, x)
+    # gate and up with the activation, from the lazy norm's output
+    F = (N + 31) // 32 * 32
+    wg, wu = ((rng.standard_normal((F, E)) / math.sqrt(E)).astype(np.float32) for _ in range(2))
+    x, h = lazily()
+    assert ops16.can_fuse_swiglu(dev(wg, bf), dev(wu, bf))
+    act = torch.empty((M, F), dtype=bf, device="cuda")
+    ops16.gemm(h, ops16.interleave_gate_up(dev(wg, bf), dev(wu, bf)), act, swiglu=True)
+    gt, up = h_want @ rounded(wg, bf).T, h_want @ rounded(wu, bf).T
+    act_want = plain.silu(gt) * up
+    assert np.max(np.abs(act.float().cpu().numpy() - act_want)) < 1.5e-2 * max(1.0, np.max(np.abs(act_want)))
+    # the same calls with the fusion off give the same values within bf16's rounding
+    ops16.fuse_rows = False
+    try:
+        x3, h3 = dev(x0), torch.empty((M, E), dtype=bf, device="cuda")
+        ops16.gemm(dev(a, bf), dev(w, bf), x3, bias=dev(b), accumulate=True, defer=True)
+        ops16.rmsnorm(x3, dev(g), 1e-5, h3, lazy=True)
+        assert h3.data_ptr() not in ops16._scaled
+        assert float((x3 - x).abs().max()) < 2e-5 * max(1.0, np.max(np.abs(x_want)))
+    finally:
+        ops16.fuse_rows = True
 
 
 def test_gemm_matches_library_product(ops32):

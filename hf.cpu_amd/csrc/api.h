@@ -98,6 +98,21 @@ int hfa_paged_attention(const void* q, int dtype, int ldq, const void* k_cache, 
                         int page_tokens, int window, float scale, const float* slopes, void* workspace,
                         size_t workspace_bytes, int force_plain, hipStream_t stream);
 
+// Decoded tokens (one a request) whose queries, new keys and new values are still the 32-bit rows [q | k | v] that
+// the product left (`raw`, bias added): rotation of queries and keys (cos_sin: hfa_rope_table's output for the step's
+// tokens, [token][head_dim / 2 cosines, head_dim / 2 sines]; null: none), the store of the new key and value into
+// cache rows slot_map[t], and attention over the cache, in one kernel (plus the merge of key chunks): what
+// hfa_rope_store and hfa_paged_attention give one after the other. bf16 cache, matrix cores only: ask
+// hfa_decode_attention_supports first.
+int hfa_rope_table(const int* positions, const float* inv_freq, int half, float* out, int n_tokens, hipStream_t stream);
+int hfa_decode_attention_supports(int n_heads, int n_kv_heads, int head_dim, int rot_dim, int page_tokens, int kv_width,
+                                  int ld_raw, int ldo);
+int hfa_decode_attention(const float* raw, int ld_raw, const float* cos_sin, void* k_cache, void* v_cache, int kv_width,
+                         const int* slot_map, const int* block_table, int max_blocks, const int* token_slot,
+                         const int* positions, const int* q_start, int n_seqs, int max_seq_len, void* out, int ldo,
+                         int n_heads, int n_kv_heads, int head_dim, int page_tokens, int window, float scale,
+                         void* workspace, size_t workspace_bytes, hipStream_t stream);
+
 // out[t, i] = silu(gate_up[t, i]) * gate_up[t, width + i].  (src/model.c:532-538)
 int hfa_swiglu(const void* gate_up, void* out, int dtype, int n_tokens, int width, hipStream_t stream);
 

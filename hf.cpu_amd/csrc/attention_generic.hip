@@ -129,6 +129,62 @@ int attn_generic_launch(const void* q, int dtype, int ldq, const void* k_cache, 
     return 0;
 }
 
+// cos_sin[t][0 .. half) = cos(positions[t] * inv_freq[i]), [half .. 2 half) the sines: the angles of src/model.c:472-476
+// as rope_store forms them, once for all the layers of a step.
+__global__ void rope_table_kernel(const int* __restrict__ positions, const float* __restrict__ inv_freq, int half,
+                                  float* __restrict__ out) {
+    const int t = blockIdx.x;
+    const float pos = (float)positions[t];
+    for (int i = threadIdx.x; i < half; i += blockDim.x) {
+        float sn, cs;
+        sincosf(pos * inv_freq[i], &sn, &cs);
+        out[(size_t)t * 2 * half + i] = cs;
+        out[(size_t)t * 2 * half + half + i] = sn;
+    }
+}
+
+extern "C" int hfa_rope_table(const int* positions, const float* inv_freq, int half, float* out, int n_tokens, hipStream_t stream) {
+    HFA_REQUIRE(positions && inv_freq && out && half > 0 && n_tokens > 0, "rope_table: bad arguments");
+    rope_table_kernel<<<n_tokens, half < 256 ? (half + 63) / 64 * 64 : 256, 0, stream>>>(positions, inv_freq, half, out);
+    HFA_LAUNCH_CHECK("rope_table");
+    return 0;
+}
+
+// Whether hfa_decode_attention takes a step: bf16 on the matrix cores, one head size of 32 to 128 in steps of 32
+// for keys and values, rotation of whole heads (rot_dim == head_dim) or none.
+extern "C" int hfa_decode_attention_supports(int n_heads, int n_kv_heads, int head_dim, int rot_dim, int page_tokens,
+                                             int kv_width, int ld_raw, int ldo) {
+    if (n_kv_heads <= 0 || n_heads % n_kv_heads != 0 || !(rot_dim == head_dim || rot_dim == 0) || ld_raw % 4 != 0) return 0;
+    AttnArgs a = {};
+    a.scale = 1.f; a.head_dim = head_dim; a.page_tokens = page_tokens; a.n_heads = n_heads; a.n_kv_heads = n_kv_heads;
+    a.q_start = (const int*)16; a.ldq = 8; a.ldo = ldo; a.kv_width = kv_width;
+    return attn_mfma_supports(a) ? 1 : 0;
+}
+
+// Attention of decoded tokens (one token a request) whose queries, new keys and new values are still the 32-bit rows
+// [q | k | v] that the product left (`raw`, row stride ld_raw, bias added): rotation of queries and keys, the store
+// of the new key and value into the cache rows slot_map[t], and attention over the cache in one kernel (and the merge
+// of the key chunks). cos_sin: hfa_rope_table's output for these tokens, or null for no rotation. Everything else as
+// in hfa_paged_attention, whose result with hfa_rope_store before it this equals.
+extern "C" int hfa_decode_attention(const float* raw, int ld_raw, const float* cos_sin, void* k_cache, void* v_cache,
+                                    int kv_width, const int* slot_map, const int* block_table, int max_blocks,
+                                    const int* token_slot, const int* positions, const int* q_start, int n_seqs,
+                                    int max_seq_len, void* out, int ldo, int n_heads, int n_kv_heads, int head_dim,
+                                    int page_tokens, int window, float scale, void* workspace, size_t workspace_bytes,
+                                    hipStream_t stream) {
+    HFA_REQUIRE(raw && k_cache && v_cache && slot_map && block_table && token_slot && positions && q_start && out,
+                "decode_attention: a null argument");
+    HFA_REQUIRE(n_seqs > 0 && max_seq_len > 0 && max_blocks > 0 && window >= 0, "decode_attention: bad sizes");
+    HFA_REQUIRE(ld_raw >= (n_heads + 2 * n_kv_heads) * head_dim && ldo >= n_heads * head_dim && kv_width >= n_kv_heads * head_dim,
+                "decode_attention: a row stride is smaller than its row");
+    AttnArgs a = {nullptr, 8, k_cache, v_cache, kv_width, block_table, max_blocks, token_slot, positions, q_start,
+                  n_seqs, 1, max_seq_len, out, ldo, n_seqs, n_heads, n_kv_heads, head_dim, page_tokens,
+                  window, scale, workspace, workspace_bytes, stream, raw, ld_raw, cos_sin, slot_map};
+    HFA_REQUIRE(((uintptr_t)raw & 15) == 0 && (cos_sin == nullptr || ((uintptr_t)cos_sin & 15) == 0) && attn_mfma_supports(a),
+                "decode_attention: this shape is not taken (see hfa_decode_attention_supports)");
+    return attn_mfma_launch(a);
+}
+
 extern "C" int hfa_paged_attention(const void* q, int dtype, int ldq, const void* k_cache, const void* v_cache,
                                    int kv_width, int v_width, const int* block_table, int max_blocks, const int* token_slot,
                                    const int* positions, const int* q_start, int n_seqs, int max_q_len,
@@ -146,7 +202,7 @@ extern "C" int hfa_paged_attention(const void* q, int dtype, int ldq, const void
     HFA_REQUIRE(dtype == HFA_F32 || dtype == HFA_BF16, "paged_attention: unknown dtype %d", dtype);
     AttnArgs a = {q, ldq, k_cache, v_cache, kv_width, block_table, max_blocks, token_slot, positions, q_start,
                   n_seqs, max_q_len, max_seq_len, out, ldo, n_tokens, n_heads, n_kv_heads, head_dim, page_tokens,
-                  window, scale, workspace, workspace_bytes, stream};
+                  window, scale, workspace, workspace_bytes, stream, nullptr, 0, nullptr, nullptr};
     // the matrix-core kernels take no slopes: scores with a position term go the plain way
     // and they know one head size and one row width for keys and values
     if (!force_plain && !slopes && dtype == HFA_BF16 && v_head_dim == head_dim && v_width == kv_width && attn_mfma_supports(a))

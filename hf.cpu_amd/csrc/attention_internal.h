@@ -13,6 +13,11 @@ struct AttnArgs {
     float scale;
     void* workspace; size_t workspace_bytes;
     hipStream_t stream;
+    // decoded tokens whose queries, new key and new value still lie in 32-bit rows [q | k | v] (see attn_mfma_kernel,
+    // FUSED): raw is null otherwise
+    const float* raw; int ld_raw;
+    const float* cos_sin;          // [token][head_dim / 2 cosines, head_dim / 2 sines], null: no rotation
+    const int* slot_map;           // the cache row of each token's key and value
 };
 
 int attn_generic_launch(const void* q, int dtype, int ldq, const void* k_cache, const void* v_cache, int kv_width,

@@ -64,13 +64,21 @@ union Frag {
     bf16x8 v;
 };
 
-template <int NDB, bool SPLIT>
+// FUSED (decoded tokens only, one token a tile): queries, the new key and the new value are not in `q` and in the
+// cache yet but in `raw`, fp32 rows [q | k | v] as the product left them (bias added). The wave rotates its queries
+// while it loads them (cosines and sines of the token's angles come from `cs`, [token][D / 2 cosines, D / 2 sines];
+// rot_dim = D, or no rotation when cs is null); the wave whose keys include the token's own position rotates the
+// new key, stores it and the new value into the cache (rows slot_map[token]) for the steps to come, and uses them
+// from LDS itself, since what the cache row held before is not the token's. What rope_store would have done in a
+// kernel and a pass over memory of its own.
+template <int NDB, bool SPLIT, bool FUSED>
 __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
     const uint16_t* __restrict__ q, int ldq, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc, int kvw,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ token_slot,
     const int* __restrict__ positions, const int* __restrict__ q_start, int n_seqs, uint16_t* __restrict__ out,
     int ldo, float* __restrict__ partial, int H, int psh, int window, float scale_log2e, int tpt, int cpt,
-    int chunk_keys, int n_chunks, int one_tile_each) {
+    int chunk_keys, int n_chunks, int one_tile_each, const float* __restrict__ raw, int ld_raw,
+    const float* __restrict__ cs, const int* __restrict__ slot_map, int G) {
     constexpr int D = NDB * 32, KS = D / 16;
     const int P = 1 << psh;                                // tokens per page, a power of two
     const int lane = threadIdx.x, col = lane & 31, half = lane >> 5;
@@ -116,12 +124,107 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
     // The query fragments stay in registers: read from LDS one by one before each product, they
     // cost an LDS round trip a product that a single wave on its SIMD has nothing to hide behind.
     Frag qf[KS];
-    {
+    __shared__ __attribute__((aligned(16))) uint16_t new_s[FUSED ? 2 * D : 8];     // the token's own key (rotated) and value
+    bool owns_new = false;                                 // this wave's keys include the token's own position
+    if (!FUSED) {
         const uint16_t* qp = q + (size_t)my_tok * ldq + my_head * D + half * 8;
 #pragma unroll
         for (int ks = 0; ks < KS; ks++)
             qf[ks].u = col_ok ? *reinterpret_cast<const uint4*>(qp + ks * 16) : make_uint4(0, 0, 0, 0);
     }
+    // FUSED: called once the first blocks of keys and values are on their way, so that the trip for the 32-bit rows
+    // is not a trip of its own at the head of the kernel
+    auto fused_prologue = [&]() {
+        // A head's fragments ks and ks + KS / 2 hold the two halves of its rotated pairs (i, i + D / 2), i = 16 ks + 8 half + e.
+        // Everything a pass needs from memory is asked for before anything is computed (left alone, the compiler asks,
+        // waits and computes fragment by fragment: eight trips to L2 one after the other), in two passes over the
+        // fragments so that the registers suffice.
+        const float* row = raw + (size_t)my_tok * ld_raw;
+        const float* qsrc = row + my_head * D + half * 8;
+        const float* ksrc = row + (H + g) * D + half * 8;
+        const float* cp = cs ? cs + (size_t)my_tok * D + half * 8 : nullptr;
+        owns_new = k_begin <= hi && hi <= k_end;            // uniform: hi is the token's own position
+        const int slot = owns_new ? slot_map[my_tok] : 0;
+        float vraw[NDB];
+        if (owns_new && half == 0) {
+#pragma unroll
+            for (int db = 0; db < NDB; db++) vraw[db] = row[(H + G) * D + g * D + 32 * db + col];
+        }
+        // (x0, x1) -> (x0 c - x1 s, x0 s + x1 c), src/model.c:488-490; without rotation the values pass as they are
+        auto lo_of = [&](float x0, float x1, float c, float s) { return cp ? x0 * c - x1 * s : x0; };
+        auto hi_of = [&](float x0, float x1, float c, float s) { return cp ? x0 * s + x1 * c : x1; };
+        auto two = [](float a, float b) { return (uint32_t)bf16_bits(a) | ((uint32_t)bf16_bits(b) << 16); };
+        auto turn = [&](const float4 (&lo)[2], const float4 (&hh)[2], const float4 (&c)[2], const float4 (&sn)[2], Frag& fl, Frag& fh) {
+            fl.u = make_uint4(two(lo_of(lo[0].x, hh[0].x, c[0].x, sn[0].x), lo_of(lo[0].y, hh[0].y, c[0].y, sn[0].y)),
+                              two(lo_of(lo[0].z, hh[0].z, c[0].z, sn[0].z), lo_of(lo[0].w, hh[0].w, c[0].w, sn[0].w)),
+                              two(lo_of(lo[1].x, hh[1].x, c[1].x, sn[1].x), lo_of(lo[1].y, hh[1].y, c[1].y, sn[1].y)),
+                              two(lo_of(lo[1].z, hh[1].z, c[1].z, sn[1].z), lo_of(lo[1].w, hh[1].w, c[1].w, sn[1].w)));
+            fh.u = make_uint4(two(hi_of(lo[0].x, hh[0].x, c[0].x, sn[0].x), hi_of(lo[0].y, hh[0].y, c[0].y, sn[0].y)),
+                              two(hi_of(lo[0].z, hh[0].z, c[0].z, sn[0].z), hi_of(lo[0].w, hh[0].w, c[0].w, sn[0].w)),
+                              two(hi_of(lo[1].x, hh[1].x, c[1].x, sn[1].x), hi_of(lo[1].y, hh[1].y, c[1].y, sn[1].y)),
+                              two(hi_of(lo[1].z, hh[1].z, c[1].z, sn[1].z), hi_of(lo[1].w, hh[1].w, c[1].w, sn[1].w)));
+        };
+        constexpr int HALF_KS = KS / 2, PASS = HALF_KS > 2 ? 2 : HALF_KS;         // fragments of a half head per pass
+        Frag kn[KS];
+#pragma unroll
+        for (int k0 = 0; k0 < HALF_KS; k0 += PASS) {
+            float4 c[PASS][2], sn[PASS][2], ql[PASS][2], qh[PASS][2], kl[PASS][2], kh[PASS][2];
+#pragma unroll
+            for (int j = 0; j < PASS; j++) {
+                const int ks = k0 + j;
+                if (ks < HALF_KS) {
+#pragma unroll
+                    for (int u = 0; u < 2; u++) {
+                        c[j][u] = make_float4(1.f, 1.f, 1.f, 1.f);
+                        sn[j][u] = make_float4(0.f, 0.f, 0.f, 0.f);
+                        if (cp) {
+                            c[j][u] = *reinterpret_cast<const float4*>(cp + ks * 16 + 4 * u);
+                            sn[j][u] = *reinterpret_cast<const float4*>(cp + D / 2 + ks * 16 + 4 * u);
+                        }
+                        ql[j][u] = *reinterpret_cast<const float4*>(qsrc + ks * 16 + 4 * u);
+                        qh[j][u] = *reinterpret_cast<const float4*>(qsrc + (ks + HALF_KS) * 16 + 4 * u);
+                        if (owns_new) {
+                            kl[j][u] = *reinterpret_cast<const float4*>(ksrc + ks * 16 + 4 * u);
+                            kh[j][u] = *reinterpret_cast<const float4*>(ksrc + (ks + HALF_KS) * 16 + 4 * u);
+                        }
+                    }
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int j = 0; j < PASS; j++) {
+                const int ks = k0 + j;
+                if (ks < HALF_KS) {
+                    turn(ql[j], qh[j], c[j], sn[j], qf[ks], qf[ks + HALF_KS]);
+                    if (owns_new) turn(kl[j], kh[j], c[j], sn[j], kn[ks], kn[ks + HALF_KS]);
+                }
+            }
+        }
+        if (!col_ok) {
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++) qf[ks].u = make_uint4(0, 0, 0, 0);
+        }
+        if (owns_new) {
+            const int P_ = 1 << psh;
+            if (col == 0) {                                  // every lane of a half computed the same key: one lane of each stores
+                uint16_t* dst = const_cast<uint16_t*>(kc) + (size_t)slot * kvw + g * D + half * 8;
+#pragma unroll
+                for (int ks = 0; ks < KS; ks++) {
+                    *reinterpret_cast<uint4*>(dst + ks * 16) = kn[ks].u;
+                    *reinterpret_cast<uint4*>(&new_s[ks * 16 + half * 8]) = kn[ks].u;
+                }
+            }
+            if (half == 0) {                                 // the value: dimension 32 db + col, transposed inside its page
+                uint16_t* vdst = const_cast<uint16_t*>(vc) + (size_t)(slot >> psh) * P_ * kvw + (slot & (P_ - 1));
+#pragma unroll
+                for (int db = 0; db < NDB; db++) {
+                    const uint16_t v = bf16_bits(vraw[db]);
+                    vdst[(size_t)(g * D + 32 * db + col) * P_] = v;
+                    new_s[D + 32 * db + col] = v;
+                }
+            }
+        }
+    };
     floatx16 o[NDB];
 #pragma unroll
     for (int db = 0; db < NDB; db++)
@@ -168,7 +271,13 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
     // One block of 32 keys in two halves, so that the registers of its keys can be refilled as
     // soon as the scores are formed: scores + online softmax, then weighted values.
     Frag pf[2];
-    auto scores = [&](int key0, const Frag (&kf)[KS]) {
+    auto scores = [&](int key0, Frag (&kf)[KS]) {
+        if (FUSED && owns_new && key0 <= hi && hi < key0 + KB) {       // the block of the token's own key (uniform)
+            if (key0 + col == hi) {
+#pragma unroll
+                for (int ks = 0; ks < KS; ks++) kf[ks].u = *reinterpret_cast<const uint4*>(&new_s[ks * 16 + half * 8]);
+            }
+        }
         floatx16 st;
 #pragma unroll
         for (int r = 0; r < 16; r++) st[r] = 0.f;
@@ -236,6 +345,24 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
     // whatever their last owner left, Inf and NaN included, and 0 x Inf is NaN. Their values are
     // replaced by zeros; only the first and the last block of a walk have such keys.
     auto values = [&](int key0, Frag (&vf)[NDB][2]) {
+        if (FUSED && owns_new && key0 <= hi && hi < key0 + KB) {       // the token's own value, in the run of four keys that holds it
+#pragma unroll
+            for (int kk = 0; kk < 2; kk++)
+#pragma unroll
+                for (int run = 0; run < 2; run++) {
+                    const int ka = key0 + 16 * kk + 8 * run + 4 * half;
+                    if (ka <= hi && hi < ka + 4) {
+                        const int e = hi - ka;
+#pragma unroll
+                        for (int db = 0; db < NDB; db++) {
+                            const uint32_t v = new_s[D + 32 * db + col];
+                            const uint32_t x = vf[db][kk].h[run].x, y = vf[db][kk].h[run].y;
+                            vf[db][kk].h[run].x = e == 0 ? (x & 0xffff0000u) | v : e == 1 ? (x & 0x0000ffffu) | (v << 16) : x;
+                            vf[db][kk].h[run].y = e == 2 ? (y & 0xffff0000u) | v : e == 3 ? (y & 0x0000ffffu) | (v << 16) : y;
+                        }
+                    }
+                }
+        }
         if (key0 < k_begin || key0 + KB - 1 > k_end) {         // uniform over the wave
 #pragma unroll
             for (int kk = 0; kk < 2; kk++)
@@ -292,6 +419,7 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
         load_v(at(wb), v0f);
         load_k(at(wb + 1), k1f);
         load_v(at(wb + 1), v1f);
+        if (FUSED && wb == 0) fused_prologue();
         for (int b = wb; b < we; b += 2) {
             scores(first + b * KB, k0f);
             load_k(at(b + 2), k0f);
@@ -755,17 +883,19 @@ template <int NDB>
 static int launch_ndb(const AttnArgs& a, int tiles, int tpt, int cpt, int chunk_keys, int n_chunks) {
     dim3 grid(tiles, a.n_kv_heads, n_chunks);
     const float sl = a.scale * 1.4426950408889634f;
-    if (n_chunks > 1)
-        attn_mfma_kernel<NDB, true><<<grid, WAVE, 0, a.stream>>>(
-            (const uint16_t*)a.q, a.ldq, (const uint16_t*)a.k_cache, (const uint16_t*)a.v_cache, a.kv_width,
-            a.block_table, a.max_blocks, a.token_slot, a.positions, a.q_start, a.n_seqs, (uint16_t*)a.out, a.ldo,
-            (float*)a.workspace, a.n_heads, page_shift(a.page_tokens), a.window, sl, tpt, cpt, chunk_keys, n_chunks,
-            a.max_q_len <= tpt);
-    else
-        attn_mfma_kernel<NDB, false><<<grid, WAVE, 0, a.stream>>>(
-            (const uint16_t*)a.q, a.ldq, (const uint16_t*)a.k_cache, (const uint16_t*)a.v_cache, a.kv_width,
-            a.block_table, a.max_blocks, a.token_slot, a.positions, a.q_start, a.n_seqs, (uint16_t*)a.out, a.ldo,
-            nullptr, a.n_heads, page_shift(a.page_tokens), a.window, sl, tpt, cpt, chunk_keys, n_chunks, a.max_q_len <= tpt);
+#define ATTN_ARGS(PARTIAL)                                                                                              \
+    (const uint16_t*)a.q, a.ldq, (const uint16_t*)a.k_cache, (const uint16_t*)a.v_cache, a.kv_width, a.block_table,      \
+        a.max_blocks, a.token_slot, a.positions, a.q_start, a.n_seqs, (uint16_t*)a.out, a.ldo, PARTIAL, a.n_heads,         \
+        page_shift(a.page_tokens), a.window, sl, tpt, cpt, chunk_keys, n_chunks, a.max_q_len <= tpt, a.raw, a.ld_raw,      \
+        a.cos_sin, a.slot_map, a.n_kv_heads
+    if (a.raw) {
+        if (n_chunks > 1) attn_mfma_kernel<NDB, true, true><<<grid, WAVE, 0, a.stream>>>(ATTN_ARGS((float*)a.workspace));
+        else attn_mfma_kernel<NDB, false, true><<<grid, WAVE, 0, a.stream>>>(ATTN_ARGS(nullptr));
+    } else {
+        if (n_chunks > 1) attn_mfma_kernel<NDB, true, false><<<grid, WAVE, 0, a.stream>>>(ATTN_ARGS((float*)a.workspace));
+        else attn_mfma_kernel<NDB, false, false><<<grid, WAVE, 0, a.stream>>>(ATTN_ARGS(nullptr));
+    }
+#undef ATTN_ARGS
     HFA_LAUNCH_CHECK("attn_mfma");
     return 0;
 }
@@ -844,7 +974,7 @@ int attn_mfma_launch(const AttnArgs& a) {
     // fill its tiles badly: those go to the kernel below, one wave per tile, which also cuts the keys.
     const long prompt_blocks = ((long)(a.n_tokens + 4 * tpt - 1) / (4 * tpt)) * a.n_kv_heads;
     const bool few_long = 8 * prompt_blocks < attn_cu_count() && a.max_seq_len >= 1024 && a.workspace != nullptr;
-    if (a.max_q_len >= PROMPT_ROWS && !few_long && a.page_tokens % 8 == 0 &&
+    if (a.raw == nullptr && a.max_q_len >= PROMPT_ROWS && !few_long && a.page_tokens % 8 == 0 &&
         (a.n_tokens + 4 * tpt - 1) / (4 * tpt) + a.n_seqs <= 65535) {
         switch (a.head_dim / 32) {
             case 1: return launch_prefill<1>(a, tpt, cpt);

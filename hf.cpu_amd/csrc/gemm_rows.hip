@@ -126,13 +126,27 @@ __global__ __launch_bounds__(RG_WAVES * WAVE) void gemm_rows_kernel(const RowGem
     // the row of A this lane reads (rows past the last one repeat it), and its 16 bytes of a 32-column step
     const uint32_t a_off = (uint32_t)((lane & 15) < p.T ? (lane & 15) : p.T - 1) * (uint32_t)p.lda * 2u + (uint32_t)(lane >> 4) * 16u;
 
-    // the shares of the sums of squares of the normed rows: thread (m = tid % 16, slice = tid / 16) adds the
-    // shares slice, slice + 32, ... here, ahead of every request below (the loads are the compiler's own)
-    float ssq_part = 0.f;
-    if (MODE != HFA_ROWS_RESID && p.ssq_in) {
-        for (int q = tid >> 4; q < p.parts_in; q += 32) ssq_part += p.ssq_in[q * 16 + (tid & 15)];
+    // What the last lines need from memory is asked for first and waited for last, so that it costs no trip of its
+    // own: the shares of the sums of squares of the normed rows (thread (m = tid % 16, slice = tid / 16) takes the
+    // shares slice, slice + 32, ..., eight at most: more shares than 256 are added up by the compiler's own loads
+    // below), or, for the residual sum, this thread's value of the residual stream (the first 512 outputs of the block).
+    float early[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) early[i] = 0.f;
+    if (MODE != HFA_ROWS_RESID) {
+        if (p.ssq_in) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const int q = (tid >> 4) + 32 * i;
+                const float* src = p.ssq_in + (q < p.parts_in ? q : 0) * 16 + (tid & 15);
+                asm volatile("global_load_dword %0, %1, off" : "=v"(early[i]) : "v"(src) : "memory");
+            }
+        }
+    } else {
+        const int tt = tid >> 8, m = (tid >> 4) & 15, col = own0 + 16 * tt + (tid & 15);
+        const float* src = p.x + (size_t)(m < p.T ? m : 0) * p.ldx + (col < own1 ? col : own0 < own1 ? own1 - 1 : 0);
+        asm volatile("global_load_dword %0, %1, off" : "=v"(early[0]) : "v"(src) : "memory");
     }
-    asm volatile("" ::"v"(ssq_part));
     float ssq_run = 0.f;                                                    // RESID: thread m's sum over the groups of tiles
 
     for (int tg0 = 0; tg0 < nt_all; tg0 += NT) {
@@ -206,6 +220,10 @@ __global__ __launch_bounds__(RG_WAVES * WAVE) void gemm_rows_kernel(const RowGem
             });
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        if (tg0 == 0) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) asm volatile("" : "+v"(early[i]));     // what was asked for first has landed too
+        }
         // ---- the waves' sums meet in LDS: [wave][tile][m][n], in the wave's own ring (free by now) ----
         // element r of a lane's accumulator: token 4 (lane / 16) + r, weight row lane % 16 of the tile
         float* red = reinterpret_cast<float*>(smem);
@@ -222,6 +240,12 @@ __global__ __launch_bounds__(RG_WAVES * WAVE) void gemm_rows_kernel(const RowGem
         float* behind = reinterpret_cast<float*>(smem) + RG_WAVES * RG_RING_FLOATS;     // LDS behind the rings
         if (tg0 == 0 && MODE != HFA_ROWS_RESID) {
             // r[m] from the shares: 32 slices per row, added in a fixed order
+            float ssq_part = 0.f;
+            if (p.ssq_in) {
+#pragma unroll
+                for (int i = 0; i < 8; i++) ssq_part += (tid >> 4) + 32 * i < p.parts_in ? early[i] : 0.f;
+                for (int q = (tid >> 4) + 256; q < p.parts_in; q += 32) ssq_part += p.ssq_in[q * 16 + (tid & 15)];
+            }
             behind[tid] = ssq_part;
             __syncthreads();
             if (tid < 16) {
@@ -260,7 +284,8 @@ __global__ __launch_bounds__(RG_WAVES * WAVE) void gemm_rows_kernel(const RowGem
                 const int tt = i >> 8, m = (i >> 4) & 15, n = i & 15, col = own0 + 16 * (tg0 + tt) + n;
                 float v = 0.f;
                 if (m < p.T && col < own1) {
-                    v = p.x[(size_t)m * p.ldx + col] + (total(tt, m, n) + (p.bias ? p.bias[col] : 0.f));
+                    const float was = (tg0 == 0 && i == tid) ? early[0] : p.x[(size_t)m * p.ldx + col];
+                    v = was + (total(tt, m, n) + (p.bias ? p.bias[col] : 0.f));
                     p.x[(size_t)m * p.ldx + col] = v;
                     if (p.xg) p.xg[(size_t)m * p.ldxg + col] = rg_bf16(v * p.g[col]);
                 }
@@ -314,12 +339,13 @@ static int rows_dispatch(const RowGemm& p, hipStream_t stream) {
     const int G = rows_cu_count();
     int nt = ((p.N + G - 1) / G + 15) / 16;                  // the most tiles a block has
     if (MODE == HFA_ROWS_SWIGLU) nt *= 2;
-    // tiles a wave takes at a time: the size that leaves the fewest repeated tiles, the larger one of equals
+    // tiles a wave takes at a time: few repeated tiles and few passes over K (a pass costs about what two tiles
+    // cost: its own ramp, and the waves' sums meeting at its end), the larger one of equals
     const int opts[] = {1, 2, 4, 6, 8, 10, 12};
     int best = 12, best_cost = 1 << 30;
     for (int o : opts) {
         if (MODE == HFA_ROWS_SWIGLU && (o & 1)) continue;
-        const int cost = (nt + o - 1) / o * o;
+        const int cost = (nt + o - 1) / o * (o + 2);
         if (cost < best_cost || (cost == best_cost && o > best)) { best = o; best_cost = cost; }
     }
     switch (best) {

@@ -22,6 +22,9 @@ _SIGNATURES = {
     "hfa_gemm_rows_supports": [I, I, I, I, I, I],
     "hfa_rope_store": [P, I, I, P, P, I, I, I, I, I, P, P, P, I, I, P, I, P, P],
     "hfa_paged_attention": [P, I, I, P, P, I, I, P, I, P, P, P, I, I, I, P, I, I, I, I, I, I, I, I, F, P, P, c_size_t, I, P],
+    "hfa_rope_table": [P, P, I, P, I, P],
+    "hfa_decode_attention_supports": [I, I, I, I, I, I, I, I],
+    "hfa_decode_attention": [P, I, P, P, P, I, P, P, I, P, P, P, I, I, P, I, I, I, I, I, I, F, P, c_size_t, P],
     "hfa_swiglu": [P, P, I, I, I, P],
     "hfa_scatter_i32": [P, P, P, I, P],
     "hfa_move_i32": [P, P, P, P, I, P],

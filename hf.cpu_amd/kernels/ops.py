@@ -69,6 +69,15 @@ class LazyProduct:
 
 
 @dataclass
+class LazyRope:
+    """A rotation of queries and keys and a store of keys and values that has not been launched: if attention over
+    the same rows of decoded tokens is asked for next, one kernel does all of it (``hfa_decode_attention``)."""
+    args: tuple              # what rope_store was called with
+    qkv: torch.Tensor
+    cache: object
+
+
+@dataclass
 class Scaled:
     """A norm's output that holds ``x * weight`` only, not yet divided by the root mean square: the products that
     read it scale their sums by ``rsqrt(sum(ssq) / width + eps)`` instead. ``x``, ``weight`` and ``eps`` make it whole
@@ -78,6 +87,7 @@ class Scaled:
     weight: torch.Tensor
     eps: float
     ssq: torch.Tensor
+    source_changed: bool = False       # x has gone on since: products may still read `out`, nothing can make it whole
 
 
 class _NoSection:
@@ -120,6 +130,7 @@ class Ops:
         self.lib = library()
         self.prompt_rows = int(self.lib.hfa_attention_prompt_rows())   # see StepInputs and paged_attention
         self._scratch = {}
+        self._shared = {}
         self._scratch_views = {}             # (name, shape, dtype) -> the view handed out last time
         self._stream_handle = None
         self.scratch_generation = 0
@@ -127,6 +138,8 @@ class Ops:
         self.attn_workspace = memory.empty(WORKSPACE_BYTES, torch.uint8, self.device, "workspace of attention")
         self._pending = None
         self._lazy = None                    # a LazyProduct
+        self._lazy_rope = None               # a LazyRope
+        self._rope_tables = {}               # (positions, frequencies, tokens) -> cosines and sines of a pass's angles
         self._scaled = {}                    # data_ptr of a norm's output -> Scaled
         self.rows_parts = int(self.lib.hfa_gemm_rows_parts())
         self.fuse_rows = True                # tests switch it off to compare with the chain of separate kernels
@@ -166,6 +179,7 @@ class Ops:
         before = self._stream_handle
         self._stream_handle = torch.cuda.current_stream(self.device).cuda_stream
         self._scaled.clear()                 # what an earlier pass left in its work buffers is of no use to this one
+        self._rope_tables.clear()
         try:
             yield self
         finally:
@@ -184,6 +198,12 @@ class Ops:
         if rc != 0:
             raise EngineError(EINVAL if rc == 1 else ENOTSUP,
                               f"{what or getattr(entry_point, '__name__', 'extension kernel')} returned {rc}")
+
+    def shared(self, key, make):
+        """A constant tensor that several parts want (``make()`` builds it the first time ``key`` is asked for)."""
+        if key not in self._shared:
+            self._shared[key] = make()
+        return self._shared[key]
 
     def scratch(self, name, shape, dtype):
         """A named work buffer that is reused from step to step; its contents are
@@ -265,6 +285,7 @@ class Ops:
         """Forgets a deferred product (after a step that failed: its partial sums are of no use)."""
         self._pending = None
         self._lazy = None
+        self._lazy_rope = None
         self._scaled.clear()
 
     # ---- products of few rows that finish their outputs themselves (csrc/gemm_rows.hip) -----------------------
@@ -309,22 +330,30 @@ class Ops:
         """Makes a norm's output that was left undivided (``Scaled``) whole before something other than ``gemm`` reads it."""
         sc = self._scaled.pop(t.data_ptr(), None)
         if sc is not None:
+            if sc.source_changed:
+                fail(EINVAL, "a norm's output that was asked for lazily is read by something other than a product after "
+                             "the normed tensor has changed: ask for the norm without lazy=True, or settle() its output first")
             self._check(self.lib.hfa_rmsnorm(sc.x.data_ptr(), sc.weight.data_ptr(), sc.out.data_ptr(), _code(sc.out), None,
                                              sc.out.shape[0], sc.out.shape[1], sc.eps, None, 0, None, self._stream()))
 
     def _source_changes(self, x, keep=None):
-        """``x`` is about to change: norm outputs that could only be made whole from it are made whole now (``keep``:
-        one that is about to be overwritten anyway is dropped instead)."""
+        """``x`` is about to change: norm outputs that were left undivided can no longer be made whole from it
+        (products can still read them: x * weight and the sums of squares stay). ``keep``: one that is about to be
+        overwritten is dropped."""
         for key, sc in list(self._scaled.items()):
             if sc.x.data_ptr() == x.data_ptr():
                 if keep is not None and key == keep.data_ptr():
                     del self._scaled[key]
                 else:
-                    self._whole(sc.out)
+                    sc.source_changed = True
 
     def settle(self, tensor=None):
         """Adds up a deferred product now (all of them if ``tensor`` is None, else only one that
         writes ``tensor``), and makes ``tensor`` whole if it is a norm's output that was left undivided."""
+        lr = self._lazy_rope
+        if lr is not None and (tensor is None or lr.qkv.data_ptr() == tensor.data_ptr()):
+            self._lazy_rope = None
+            self.rope_store(*lr.args, lazy=False)
         z = self._lazy
         if z is not None and (tensor is None or z.x.data_ptr() == tensor.data_ptr()):
             self._lazy = None
@@ -406,13 +435,24 @@ class Ops:
         return torch.stack([w_gate.view(F // 32, 32, E), w_up.view(F // 32, 32, E)], dim=1).reshape(2 * F, E).contiguous()
 
     def rope_store(self, qkv, positions, inv_freq, rot_dim, n_heads, n_kv_heads, head_dim, cache, slot_map,
-                   v_head_dim=None):
+                   v_head_dim=None, lazy=True):
         """Rotates q (and k) inside ``qkv`` and, if ``slot_map`` is given, stores k and v
         rows into ``cache.k`` / ``cache.v`` at the rows it names (values transposed inside
-        their page, see csrc/api.h). ``v_head_dim``: the size of a value head if it is not ``head_dim``."""
+        their page, see csrc/api.h). ``v_head_dim``: the size of a value head if it is not ``head_dim``.
+        When ``qkv`` is still the 32-bit plane that a product of few rows left and the shape allows it, the call
+        waits (``lazy``): attention over the same rows may take it along (``paged_attention``)."""
         v_head_dim = head_dim if v_head_dim is None else int(v_head_dim)
         row_width = (n_heads + n_kv_heads) * head_dim + n_kv_heads * v_head_dim
         pend = self._pending
+        if lazy and self.fuse_rows and pend is not None and pend.splits == 1 and pend.bias is None and not pend.accumulate \
+                and pend.out.data_ptr() == qkv.data_ptr() and pend.out.shape == qkv.shape and qkv.shape[1] == row_width \
+                and qkv.dtype == torch.bfloat16 and slot_map is not None and n_kv_heads and v_head_dim == head_dim \
+                and qkv.is_contiguous() and getattr(cache, "k", None) is not None and cache.k.dtype == torch.bfloat16 \
+                and self.lib.hfa_decode_attention_supports(n_heads, n_kv_heads, head_dim, rot_dim, cache.page_tokens,
+                                                           cache.k.shape[1], row_width, n_heads * head_dim):
+            self._lazy_rope = LazyRope((qkv, positions, inv_freq, rot_dim, n_heads, n_kv_heads, head_dim, cache, slot_map,
+                                        v_head_dim), qkv, cache)
+            return
         if pend is not None and not pend.accumulate and pend.out.data_ptr() == qkv.data_ptr() \
                 and pend.out.shape == qkv.shape and qkv.shape[1] == row_width:
             self._pending = None
@@ -450,8 +490,14 @@ class Ops:
         (fp32, one per query head): the score of key j for the query at p gets ``slopes[h] * (j - p)``
         added, for position encodings that enter the scores; the plain kernel then runs, as it does when
         value heads have a size of their own (``v_head_dim``; ``out`` then has that many columns a head)."""
-        self.settle()
         v_head_dim = head_dim if v_head_dim is None else int(v_head_dim)
+        lr = self._lazy_rope
+        if lr is not None and lr.qkv.data_ptr() == q.data_ptr() and lr.cache is cache and slopes is None \
+                and step.max_q_len == 1 and step.n_seqs == q.shape[0] and not self.force_plain_attention \
+                and out.dtype == torch.bfloat16 and v_head_dim == head_dim and lr.args[4:7] == (n_heads, n_kv_heads, head_dim) \
+                and cache.k.numel() < 1 << 32 and cache.k.shape[0] < 1 << 24:
+            return self._decode_attention(lr, step, window, scale, out)
+        self.settle()
         if slopes is not None and (slopes.dtype != torch.float32 or slopes.numel() != n_heads or not slopes.is_contiguous()
                                    or slopes.device != q.device):
             fail(EINVAL, "paged_attention: slopes must be contiguous fp32 on the device, one per query head")
@@ -490,6 +536,31 @@ class Ops:
             call(ts, T - ts, step.q_start_long, step.n_seqs - n_short, step.max_q_len)
         else:
             call(0, T, step.q_start, step.n_seqs, step.max_q_len)
+
+    def _decode_attention(self, lr, step, window, scale, out):
+        """Rotation, the store of the new keys and values and attention over the cache for decoded tokens, in one
+        kernel: the queued ``rope_store`` (``lr``) and this call together."""
+        qkv, positions, inv_freq, rot_dim, n_heads, n_kv_heads, head_dim, cache, slot_map, _ = lr.args
+        T = qkv.shape[0]
+        table = None
+        if rot_dim:
+            key = (positions.data_ptr(), inv_freq.data_ptr(), T, rot_dim)
+            table = self._rope_tables.get(key)
+            if table is None:                # the angles of this pass's tokens, once for all its layers
+                table = self.scratch(f"rope_table@{inv_freq.data_ptr()}", (T, rot_dim), torch.float32)
+                self._check(self.lib.hfa_rope_table(_ints(positions, "positions", T), inv_freq.data_ptr(), rot_dim // 2,
+                                                    table.data_ptr(), T, self._stream()))
+                self._rope_tables[key] = table
+        g = step.group(cache.group)
+        self._lazy_rope = None
+        self._pending = None                 # the 32-bit plane of q, k and v is read here
+        self._check(self.lib.hfa_decode_attention(
+            self.workspace.data_ptr(), qkv.shape[1], None if table is None else table.data_ptr(), cache.k.data_ptr(),
+            cache.v.data_ptr(), cache.k.shape[1], _ints(slot_map, "slot_map", T), g.block_table.data_ptr(),
+            g.block_table.shape[1], _ints(step.token_slot, "token_slot", T), _ints(step.positions, "positions", T),
+            _ints(step.q_start, "q_start", T + 1), T, step.max_seq_len, out.data_ptr(), _rows(out, "attention out"),
+            n_heads, n_kv_heads, head_dim, cache.page_tokens, int(window), float(scale), self.attn_workspace.data_ptr(),
+            self.attn_workspace.numel(), self._stream()))
 
     def swiglu(self, gate_up, out):
         self.settle()

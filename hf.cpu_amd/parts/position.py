@@ -32,9 +32,12 @@ class Rotary(Part):
         self.inv_freq = None
 
     def bind(self, params, ops):
-        i = torch.arange(self.rot_dim // 2, dtype=torch.float64)
-        inv = torch.pow(torch.tensor(self.theta, dtype=torch.float64), -2.0 * i / self.rot_dim)
-        self.inv_freq = memory.to_device(inv.to(torch.float32), ops.device, "rotary frequencies")
+        def table():
+            i = torch.arange(self.rot_dim // 2, dtype=torch.float64)
+            inv = torch.pow(torch.tensor(self.theta, dtype=torch.float64), -2.0 * i / self.rot_dim)
+            return memory.to_device(inv.to(torch.float32), ops.device, "rotary frequencies")
+        # layers with the same rotation share one table (and with it what a step derives from it once for all of them)
+        self.inv_freq = ops.shared(("rotary frequencies", self.rot_dim, self.theta), table)
 
     def store(self, ops, step, qkv, n_heads, n_kv_heads, cache, write, v_head_dim=None):
         """Rotates the queries (and keys) inside ``qkv`` at each token's position;

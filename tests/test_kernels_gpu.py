@@ -620,6 +620,71 @@ def test_paged_attention_large_pages_long_walks(ops16, H, G, D, page, window, n,
     assert np.max(np.abs(want[0, 0])) > 0.3                        # the far keys carry weight
 
 
+@pytest.mark.parametrize("H,G,D,page,window,rot,lengths", [
+    (28, 4, 128, 16, 0, True, [2100, 700, 64, 1500, 1, 17, 16, 33]),      # the 7B shape: keys in chunks, new keys at a page's first and last row
+    (14, 2, 64, 16, 0, True, [300, 2049, 5]),
+    (6, 2, 96, 8, 40, True, [100, 41, 40, 39, 7]),                         # a window; three fragments a half head
+    (3, 1, 32, 8, 0, True, [130, 9]),
+    (8, 8, 64, 64, 0, False, [200, 65, 64]),                               # no rotation; pages of 64
+    (28, 4, 128, 128, 300, True, [5000, 129, 128]),
+    (14, 2, 64, 16, 0, True, [40000, 12]),                                 # more pages than one window of page ids
+])
+def test_decoded_tokens_rotated_stored_and_attended_in_one_kernel(ops16, H, G, D, page, window, rot, lengths):
+    """Decoded tokens whose q, k and v are still the 32-bit plane a product left: ``rope_store`` waits and
+    ``paged_attention`` does rotation, the store of the new key and value, and attention in one kernel. Against float64
+    attention over the whole sequences (queries and keys rotated by the plain implementation), and against the two
+    kernels one after the other on the same plane: the same attention output within bf16's rounding, the same cache."""
+    from hf_cpu_amd.kernels.ops import Pending
+    rng = np.random.default_rng(H + D + len(lengths))
+    bf = torch.bfloat16
+    theta = 1e6
+    S = len(lengths)
+    ks, vs, cache, table = paged_setup(rng, lengths, G, D, page, bf)
+    raw = rng.standard_normal((S, (H + 2 * G) * D)).astype(np.float32)
+    positions = [n - 1 for n in lengths]
+    slot_rows = [int(table[s, (n - 1) // page].item()) * page + (n - 1) % page for s, n in enumerate(lengths)]
+    half = D // 2
+    inv = (theta ** (-2.0 * np.arange(half, dtype=np.float64) / D)).astype(np.float32)
+    # what the step should compute, in float64 on the values as they are rounded: the new key replaces the last row
+    wants = []
+    for s, n in enumerate(lengths):
+        q = raw[s, :H * D].reshape(1, H, D).astype(np.float64)
+        k_new = raw[s, H * D:(H + G) * D].reshape(1, G, D).astype(np.float64)
+        v_new = raw[s, (H + G) * D:].reshape(1, G, D).astype(np.float64)
+        if rot:
+            q, k_new = plain.rope(q, [n - 1], D, theta), plain.rope(k_new, [n - 1], D, theta)
+        k_all = np.concatenate([rounded(ks[s][:n - 1], bf), rounded(k_new, bf)])
+        v_all = np.concatenate([rounded(vs[s][:n - 1], bf), rounded(v_new, bf)])
+        wants.append(tail_attention(rounded(q, bf), k_all, v_all, window)[0])
+    want = np.stack(wants).reshape(S, H * D)
+    step = FakeStep(ints(positions), ints(list(range(S))), table, ints(slot_rows))
+    outs, caches = [], []
+    for fused in (True, False):
+        c = FakeCache(group=0, k=cache.k.clone(), v=cache.v.clone(), page_tokens=page, window=0)
+        qkv = torch.zeros((S, (H + 2 * G) * D), dtype=bf, device="cuda")
+        ops16.workspace[:raw.size * 4].view(torch.float32).copy_(dev(raw).view(-1))
+        ops16._pending = Pending(qkv, 1, None, False)
+        ops16.fuse_rows = fused
+        try:
+            ops16.rope_store(qkv, step.positions, dev(inv) if rot else None, D if rot else 0, H, G, D, c, step.group(0).slot_map)
+            assert (ops16._lazy_rope is not None) == fused
+            out = torch.empty((S, H * D), dtype=bf, device="cuda")
+            ops16.paged_attention(qkv, H, G, D, c, step, window, 1.0 / math.sqrt(D), out)
+            assert ops16._lazy_rope is None and ops16._pending is None
+        finally:
+            ops16.fuse_rows = True
+        outs.append(out.float().cpu().numpy())
+        caches.append((c.k.float().cpu().numpy(), c.v.float().cpu().numpy()))
+    for name, got in zip(("one kernel", "two kernels"), outs):
+        err = np.max(np.abs(got - want))
+        assert err <= 0.02, f"{name}: max |diff| {err:.3e}"
+    assert np.max(np.abs(outs[0] - outs[1])) <= 0.02
+    for a, b in zip(caches[0], caches[1]):                 # the same rows written, to a rounding of the rotation
+        assert np.max(np.abs(a - b)) <= 0.04 and np.mean(a != b) < 1e-3
+    k_rows = caches[0][0][slot_rows]
+    assert np.max(np.abs(k_rows - np.stack([w for w in (rounded(plain.rope(raw[s, H * D:(H + G) * D].reshape(1, G, D).astype(np.float64), [lengths[s] - 1], D, theta) if rot else raw[s, H * D:(H + G) * D].reshape(1, G, D), bf).reshape(G * D) for s in range(S))]))) <= 0.04
+
+
 def test_attention_special_cases(ops32):
     """A single query at position 0 returns value row 0 exactly; equal scores (zero query)
     return the mean of the visible value rows (softmax of equal numbers)."""

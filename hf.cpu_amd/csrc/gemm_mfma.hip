@@ -382,7 +382,8 @@ __global__ __launch_bounds__(WM* WN* WAVE) void gemm_dma_kernel(
         const uint32_t dst = lds0 + stage * C::STAGE_BYTES + request_no(i) * 1024;
         const bool is_a = request_no(i) * C::ROWS_PER_LOAD < BM;           // uniform over the wave
         const uint16_t* base = (is_a ? a_base : w_base) + (size_t)t * BK;
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(src[i]), "s"(base) : "m0");
+        uint64_t sbase;           // the address in registers that a scalar instruction wrote (gemm_rows.hip: hazards)
+        asm volatile("s_mov_b32 m0, %1\n\ts_mov_b64 %0, %3\n\tglobal_load_lds_dwordx4 %2, %0" : "=&s"(sbase) : "s"(dst), "v"(src[i]), "s"(base) : "m0");
     };
     // Piece offsets (in elements) of the 16-column steps of a tile for this lane's rows: the rows
     // a lane reads differ from lane % 32 by multiples of 32, so their swizzle is the lane's.

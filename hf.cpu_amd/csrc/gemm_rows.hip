@@ -54,14 +54,37 @@ struct RowGemm {
     uint16_t* act; int ldact;              // SWIGLU
 };
 
+// The requests below are written in assembly, and the compiler does not look into assembly for the machine's hazards.
+// One matters here: a memory instruction may read a scalar register no sooner than five wait states after a VECTOR
+// instruction wrote it (v_readlane, when the compiler brings back a scalar that it had put aside in the lanes of a
+// vector register; v_readfirstlane), and nothing makes the compiler keep that distance from a statement it cannot
+// read. So no memory instruction here reads a scalar operand of the statement: a scalar move copies it first (scalar
+// instructions wait for vector ones by themselves, and what a scalar instruction wrote may be read at once).
+//
 // A lane's 16 bytes of each of the four 32-column steps of a unit of K, straight into registers. The compiler takes
 // the registers as written when the statement ends: whoever uses them waits for the loads first and then passes
 // them through rg_landed.
 __device__ __forceinline__ void rg_load_a(u32x4 (&f)[4], uint32_t off, const uint16_t* base) {
-    asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(f[0]) : "v"(off), "s"(base) : "memory");
-    asm volatile("global_load_dwordx4 %0, %1, %2 offset:64" : "=v"(f[1]) : "v"(off), "s"(base) : "memory");
-    asm volatile("global_load_dwordx4 %0, %1, %2 offset:128" : "=v"(f[2]) : "v"(off), "s"(base) : "memory");
-    asm volatile("global_load_dwordx4 %0, %1, %2 offset:192" : "=v"(f[3]) : "v"(off), "s"(base) : "memory");
+    uint64_t b;
+    asm volatile("s_mov_b64 %4, %6\n\t"
+                 "global_load_dwordx4 %0, %5, %4\n\t"
+                 "global_load_dwordx4 %1, %5, %4 offset:64\n\t"
+                 "global_load_dwordx4 %2, %5, %4 offset:128\n\t"
+                 "global_load_dwordx4 %3, %5, %4 offset:192"
+                 : "=&v"(f[0]), "=&v"(f[1]), "=&v"(f[2]), "=&v"(f[3]), "=&s"(b) : "v"(off), "s"(base) : "memory");
+}
+// Four requests: 16 rows x 128 columns of K into 4 KB of LDS at dst (rows 0-7 and 8-15 of the first 64 columns, then
+// of the second 64): 64 lanes x 16 bytes = 8 rows of 128 bytes a request, to M0 + 16 * lane. (An `offset:` on the
+// instruction would move the place in LDS as well as the address, so the second half has a base of its own.)
+__device__ __forceinline__ void rg_request(const uint16_t* base, uint32_t off0, uint32_t off1, uint32_t dst) {
+    const uint16_t* base1 = base + 64;
+    uint64_t b0, b1;
+    asm volatile("s_mov_b32 m0, %2\n\ts_mov_b64 %0, %5\n\ts_mov_b64 %1, %6\n\t"
+                 "global_load_lds_dwordx4 %3, %0\n\t"
+                 "s_add_u32 m0, m0, 0x400\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %4, %0\n\t"
+                 "s_add_u32 m0, m0, 0x400\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %3, %1\n\t"
+                 "s_add_u32 m0, m0, 0x400\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %4, %1"
+                 : "=&s"(b0), "=&s"(b1) : "s"(dst), "v"(off0), "v"(off1), "s"(base), "s"(base1) : "m0", "scc", "memory");
 }
 __device__ __forceinline__ void rg_landed(u32x4 (&f)[4]) { asm volatile("" : "+v"(f[0]), "+v"(f[1]), "+v"(f[2]), "+v"(f[3])); }
 
@@ -174,13 +197,7 @@ __global__ __launch_bounds__(RG_WAVES * WAVE) void gemm_rows_kernel(const RowGem
         // of its unit of K, into register set `set`.
         auto issue = [&](int c, auto tt_c, auto set_c, int slot) {
             constexpr int tt = decltype(tt_c)::value, set = decltype(set_c)::value;
-            const uint16_t* base = p.W + (size_t)(wave + RG_WAVES * c) * 128;
-            const uint16_t* base1 = base + 64;
-            const uint32_t dst = lds0 + slot * (RG_UNIT * 2);
-            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(wrow[tt][0]), "s"(base) : "m0", "memory");
-            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst + 1024), "v"(wrow[tt][1]), "s"(base) : "m0", "memory");
-            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst + 2048), "v"(wrow[tt][0]), "s"(base1) : "m0", "memory");
-            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst + 3072), "v"(wrow[tt][1]), "s"(base1) : "m0", "memory");
+            rg_request(p.W + (size_t)(wave + RG_WAVES * c) * 128, wrow[tt][0], wrow[tt][1], lds0 + slot * (RG_UNIT * 2));
             if (tt == 0) rg_load_a(af[set], a_off, p.A + (size_t)(wave + RG_WAVES * c) * 128);
         };
         floatx4 acc[NT];

@@ -85,7 +85,8 @@ __global__ __launch_bounds__(WM* WN* WAVE) void gemm_stream_kernel(
         const uint32_t dst = lds0 + stage * C::STAGE_BYTES + (i * C::NW + wave) * 1024;
         const bool is_a = (i * C::NW + wave) * 8 < BM;       // uniform over the wave
         const uint16_t* base = is_a ? A + (size_t)req_kt * C::BK : W + (size_t)req_tile * BN * ldw + (size_t)req_kt * C::BK;
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(src[i]), "s"(base) : "m0");
+        uint64_t sbase;           // the address in registers that a scalar instruction wrote (gemm_rows.hip: hazards)
+        asm volatile("s_mov_b32 m0, %1\n\ts_mov_b64 %0, %3\n\tglobal_load_lds_dwordx4 %2, %0" : "=&s"(sbase) : "s"(dst), "v"(src[i]), "s"(base) : "m0");
     };
     auto requested = [&]() {
         if (++req_kt == nk) { req_kt = 0; req_tile++; }

@@ -89,12 +89,14 @@ __global__ __launch_bounds__(WAVES* WAVE) void gemm_wave_kernel(const uint16_t* 
         for (int q = 0; q < 4; q++) {
             const uint32_t dst = lds0 + (slot * UNIT + q * 512) * 2;
             const uint32_t off = last ? wsrc_last[q] : wsrc[q];
-            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(off), "s"(wbase) : "m0", "memory");
+            uint64_t sbase;           // the address in registers that a scalar instruction wrote (gemm_rows.hip: hazards)
+            asm volatile("s_mov_b32 m0, %1\n\ts_mov_b64 %0, %3\n\tglobal_load_lds_dwordx4 %2, %0" : "=&s"(sbase) : "s"(dst), "v"(off), "s"(wbase) : "m0", "memory");
         }
 #pragma unroll
         for (int q = 0; q < AR; q++) {
             const uint32_t dst = lds0 + (slot * UNIT + (4 + q) * 512) * 2;
-            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(asrc[q]), "s"(abase) : "m0", "memory");
+            uint64_t sbase;           // the address in registers that a scalar instruction wrote (gemm_rows.hip: hazards)
+            asm volatile("s_mov_b32 m0, %1\n\ts_mov_b64 %0, %3\n\tglobal_load_lds_dwordx4 %2, %0" : "=&s"(sbase) : "s"(dst), "v"(asrc[q]), "s"(abase) : "m0", "memory");
         }
     };
     // piece offsets (in elements) of the 16-column steps of a unit for this lane's row (rows differ from lane % 32

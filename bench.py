@@ -9,7 +9,8 @@ random ids were prefilled before; W steps are run untimed, then exactly K steps 
 between device synchronisations. One JSON line is printed: ``value`` is decoded tokens per
 second; ``prefill`` is one 2,048-token prompt in one step; ``roofline`` prices the decode
 step against HBM bandwidth (every weight it uses once, plus the cache of the live
-requests); ``points`` holds decode at batch 1 and 64. Peaks: HBM 8 TB/s, dense bf16 MFMA
+requests); ``points`` holds decode at batch 1, 64, 128 and 256 (tokens a second, and the fraction of
+the HBM peak that the step's bytes over its time come to). Peaks: HBM 8 TB/s, dense bf16 MFMA
 2.5 PFLOP/s, fp32 157.3 TFLOP/s. ``measured_peaks`` is what this device's own probes reach (a
 streaming read, a copy, the matrix cores on random and on all-zero operands); ``kernels`` prices
 every dominant part of the decode step (bytes / time) and of the prefill (flops / time) against both.
@@ -171,7 +172,7 @@ def main():
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--layers", type=int, default=0, help="run fewer layers than the shape has (0 = all)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
-    ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
+    ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1, 64, 128 and 256")
     ap.add_argument("--prefill-reps", type=int, default=3)
     ap.add_argument("--only", choices=["prefill", "decode"], default=None,
                     help="run one phase only and print a short line (for profiling a phase by itself)")
@@ -216,7 +217,8 @@ def main():
     cfg = hf_cpu_amd.config_from_dict(shape)
     short = "bf16" if args.dtype == "bfloat16" else "fp32"
     elem = 2 if short == "bf16" else 4
-    biggest = max(args.batch, 1 if args.no_points else 64)
+    point_batches = () if args.no_points or args.only else (1, 64, 128, 256)
+    biggest = max((args.batch,) + point_batches)
     t_load = time.perf_counter()
     s = S.Session(cfg, dtype=args.dtype, ctx_max=args.context + NEW, batch=PROMPT, page_size=PAGE, max_seqs=biggest,
                   kv_tokens=biggest * (args.context + NEW), seed=0)
@@ -312,12 +314,12 @@ def main():
     nbytes = decode_bytes(shape, elem, args.batch, mean_ctx)
     achieved = nbytes / (dt / args.steps) / 1e9
     points = {}
-    if not args.no_points:
-        for b in (1, 64):
-            k = min(args.steps, 32)
-            d = decode(b, k, min(args.warmup, 4))
-            points[f"decode_b{b}"] = round(b * k / d, 1)
-            print(f"[bench] decode batch {b}: {d / k * 1e3:.3f} ms/step", file=sys.stderr, flush=True)
+    for b in point_batches:
+        k, w = min(args.steps, 32), min(args.warmup, 4)
+        d = decode(b, k, w)
+        points[f"decode_b{b}"] = round(b * k / d, 1)
+        points[f"decode_b{b}_hbm_frac"] = round(decode_bytes(shape, elem, b, PROMPT + w + (k + 1) / 2.0) / (d / k) / HBM_PEAK, 4)
+        print(f"[bench] decode batch {b}: {d / k * 1e3:.3f} ms/step", file=sys.stderr, flush=True)
     flops = prefill_flops(shape, PROMPT)
     line = {
         "metric": "decode tok/s at batch 8 (Qwen2.5-7B shape, 2048-token prompts)" if args.batch == 8

@@ -176,12 +176,6 @@ int hfa_probe_read(const void* src, size_t bytes, void* sink, int blocks_per_cu,
 int hfa_probe_copy(const void* src, void* dst, size_t bytes, hipStream_t stream);
 int hfa_probe_mfma_threads(void);
 int hfa_probe_mfma(float* out, int iters, int zeros, double* flops, hipStream_t stream);
-// `rounds` barriers among hfa_probe_barrier_blocks() resident blocks (one a CU) with a value handed from
-// block to block across each: what a phase boundary inside one persistent kernel costs. state: counter,
-// error flag (set if a block waited too long: every block then leaves), count of wrong values; zeroed
-// by the caller. data: 2 * 64 * blocks unsigned.
-int hfa_probe_barrier_blocks(void);
-int hfa_probe_barrier(unsigned* state, unsigned* data, int rounds, hipStream_t stream);
 
 #ifdef __cplusplus
 }

@@ -74,45 +74,6 @@ __global__ __launch_bounds__(256) void probe_mfma_kernel(float* __restrict__ out
     out[(size_t)blockIdx.x * 256 + threadIdx.x] = v;
 }
 
-// What a step of one persistent kernel would cost in place of a kernel boundary: `rounds` times, every
-// block stores a value for a block of another XCD (write-through), all blocks meet at a barrier built
-// on one counter in device memory (every block adds one and polls until all have), and every block
-// reads its neighbour's value (past the caches). Each poll loop is bounded: a block that waits longer
-// than `spin_limit` polls sets *err and every block leaves. *bad counts values that arrived wrong.
-__global__ __launch_bounds__(256) void probe_barrier_kernel(unsigned* ctr, unsigned* err, unsigned* data, unsigned* bad,
-                                                           int rounds, int spin_limit) {
-    const int b = blockIdx.x, G = gridDim.x;
-    __shared__ int ok_s;
-    for (int it = 0; it < rounds; it++) {
-        unsigned* buf = data + (size_t)(it & 1) * G * 64;
-        if (threadIdx.x < 64)
-            __hip_atomic_store(buf + (size_t)b * 64 + threadIdx.x, (unsigned)(it * 1000 + b), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __builtin_amdgcn_s_waitcnt(0);                       // the stores are acknowledged
-        __syncthreads();
-        if (threadIdx.x == 0) {
-            __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            const unsigned target = (unsigned)(it + 1) * G;
-            int spins = 0, ok = 1;
-            while (__hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
-                __builtin_amdgcn_s_sleep(1);
-                if (++spins > spin_limit || __hip_atomic_load(err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) {
-                    __hip_atomic_store(err, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    ok = 0;
-                    break;
-                }
-            }
-            ok_s = ok;
-        }
-        __syncthreads();
-        if (!ok_s) return;
-        const int nb = (b + 37) % G;
-        if (threadIdx.x < 64) {
-            const unsigned v = __hip_atomic_load(buf + (size_t)nb * 64 + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            if (v != (unsigned)(it * 1000 + nb)) atomicAdd(bad, 1u);
-        }
-    }
-}
-
 static int probe_blocks(int per_cu) {
     int dev = 0, cus = 0;
     if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
@@ -144,17 +105,5 @@ extern "C" int hfa_probe_mfma(float* out, int iters, int zeros, double* flops, h
     probe_mfma_kernel<<<blocks, 256, 0, stream>>>(out, iters, zeros);
     HFA_LAUNCH_CHECK("probe_mfma");
     if (flops) *flops = (double)blocks * 4 /* waves */ * iters * 4.0 * (2.0 * 32 * 32 * 16);
-    return 0;
-}
-
-// state: 3 unsigned (counter, error flag, wrong values), zeroed by the caller; data: 2 * 64 * hfa_probe_barrier_blocks()
-// unsigned. One block a CU, so that all of them are resident at once (a barrier among blocks that wait for a
-// free CU would never be passed; the poll limit ends such a launch with *err set).
-extern "C" int hfa_probe_barrier_blocks(void) { return probe_blocks(1); }
-
-extern "C" int hfa_probe_barrier(unsigned* state, unsigned* data, int rounds, hipStream_t stream) {
-    HFA_REQUIRE(state && data && rounds > 0 && rounds <= 100000, "probe_barrier: needs its state, its data and 1 to 100000 rounds");
-    probe_barrier_kernel<<<probe_blocks(1), 256, 0, stream>>>(state, state + 1, data, state + 2, rounds, 1 << 20);
-    HFA_LAUNCH_CHECK("probe_barrier");
     return 0;
 }

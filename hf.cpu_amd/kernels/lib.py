@@ -37,7 +37,6 @@ _SIGNATURES = {
     "hfa_probe_read": [P, c_size_t, P, I, P],
     "hfa_probe_copy": [P, P, c_size_t, P],
     "hfa_probe_mfma": [P, I, I, P, P],
-    "hfa_probe_barrier": [P, P, I, P],
 }
 
 
@@ -57,8 +56,6 @@ def library():
             lib.hfa_order_rows_scratch.argtypes = [c_int, c_int]
             lib.hfa_gemm_rows_parts.restype = c_int
             lib.hfa_gemm_rows_parts.argtypes = []
-            lib.hfa_probe_barrier_blocks.restype = c_int
-            lib.hfa_probe_barrier_blocks.argtypes = []
             lib.hfa_probe_mfma_threads.restype = c_int
             lib.hfa_probe_mfma_threads.argtypes = []
             lib.hfa_attention_prompt_rows.restype = c_int

@@ -66,6 +66,7 @@ class LazyProduct:
     w: torch.Tensor
     x: torch.Tensor
     bias: object
+    section: object = None   # while timing: the section in which it was asked for (its time is booked there)
 
 
 @dataclass
@@ -108,6 +109,9 @@ class _Section:
         self.ops, self.name = ops, name
 
     def __enter__(self):
+        stack = self.ops._section_stack
+        self.parent = stack[-1] if stack else None
+        stack.append(self.name)
         self.start = torch.cuda.Event(enable_timing=True)
         self.start.record()
         return self
@@ -115,7 +119,8 @@ class _Section:
     def __exit__(self, *exc):
         end = torch.cuda.Event(enable_timing=True)
         end.record()
-        self.ops._sections.append((self.name, self.start, end))
+        self.ops._section_stack.pop()
+        self.ops._sections.append((self.name, self.start, end, self.parent))
         return False
 
 
@@ -144,7 +149,8 @@ class Ops:
         self.rows_parts = int(self.lib.hfa_gemm_rows_parts())
         self.fuse_rows = True                # tests switch it off to compare with the chain of separate kernels
         self._splits_out = ctypes.c_int(0)
-        self._sections = None                # while timing: (name, start event, end event) of every section left
+        self._sections = None                # while timing: (name, start event, end event, enclosing section) of every section left
+        self._section_stack = []
         self.force_plain_gemm = False        # tests set these to compare the matrix-core paths with the plain ones
         self.force_plain_attention = False
 
@@ -156,14 +162,18 @@ class Ops:
 
     def timing(self, on):
         self._sections = [] if on else None
+        self._section_stack = []
 
     def take_times(self):
         """Milliseconds per section name since the last call; waits for the device."""
         out = {}
         if self._sections:
             torch.cuda.synchronize(self.device)
-            for name, start, end in self._sections:
-                out[name] = out.get(name, 0.0) + start.elapsed_time(end)
+            for name, start, end, parent in self._sections:
+                ms = start.elapsed_time(end)
+                out[name] = out.get(name, 0.0) + ms
+                if parent is not None and parent != "total":       # (what "total" encloses is taken off it by the caller)
+                    out[parent] = out.get(parent, 0.0) - ms
             self._sections = []
         return out
 
@@ -321,7 +331,15 @@ class Ops:
             self._stream()))
 
     def _rows_resid(self, z, g=None, xg=None, ssq=None):
-        """Launches a LazyProduct; with ``g`` and ``xg`` the kernel also leaves ``xg = x * g`` and the sums of squares."""
+        """Launches a LazyProduct; with ``g`` and ``xg`` the kernel also leaves ``xg = x * g`` and the sums of squares.
+        While timing, its time goes to the section in which the product was asked for, not to the one that launches it."""
+        if self._sections is not None and z.section is not None and \
+                (not self._section_stack or self._section_stack[-1] != z.section):
+            with _Section(self, z.section):
+                return self._rows_resid_now(z, g, xg, ssq)
+        return self._rows_resid_now(z, g, xg, ssq)
+
+    def _rows_resid_now(self, z, g, xg, ssq):
         if ssq is None:
             ssq = self.scratch("ssq@none", (self.rows_parts * 16,), torch.float32)
         self._rows_call(1, z.a, z.w, z.w.shape[0], z.bias, x=z.x, ssq_out=ssq, g=g, xg=xg)
@@ -391,7 +409,7 @@ class Ops:
         if mode is not None and not (mode == 1 and scaled is not None):
             self._scaled.pop(out.data_ptr(), None)
             if mode == 1:                            # into the residual stream
-                z = LazyProduct(a, w, out, bias)
+                z = LazyProduct(a, w, out, bias, self._section_stack[-1] if self._section_stack else None)
                 if defer:
                     self._lazy = z                   # the next norm of `out` may take it along
                 else:

@@ -25,11 +25,9 @@ def _timed(fn, reps):
 
 
 def measure_peaks(ops, read_bytes=2 << 30, reps=5, mfma_iters=1 << 15):
-    """{"hbm_read_GBps", "hbm_copy_GBps", "mfma_bf16_TFLOPs", "mfma_bf16_zero_TFLOPs", "grid_barrier_us"}: a
+    """{"hbm_read_GBps", "hbm_copy_GBps", "mfma_bf16_TFLOPs", "mfma_bf16_zero_TFLOPs"}: a
     flat read of ``read_bytes`` (far more than the caches hold), a copy of half as much (bytes read plus
-    bytes written count), the matrix cores on random and on all-zero register operands, and what a
-    barrier among one resident block per CU costs with a value handed across it (the price of a phase
-    boundary inside one persistent kernel, to set beside the few microseconds of a kernel boundary)."""
+    bytes written count), and the matrix cores on random and on all-zero register operands."""
     lib = ops.lib
     stream = lambda: torch.cuda.current_stream(ops.device).cuda_stream
 
@@ -55,18 +53,4 @@ def measure_peaks(ops, read_bytes=2 << 30, reps=5, mfma_iters=1 << 15):
     for key, zeros in (("mfma_bf16_TFLOPs", 0), ("mfma_bf16_zero_TFLOPs", 1)):
         ms = _timed(lambda: check(lib.hfa_probe_mfma(acc.data_ptr(), mfma_iters, zeros, ctypes.byref(flops), stream())), reps)
         out[key] = round(flops.value / ms / 1e9, 1)
-    # a barrier among one resident block per CU, with a value handed across it
-    blocks = int(lib.hfa_probe_barrier_blocks())
-    state = torch.zeros(3, dtype=torch.int32, device=ops.device)
-    data = torch.zeros(2 * 64 * blocks, dtype=torch.int32, device=ops.device)
-    rounds = 500
-
-    def barrier():
-        state.zero_()
-        check(lib.hfa_probe_barrier(state.data_ptr(), data.data_ptr(), rounds, stream()))
-    ms = _timed(barrier, 3)
-    flags = state.cpu().tolist()
-    if flags[1] or flags[2]:
-        raise EngineError(EINVAL, f"the barrier probe failed: gave up waiting {flags[1]}, wrong values {flags[2]}")
-    out["grid_barrier_us"] = round(ms * 1e3 / rounds, 2)
     return out

@@ -1009,15 +1009,13 @@ def test_kernels_refuse_what_they_cannot_do(ops32):
 
 
 def test_probes_of_the_device_peaks(ops16):
-    """The bench's yardsticks: a streaming read, a copy, the matrix cores on random and on zero operands,
-    a barrier among resident blocks. Sanity of the numbers, not their size: a read faster than the
-    published peak, a burn slower with zeros than with random operands, or a barrier that gave up or
-    handed on wrong values would mean a broken probe."""
+    """The bench's yardsticks: a streaming read, a copy, the matrix cores on random and on zero operands.
+    Sanity of the numbers, not their size: a read faster than the published peak or a burn slower with zeros
+    than with random operands would mean a broken probe."""
     from hf_cpu_amd.probe import measure_peaks
     p = measure_peaks(ops16, read_bytes=256 << 20, reps=3, mfma_iters=1 << 12)
     assert 1000 < p["hbm_copy_GBps"] and 1000 < p["hbm_read_GBps"] < 8000
     assert 200 < p["mfma_bf16_TFLOPs"] <= p["mfma_bf16_zero_TFLOPs"] * 1.05 < 2700
-    assert 0.5 < p["grid_barrier_us"] < 50
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 4608, 3584), (8, 3584, 18944), (3, 2016, 896), (9, 37888, 3584), (16, 1000, 1024),

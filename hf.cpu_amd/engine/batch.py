@@ -34,7 +34,7 @@ class StepInputs:
     token's request), q_start[S + 1] (token range of each request), seq_slot[S],
     seq_len[S] (the request's length after this step), logit_rows[R].
 
-    Requests that bring few tokens (fewer than ``Ops.prompt_rows``: decoded tokens, ends of prompts)
+    Requests that bring few tokens (fewer than the model's ``short_request_rows``, which a part sets: decoded tokens, ends of prompts)
     come first in a step: the first ``n_short_seqs`` requests with ``n_short_tokens`` tokens, none
     of them more than ``max_short_q_len``. ``q_start_long`` is ``q_start`` of the remaining requests
     counted from their first token, so that a kernel can be given either part as a step of its own.

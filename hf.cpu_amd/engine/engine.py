@@ -40,6 +40,7 @@ class Engine:
         self.storage = CacheStorage(self.manager, model.dtype, ops.device)
         self.staging = IntStaging(ops.device)
         self.vocab_size = model.vocab_size
+        self._short_rows = int(getattr(model, "short_request_rows", 0))      # see _inputs
         self.steps_run = 0
         self.use_graphs = bool(graphs) and bool(getattr(model, "graph_safe", False))
         self._graphs = {}
@@ -306,7 +307,7 @@ class Engine:
         at = 0
         max_q = max_len = 0
         # Requests with few tokens first (see StepInputs); logits keep the order of the entries.
-        few = self.ops.prompt_rows
+        few = self._short_rows
         order = sorted(range(S), key=lambda i: len(entries[i].tokens) >= few)
         n_short = n_short_tokens = max_short = 0
         for s, i in enumerate(order):

@@ -89,6 +89,12 @@ class Model:
             parts.extend(layer.parts())
         return parts + [self.final_norm, self.head]
 
+    @property
+    def short_request_rows(self):
+        """Requests that bring fewer tokens than this to a step are laid first in it (0: no such line): the largest
+        that a part asks for (``Part.short_request_rows``)."""
+        return max([getattr(p, "short_request_rows", 0) for p in self._all_parts()] + [0])
+
     def param_specs(self):
         specs, seen = [], set()
         for p in self._all_parts():

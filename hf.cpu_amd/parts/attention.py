@@ -77,6 +77,7 @@ class Attention(Part):
         if self.qkv_bias:
             self.b_qkv = memory.cat([params[p + n + "_proj.bias"] for n in "qkv"], 0, f"{p}q, k and v biases in one vector")
         self.w_o = params[p + "o_proj.weight"]
+        self.short_request_rows = ops.prompt_rows     # where the attention kernels for decoded tokens and for prompt portions part
         if self.out_bias:
             self.b_o = params[p + "o_proj.bias"]
 

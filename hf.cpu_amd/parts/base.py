@@ -59,6 +59,10 @@ class Part:
     # True if forward() reads its input activations (the norm's output it is handed) through ``ops.gemm`` alone: the
     # block may then ask the norm in front of it to be lazy (``Ops.rmsnorm``), which saves a kernel in decode steps.
     lazy_input_ok = False
+    # A part whose kernels treat requests that bring fewer than this many tokens to a step differently from the
+    # others (decoded tokens beside prompt portions) says so here: the step function then lays those requests first
+    # (``StepInputs.n_short_seqs``), so that the part can take the two groups as steps of their own. 0: no such line.
+    short_request_rows = 0
 
     def __init__(self, prefix=""):
         self.prefix = prefix

@@ -46,10 +46,10 @@ struct RowGemm {
     const uint16_t* W; int ldw;            // weights, bf16 [rows][K]
     int T, N, K;                           // N: outputs (features for SWIGLU)
     const float* bias;                     // [N] or null
-    const float* ssq_in; int parts_in;     // [parts_in][16] shares of the sums of squares of the normed rows, or null
+    const float* ssq_in; int parts_in;     // [parts_in][16 or 32] shares of the sums of squares of the normed rows (32 from 17 rows up), or null
     float inv_width, eps;                  // r[m] = rsqrt(sum * inv_width + eps)
     void* out; int ldo; int out_bf16;      // OUT
-    float* x; int ldx; float* ssq_out;     // RESID: residual stream; [gridDim.x][16] shares of the sums of squares
+    float* x; int ldx; float* ssq_out;     // RESID: residual stream; [gridDim.x][16 or 32] shares of the sums of squares
     const float* g; uint16_t* xg; int ldxg;   // RESID: the next norm's weight and x * g in bf16 (or null)
     uint16_t* act; int ldact;              // SWIGLU
 };
@@ -103,22 +103,24 @@ __device__ __forceinline__ void rg_wait() {                  // at most N reques
 }
 
 // Requests newer than those of unit u when it is waited for, in the steady state: the R - 1 units after it, four
-// requests each, and four more for every one of them that begins a unit of K (it brings that unit's activations).
-template <int NT, int TT>
+// requests each, and 4 MT more for every one of them that begins a unit of K (it brings that unit's activations).
+template <int NT, int TT, int MT>
 constexpr int rg_newer() {
     int n = 0;
-    for (int j = 1; j < RG_R; j++) n += 4 + ((TT + j) % NT == 0 ? 4 : 0);
+    for (int j = 1; j < RG_R; j++) n += 4 + ((TT + j) % NT == 0 ? 4 * MT : 0);
     return n;
 }
 
 __device__ __forceinline__ uint16_t rg_bf16(float v) { return bf16_bits(v); }
 
 // NT: tiles of 16 weight rows a wave accumulates at a time (even for SWIGLU: gate and up tiles alternate);
-// AD: register sets of activations (units of K that may be on their way or in use at once).
-template <int NT, int AD, int MODE>
+// AD: register sets of activations (units of K that may be on their way or in use at once); MT: tiles of 16 rows of
+// activations (1 for up to 16 rows, 2 for up to 32: every unit of weights that has come through LDS is then used twice).
+template <int NT, int AD, int MODE, int MT>
 __global__ __launch_bounds__(RG_WAVES * WAVE) void gemm_rows_kernel(const RowGemm p) {
     extern __shared__ __attribute__((aligned(1024))) uint16_t smem[];
-    __shared__ float r_s[16];
+    constexpr int MR = 16 * MT;                                            // rows of activations the kernel holds
+    __shared__ float r_s[MR];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int G = gridDim.x, b = blockIdx.x;
     const int own0 = (int)((long long)b * p.N / G), own1 = (int)((long long)(b + 1) * p.N / G);
@@ -146,27 +148,34 @@ __global__ __launch_bounds__(RG_WAVES * WAVE) void gemm_rows_kernel(const RowGem
         const int n = lane & 15, pc = 4 * (s & 1) + (lane >> 4);
         frag_off[s] = ((s >> 1) * 16 + n) * 64 + ((pc ^ ((n >> 1) & 7)) * 8);
     }
-    // the row of A this lane reads (rows past the last one repeat it), and its 16 bytes of a 32-column step
-    const uint32_t a_off = (uint32_t)((lane & 15) < p.T ? (lane & 15) : p.T - 1) * (uint32_t)p.lda * 2u + (uint32_t)(lane >> 4) * 16u;
+    // the rows of A this lane reads (rows past the last one repeat it), and its 16 bytes of a 32-column step
+    uint32_t a_off[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; mt++) {
+        const int row = 16 * mt + (lane & 15);
+        a_off[mt] = (uint32_t)(row < p.T ? row : p.T - 1) * (uint32_t)p.lda * 2u + (uint32_t)(lane >> 4) * 16u;
+    }
 
     // What the last lines need from memory is asked for first and waited for last, so that it costs no trip of its
-    // own: the shares of the sums of squares of the normed rows (thread (m = tid % 16, slice = tid / 16) takes the
-    // shares slice, slice + 32, ..., eight at most: more shares than 256 are added up by the compiler's own loads
-    // below), or, for the residual sum, this thread's value of the residual stream (the first 512 outputs of the block).
-    float early[8];
+    // own: the shares of the sums of squares of the normed rows ([share][MR]; thread (m = tid % MR, slice = tid / MR)
+    // takes the shares slice, slice + SL, ..., EARLY at most, which covers 256 shares: more are added up by the
+    // compiler's own loads below), or, for the residual sum, this thread's value of the residual stream (the first
+    // 512 values of the block's outputs).
+    constexpr int SL = RG_WAVES * WAVE / MR, EARLY = 8 * MT;               // slices of shares; early loads a thread
+    float early[EARLY];
 #pragma unroll
-    for (int i = 0; i < 8; i++) early[i] = 0.f;
+    for (int i = 0; i < EARLY; i++) early[i] = 0.f;
     if (MODE != HFA_ROWS_RESID) {
         if (p.ssq_in) {
 #pragma unroll
-            for (int i = 0; i < 8; i++) {
-                const int q = (tid >> 4) + 32 * i;
-                const float* src = p.ssq_in + (q < p.parts_in ? q : 0) * 16 + (tid & 15);
+            for (int i = 0; i < EARLY; i++) {
+                const int q = tid / MR + SL * i;
+                const float* src = p.ssq_in + (q < p.parts_in ? q : 0) * MR + (tid % MR);
                 asm volatile("global_load_dword %0, %1, off" : "=v"(early[i]) : "v"(src) : "memory");
             }
         }
     } else {
-        const int tt = tid >> 8, m = (tid >> 4) & 15, col = own0 + 16 * tt + (tid & 15);
+        const int tt = tid / (16 * MR), m = (tid >> 4) % MR, col = own0 + 16 * tt + (tid & 15);
         const float* src = p.x + (size_t)(m < p.T ? m : 0) * p.ldx + (col < own1 ? col : own0 < own1 ? own1 - 1 : 0);
         asm volatile("global_load_dword %0, %1, off" : "=v"(early[0]) : "v"(src) : "memory");
     }
@@ -192,17 +201,22 @@ __global__ __launch_bounds__(RG_WAVES * WAVE) void gemm_rows_kernel(const RowGem
                 }
                 wrow[tt][h] = (uint32_t)row * (uint32_t)p.ldw * 2u + req_piece[h];
             }
-        u32x4 af[AD][4];
+        u32x4 af[AD][MT][4];
         // Unit (c, tt): tile tt of this wave's c-th unit of K. The unit with tt == 0 also brings the activations
         // of its unit of K, into register set `set`.
         auto issue = [&](int c, auto tt_c, auto set_c, int slot) {
             constexpr int tt = decltype(tt_c)::value, set = decltype(set_c)::value;
             rg_request(p.W + (size_t)(wave + RG_WAVES * c) * 128, wrow[tt][0], wrow[tt][1], lds0 + slot * (RG_UNIT * 2));
-            if (tt == 0) rg_load_a(af[set], a_off, p.A + (size_t)(wave + RG_WAVES * c) * 128);
-        };
-        floatx4 acc[NT];
+            if (tt == 0) {
 #pragma unroll
-        for (int t = 0; t < NT; t++) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+                for (int mt = 0; mt < MT; mt++) rg_load_a(af[set][mt], a_off[mt], p.A + (size_t)(wave + RG_WAVES * c) * 128);
+            }
+        };
+        floatx4 acc[NT][MT];
+#pragma unroll
+        for (int t = 0; t < NT; t++)
+#pragma unroll
+            for (int mt = 0; mt < MT; mt++) acc[t][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
         const int n_units = nkw * NT;
         rg_static_for<0, RG_R>([&](auto v_c) {                   // the first R units
             constexpr int v = decltype(v_c)::value;
@@ -219,15 +233,20 @@ __global__ __launch_bounds__(RG_WAVES * WAVE) void gemm_rows_kernel(const RowGem
                         const int u = c * NT + tt;
                         // the unit has landed when at most the requests of the R - 1 units after it are out; at the
                         // run's end fewer are out than that, and all of them are waited for
-                        if (u + RG_R <= n_units) rg_wait<rg_newer<NT, tt>()>(); else rg_wait<0>();
-                        if (tt == 0) rg_landed(af[cc]);
+                        if (u + RG_R <= n_units) rg_wait<rg_newer<NT, tt, MT>()>(); else rg_wait<0>();
+                        if (tt == 0) {
+#pragma unroll
+                            for (int mt = 0; mt < MT; mt++) rg_landed(af[cc][mt]);
+                        }
                         const uint16_t* base = ring + slot * RG_UNIT;
                         bf16x8 fw[4];
 #pragma unroll
                         for (int s = 0; s < 4; s++) fw[s] = *reinterpret_cast<const bf16x8*>(base + frag_off[s]);
 #pragma unroll
                         for (int s = 0; s < 4; s++)
-                            acc[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, af[cc][s]), fw[s], acc[tt], 0, 0, 0);
+#pragma unroll
+                            for (int mt = 0; mt < MT; mt++)
+                                acc[tt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, af[cc][mt][s]), fw[s], acc[tt][mt], 0, 0, 0);
                         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the fragments are read: the slot may be filled again
                         if (u + RG_R < n_units)
                             issue(c + (tt + RG_R) / NT, rg_int<(tt + RG_R) % NT>{}, rg_int<(cc + (tt + RG_R) / NT) % AD>{}, slot);
@@ -239,35 +258,55 @@ __global__ __launch_bounds__(RG_WAVES * WAVE) void gemm_rows_kernel(const RowGem
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         if (tg0 == 0) {
 #pragma unroll
-            for (int i = 0; i < 8; i++) asm volatile("" : "+v"(early[i]));     // what was asked for first has landed too
+            for (int i = 0; i < EARLY; i++) asm volatile("" : "+v"(early[i]));     // what was asked for first has landed too
         }
-        // ---- the waves' sums meet in LDS: [wave][tile][m][n], in the wave's own ring (free by now) ----
-        // element r of a lane's accumulator: token 4 (lane / 16) + r, weight row lane % 16 of the tile
+        // ---- the waves' sums meet in LDS, in the rings (free by now): records of [tile][m][n] ----
+        // element r of a lane's accumulator: token 16 mt + 4 (lane / 16) + r, weight row lane % 16 of the tile.
+        // A record that fits a wave's own ring lies there, one a wave; larger ones (NT MT > 16) are four, and the
+        // waves 4 .. 7 hand theirs to the waves 0 .. 3 first.
+        constexpr bool HAND = NT * MT * 256 > RG_RING_FLOATS;
+        constexpr int SUMS = HAND ? 4 : RG_WAVES, REC = HAND ? NT * MT * 256 : RG_RING_FLOATS;
+        static_assert(SUMS * REC <= RG_WAVES * RG_RING_FLOATS, "the records fit into the rings");
         float* red = reinterpret_cast<float*>(smem);
         {
-            float* mine = red + wave * RG_RING_FLOATS;
+            float* mine = red + (HAND ? wave & 3 : wave) * REC;
             const int n = lane & 15, mg = lane >> 4;
+            auto put = [&](bool add) {
 #pragma unroll
-            for (int tt = 0; tt < NT; tt++)
-                if (tt < nt) {
+                for (int tt = 0; tt < NT; tt++)
+                    if (tt < nt) {
 #pragma unroll
-                    for (int r = 0; r < 4; r++) mine[(tt * 16 + 4 * mg + r) * 16 + n] = acc[tt][r];
-                }
+                        for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+                            for (int r = 0; r < 4; r++) {
+                                float* at = mine + ((tt * MR + 16 * mt + 4 * mg + r) * 16 + n);
+                                *at = add ? *at + acc[tt][mt][r] : acc[tt][mt][r];
+                            }
+                    }
+            };
+            if (HAND) {
+                __syncthreads();                                           // every wave is done with its ring
+                if (wave >= 4) put(false);
+                __syncthreads();
+                if (wave < 4) put(true);
+            } else {
+                put(false);
+            }
         }
         float* behind = reinterpret_cast<float*>(smem) + RG_WAVES * RG_RING_FLOATS;     // LDS behind the rings
         if (tg0 == 0 && MODE != HFA_ROWS_RESID) {
-            // r[m] from the shares: 32 slices per row, added in a fixed order
+            // r[m] from the shares: SL slices per row, added in a fixed order
             float ssq_part = 0.f;
             if (p.ssq_in) {
 #pragma unroll
-                for (int i = 0; i < 8; i++) ssq_part += (tid >> 4) + 32 * i < p.parts_in ? early[i] : 0.f;
-                for (int q = (tid >> 4) + 256; q < p.parts_in; q += 32) ssq_part += p.ssq_in[q * 16 + (tid & 15)];
+                for (int i = 0; i < EARLY; i++) ssq_part += tid / MR + SL * i < p.parts_in ? early[i] : 0.f;
+                for (int q = tid / MR + SL * EARLY; q < p.parts_in; q += SL) ssq_part += p.ssq_in[q * MR + (tid % MR)];
             }
             behind[tid] = ssq_part;
             __syncthreads();
-            if (tid < 16) {
+            if (tid < MR) {
                 float s = 0.f;
-                for (int q = 0; q < 32; q++) s += behind[q * 16 + tid];
+                for (int q = 0; q < SL; q++) s += behind[q * MR + tid];
                 r_s[tid] = p.ssq_in ? rsqrtf(s * p.inv_width + p.eps) : 1.0f;
             }
         }
@@ -275,12 +314,12 @@ __global__ __launch_bounds__(RG_WAVES * WAVE) void gemm_rows_kernel(const RowGem
         auto total = [&](int tt, int m, int n) {
             float s = 0.f;
 #pragma unroll
-            for (int w = 0; w < RG_WAVES; w++) s += red[w * RG_RING_FLOATS + (tt * 16 + m) * 16 + n];
+            for (int w = 0; w < SUMS; w++) s += red[w * REC + (tt * MR + m) * 16 + n];
             return s;
         };
         if (MODE == HFA_ROWS_OUT) {
-            for (int i = tid; i < nt * 256; i += RG_WAVES * WAVE) {
-                const int tt = i >> 8, m = (i >> 4) & 15, n = i & 15, col = own0 + 16 * (tg0 + tt) + n;
+            for (int i = tid; i < nt * 16 * MR; i += RG_WAVES * WAVE) {
+                const int tt = i / (16 * MR), m = (i >> 4) % MR, n = i & 15, col = own0 + 16 * (tg0 + tt) + n;
                 if (m < p.T && col < own1) {
                     const float v = r_s[m] * total(tt, m, n) + (p.bias ? p.bias[col] : 0.f);
                     if (p.out_bf16) reinterpret_cast<uint16_t*>(p.out)[(size_t)m * p.ldo + col] = rg_bf16(v);
@@ -288,17 +327,17 @@ __global__ __launch_bounds__(RG_WAVES * WAVE) void gemm_rows_kernel(const RowGem
                 }
             }
         } else if (MODE == HFA_ROWS_SWIGLU) {
-            for (int i = tid; i < (nt / 2) * 256; i += RG_WAVES * WAVE) {
-                const int j = i >> 8, m = (i >> 4) & 15, n = i & 15, f = own0 + 16 * (tg0 / 2 + j) + n;
+            for (int i = tid; i < (nt / 2) * 16 * MR; i += RG_WAVES * WAVE) {
+                const int j = i / (16 * MR), m = (i >> 4) % MR, n = i & 15, f = own0 + 16 * (tg0 / 2 + j) + n;
                 if (m < p.T && f < own1) {
                     const float gt = r_s[m] * total(2 * j, m, n), up = r_s[m] * total(2 * j + 1, m, n);
                     p.act[(size_t)m * p.ldact + f] = rg_bf16(gt / (1.0f + __expf(-gt)) * up);        // src/mathx.c:34
                 }
             }
         } else {
-            // the new residual values also go to LDS, for the sums of squares: [16][NT * 16]
-            for (int i = tid; i < nt * 256; i += RG_WAVES * WAVE) {
-                const int tt = i >> 8, m = (i >> 4) & 15, n = i & 15, col = own0 + 16 * (tg0 + tt) + n;
+            // the new residual values also go to LDS, for the sums of squares: [MR][NT * 16]
+            for (int i = tid; i < nt * 16 * MR; i += RG_WAVES * WAVE) {
+                const int tt = i / (16 * MR), m = (i >> 4) % MR, n = i & 15, col = own0 + 16 * (tg0 + tt) + n;
                 float v = 0.f;
                 if (m < p.T && col < own1) {
                     const float was = (tg0 == 0 && i == tid) ? early[0] : p.x[(size_t)m * p.ldx + col];
@@ -309,7 +348,7 @@ __global__ __launch_bounds__(RG_WAVES * WAVE) void gemm_rows_kernel(const RowGem
                 behind[m * (NT * 16) + tt * 16 + n] = v;
             }
             __syncthreads();
-            if (tid < 16) {
+            if (tid < MR) {
                 float s = 0.f;
                 for (int j = 0; j < nt * 16; j++) { const float v = behind[tid * (NT * 16) + j]; s += v * v; }
                 ssq_run += s;
@@ -317,7 +356,7 @@ __global__ __launch_bounds__(RG_WAVES * WAVE) void gemm_rows_kernel(const RowGem
         }
         __syncthreads();                                                   // the rings are requested again for the next group
     }
-    if (MODE == HFA_ROWS_RESID && tid < 16) p.ssq_out[b * 16 + tid] = ssq_run;
+    if (MODE == HFA_ROWS_RESID && tid < MR) p.ssq_out[b * MR + tid] = ssq_run;
 }
 
 static int rows_cu_count() {
@@ -330,13 +369,13 @@ static int rows_cu_count() {
     return n;
 }
 
-template <int NT, int MODE>
-static int rows_launch(const RowGemm& p, hipStream_t stream) {
+template <int NT, int MODE, int MT>
+static int rows_launch_mt(const RowGemm& p, hipStream_t stream) {
     constexpr int AD = NT == 1 ? RG_R : (RG_R + NT - 1) / NT + 1;         // sets that may be live at once (see the kernel)
-    constexpr int BEHIND = MODE == HFA_ROWS_RESID ? 16 * NT * 16 * 4 : 2048;
+    constexpr int BEHIND = MODE == HFA_ROWS_RESID ? 16 * MT * NT * 16 * 4 : 2048;
     constexpr int SMEM = RG_WAVES * RG_R * RG_UNIT * 2 + (BEHIND > 2048 ? BEHIND : 2048);
     static_assert(SMEM <= 160 * 1024 - 64, "rings and records must fit into a CU's LDS");
-    auto kernel = gemm_rows_kernel<NT, AD, MODE>;
+    auto kernel = gemm_rows_kernel<NT, AD, MODE, MT>;
     static bool configured = false;
     if (!configured) {
         hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM);
@@ -351,6 +390,14 @@ static int rows_launch(const RowGemm& p, hipStream_t stream) {
     return 0;
 }
 
+template <int NT, int MODE>
+static int rows_launch(const RowGemm& p, hipStream_t stream) {
+    if constexpr (NT <= 10) {
+        if (p.T > 16) return rows_launch_mt<NT, MODE, 2>(p, stream);
+    }
+    return rows_launch_mt<NT, MODE, 1>(p, stream);
+}
+
 template <int MODE>
 static int rows_dispatch(const RowGemm& p, hipStream_t stream) {
     const int G = rows_cu_count();
@@ -359,9 +406,10 @@ static int rows_dispatch(const RowGemm& p, hipStream_t stream) {
     // tiles a wave takes at a time: few repeated tiles and few passes over K (a pass costs about what two tiles
     // cost: its own ramp, and the waves' sums meeting at its end), the larger one of equals
     const int opts[] = {1, 2, 4, 6, 8, 10, 12};
-    int best = 12, best_cost = 1 << 30;
+    int best = 10, best_cost = 1 << 30;
     for (int o : opts) {
         if (MODE == HFA_ROWS_SWIGLU && (o & 1)) continue;
+        if (p.T > 16 && o > 10) continue;                    // (with two tiles of rows, 12 tiles of weights are more than the registers hold)
         const int cost = (nt + o - 1) / o * (o + 2);
         if (cost < best_cost || (cost == best_cost && o > best)) { best = o; best_cost = cost; }
     }
@@ -379,10 +427,10 @@ static int rows_dispatch(const RowGemm& p, hipStream_t stream) {
 extern "C" int hfa_gemm_rows_parts(void) { return rows_cu_count(); }
 
 extern "C" int hfa_gemm_rows_supports(int mode, int M, int N, int K, int lda, int ldw) {
-    if (M < 1 || M > 16 || N < 1 || K < 128 || K % 128 != 0 || lda % 8 != 0 || ldw % 8 != 0) return 0;
+    if (M < 1 || M > 32 || N < 1 || K < 128 || K % 128 != 0 || lda % 8 != 0 || ldw % 8 != 0) return 0;
     if (mode == HFA_ROWS_SWIGLU && N % 32 != 0) return 0;
     const long long rows = mode == HFA_ROWS_SWIGLU ? 2LL * N : N;
-    if (rows * ldw * 2 >= (1LL << 32) || 16LL * lda * 2 >= (1LL << 32)) return 0;       // 32-bit byte offsets
+    if (rows * ldw * 2 >= (1LL << 32) || 32LL * lda * 2 >= (1LL << 32)) return 0;       // 32-bit byte offsets
     return 1;
 }
 
@@ -392,7 +440,7 @@ extern "C" int hfa_gemm_rows(int mode, const void* a, int lda, const void* w, in
                              void* xg, int ldxg, void* act, int ldact, hipStream_t stream) {
     HFA_REQUIRE(mode == HFA_ROWS_OUT || mode == HFA_ROWS_RESID || mode == HFA_ROWS_SWIGLU, "gemm_rows: unknown mode %d", mode);
     HFA_REQUIRE(hfa_gemm_rows_supports(mode, M, N, K, lda, ldw),
-                "gemm_rows: needs 1 to 16 rows, K a multiple of 128 and row strides that are multiples of 8 (M=%d N=%d K=%d lda=%d ldw=%d)",
+                "gemm_rows: needs 1 to 32 rows, K a multiple of 128 and row strides that are multiples of 8 (M=%d N=%d K=%d lda=%d ldw=%d)",
                 M, N, K, lda, ldw);
     HFA_REQUIRE(a && w && lda >= K && ldw >= K && ((uintptr_t)a & 15) == 0 && ((uintptr_t)w & 15) == 0,
                 "gemm_rows: operands must be 16-byte aligned with rows of at least K elements");

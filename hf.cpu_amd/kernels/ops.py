@@ -267,7 +267,7 @@ class Ops:
                 and out.dtype == torch.bfloat16:
             self._lazy = None
             self._source_changes(x, keep=out)
-            ssq = self.scratch(f"ssq@{out.data_ptr()}", (self.rows_parts * 16,), torch.float32)
+            ssq = self.scratch(f"ssq@{out.data_ptr()}", (self.rows_parts * 32,), torch.float32)
             self._rows_resid(z, weight, out, ssq)
             self._scaled[out.data_ptr()] = Scaled(out, x, weight, float(eps), ssq)
             return
@@ -341,7 +341,7 @@ class Ops:
 
     def _rows_resid_now(self, z, g, xg, ssq):
         if ssq is None:
-            ssq = self.scratch("ssq@none", (self.rows_parts * 16,), torch.float32)
+            ssq = self.scratch("ssq@none", (self.rows_parts * 32,), torch.float32)
         self._rows_call(1, z.a, z.w, z.w.shape[0], z.bias, x=z.x, ssq_out=ssq, g=g, xg=xg)
 
     def _whole(self, t):

@@ -503,24 +503,26 @@ def test_real_layer_sizes_at_the_batch_sizes_with_kernels_of_their_own(gpu, tmp_
     """The 7B-shaped layer in bf16 at the step sizes for which the matrix products change kernels:
     a prompt of 2,048 tokens in one step (tiles of 256 rows fed by direct loads into LDS), and 40
     requests decoded together (33 to 64 rows: one stream of units cut evenly over the CUs, the
-    norm and the rotary kernel adding up its planes), against the plain implementation on
-    weights rounded to bf16."""
+    norm and the rotary kernel adding up its planes), then 21 decoded together (17 to 32 rows: the product that
+    finishes its outputs with two tiles of rows, norms and rotation inside products and attention), against the
+    plain implementation on weights rounded to bf16."""
     import hf_cpu_amd
     cfg = dict(architectures=["Qwen2ForCausalLM"], num_hidden_layers=1, hidden_size=3584, num_attention_heads=28,
                num_key_value_heads=4, head_dim=128, intermediate_size=18944, vocab_size=4096, rope_theta=1e6,
                rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=4096)
     d = helpers.make_model_dir(str(tmp_path / "m"), cfg, seed=4)
-    reqs = helpers.random_requests(cfg, [2048] + [6 + i % 5 for i in range(40)], seed=2)
-    big, many = "r0", [f"r{i}" for i in range(1, 41)]
+    reqs = helpers.random_requests(cfg, [2048] + [6 + i % 5 for i in range(40)] + [5 + i % 7 for i in range(21)], seed=2)
+    big, many, some = "r0", [f"r{i}" for i in range(1, 41)], [f"r{i}" for i in range(41, 62)]
     steps = [helpers._step(0, [(big, reqs[big], [0, 1, 1000, 2046, 2047])], [big])]
-    steps.append(helpers._step(1, [(r, reqs[r][:-4], []) for r in many]))
-    for j in range(4, 0, -1):
-        steps.append(helpers._step(len(steps), [(r, [reqs[r][-j]], [0]) for r in many], many if j == 1 else []))
+    for group in (many, some):
+        steps.append(helpers._step(len(steps), [(r, reqs[r][:-4], []) for r in group]))
+        for j in range(4, 0, -1):
+            steps.append(helpers._step(len(steps), [(r, [reqs[r][-j]], [0]) for r in group], group if j == 1 else []))
     want = helpers.plain_logits(d, reqs, round_weights_bf16=True)
     engine = hf_cpu_amd.load_engine(d, dtype="bfloat16", page_tokens=16, max_tokens=2048 + 40 * 64, max_seqs=40)
     got = helpers.run_trace_in_engine(engine, steps)
     worst = helpers.compare(got, want, 2e-2, "7B layer, large steps")
-    print(f"7B-sized layer, 2048-token prompt and 40 decoded together: worst relative difference {worst:.2e}")
+    print(f"7B-sized layer, 2048-token prompt, 40 and 21 decoded together: worst relative difference {worst:.2e}")
     assert not engine.manager.held
     # The same steps again: every kernel adds in an order fixed by the sizes alone, so the logits
     # come out bit for bit the same (a race between waves or blocks would show here).

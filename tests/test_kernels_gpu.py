@@ -237,9 +237,12 @@ def _deferred_products(ops16, M, K, E):
 
 
 @pytest.mark.parametrize("M,K,E,N", [(1, 256, 128, 1000), (5, 4096, 896, 1152), (8, 18944, 3584, 4608), (16, 3584, 3584, 4100),
-                                     (11, 640, 2176, 77), (16, 1536, 8960, 333)])
+                                     (11, 640, 2176, 77), (16, 1536, 8960, 333),
+                                     (17, 3584, 3584, 4608), (32, 18944, 3584, 37888), (24, 896, 896, 1152), (29, 256, 8960, 77),
+                                     (32, 1024, 40000, 2100)])
 def test_products_of_few_rows_that_finish_their_outputs(ops16, M, K, E, N):
-    """Up to 16 rows: a product into the residual stream waits for the norm that follows; one kernel then does product,
+    """Up to 32 rows (from 17 on the kernel holds two tiles of 16 rows, and the shares of the sums of squares are
+    laid out for 32): a product into the residual stream waits for the norm that follows; one kernel then does product,
     residual sum, the sums of squares and x * weight, and the product that reads the norm's output scales its sums
     (``Ops.rmsnorm(..., lazy=True)``). Against the same in float64: the residual stream, the product behind the
     norm (into fp32, into bf16, and as the 32-bit plane that the rotation of queries and keys takes), gate and up

@@ -178,7 +178,8 @@ def main():
                     help="run one phase only and print a short line (for profiling a phase by itself)")
     ap.add_argument("--context", type=int, default=PROMPT,
                     help="with --only decode: tokens every sequence holds before the timed steps (prefilled in portions "
-                         "of 2,048); the default run's is 2,048")
+                         "of 2,048); with --only prefill: the length of the prompt, computed in portions of 2,048; "
+                         "the default run's is 2,048")
     ap.add_argument("--shape", choices=["7b", "0.5b", "32b"], default="7b",
                     help="with --only: the layer sizes of the step (the default measurement's are the 7B shape's)")
     ap.add_argument("--no-peaks", action="store_true", help="skip the probes of the device's own peaks")
@@ -195,8 +196,8 @@ def main():
         return 2
     if args.workload != "7b":
         return serve_workload(args.workload, args.dtype, args.temp, args.budget)
-    if args.context != PROMPT and args.only != "decode":
-        print("bench.py: --context goes with --only decode (the default measurement has 2,048-token prompts)")
+    if args.context != PROMPT and args.only is None:
+        print("bench.py: --context goes with --only decode | prefill (the default measurement has 2,048-token prompts)")
         return 2
     if args.shape != "7b" and args.only is None:
         print("bench.py: --shape goes with --only prefill | decode (the default measurement is of the 7B shape)")
@@ -260,6 +261,34 @@ def main():
             eng.step([("prefill", prompt(), [PROMPT - 1])])
             eng.release("prefill")
         kernels.update(kernel_fractions(eng, "prefill", one_prefill, 2, shape, elem, 1, PROMPT, peaks, short))
+    if args.only == "prefill" and args.context > PROMPT:
+        # A long prompt in portions of 2,048 tokens, each a step of its own: what every portion costs (later
+        # ones attend over all that lies before them), and the whole.
+        whole = []
+        for rep in range(2):
+            per = []
+            for at in range(0, args.context, PROMPT):
+                n = min(PROMPT, args.context - at)
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                logits = eng.step([("long", prompt()[:n], [n - 1] if at + n == args.context else [])])
+                if at + n == args.context:
+                    ops.argmax(logits).cpu()
+                torch.cuda.synchronize()
+                per.append(time.perf_counter() - t0)
+            eng.release("long")
+            whole.append(per)
+        per = whole[-1]
+        total = sum(per)
+        # flops: every portion's products, and attention over the causal part of the whole prompt
+        L, H, D = shape["num_hidden_layers"], shape["num_attention_heads"], shape["head_dim"]
+        per_layer, head = matmul_params(shape)
+        flops = 2.0 * args.context * L * per_layer + L * 4.0 * D * H * args.context * (args.context + 1) / 2 + 2.0 * head
+        print(json.dumps({"phase": "prefill", "shape": args.shape, "tokens": args.context, "portion": PROMPT,
+                          "ms": round(total * 1e3, 2), "tok_per_s": round(args.context / total, 1),
+                          "frac": round(flops / total / FLOP_PEAK[short], 4),
+                          "first_portion_ms": round(per[0] * 1e3, 2), "last_portion_ms": round(per[-1] * 1e3, 2)}))
+        return 0
     if args.only == "prefill":
         print(json.dumps({"phase": "prefill", "shape": args.shape, "tokens": PROMPT, "ms": round(pre_s * 1e3, 3)}))
         return 0

@@ -19,8 +19,15 @@ CONFIG_B = dict(architectures=["Qwen2ForCausalLM"], model_type="qwen2", num_hidd
                 vocab_size=1000, rope_theta=1000000.0, rms_norm_eps=1e-5, tie_word_embeddings=False,
                 use_sliding_window=True, sliding_window=32, max_window_layers=1,
                 max_position_embeddings=256, hidden_act="silu")
-PAGE = {"A": 16, "B": 8}
-CONFIGS = {"A": CONFIG_A, "B": CONFIG_B}
+# Sizes that the kernels of the serving path take (widths that are multiples of 128, a head size of 64): the tiny
+# configurations above run the plain kernels for most of a step.
+CONFIG_C = dict(architectures=["Qwen2ForCausalLM"], model_type="qwen2", num_hidden_layers=2, hidden_size=256,
+                num_attention_heads=4, num_key_value_heads=2, head_dim=64, intermediate_size=384,
+                vocab_size=777, rope_theta=50000.0, rms_norm_eps=1e-6, tie_word_embeddings=False,
+                use_sliding_window=True, sliding_window=48, max_window_layers=1,
+                max_position_embeddings=256, hidden_act="silu")
+PAGE = {"A": 16, "B": 8, "C": 16}
+CONFIGS = {"A": CONFIG_A, "B": CONFIG_B, "C": CONFIG_C}
 
 
 def bf16_round(a):

@@ -12,10 +12,10 @@ pytestmark = pytest.mark.gpu
 # bf16: activations and cache rounded to 8 bits of mantissa at every part (measured: 0.8e-2).
 TOL = {"float32": 5e-6, "bfloat16": 2e-2}
 KERNELS_AGREE = 2e-2     # bf16: another order of summation flips roundings of activations, which spread like any rounding
-LENGTHS = {"A": [7, 19, 33, 70, 101], "B": [1, 40, 77, 100, 130]}
+LENGTHS = {"A": [7, 19, 33, 70, 101], "B": [1, 40, 77, 100, 130], "C": [3, 48, 49, 120, 200]}
 
 
-@pytest.fixture(scope="module", params=["A", "B"])
+@pytest.fixture(scope="module", params=["A", "B", "C"])
 def tiny(request, tmp_path_factory):
     name = request.param
     cfg = helpers.CONFIGS[name]

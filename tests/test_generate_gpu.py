@@ -469,6 +469,47 @@ def test_serving_at_random_with_forks_a_window_and_a_tight_cache(gpu, models, se
             assert r.generated == alone, f"request {r.req_id}: preempted {r.preemptions} times"
 
 
+def test_serving_through_the_kernels_of_the_decode_path(gpu, tmp_path):
+    """A configuration whose widths the serving kernels take (multiples of 128, head size 64, one windowed layer)
+    in bf16 through the scheduler: 28 requests with prompts of 1 to 100 tokens and 10 to 40 new tokens, greedy, a
+    token budget of 64 and a cache that runs out. Decode steps of 1 to 28 requests then go through the products that
+    finish their outputs (one and two tiles of rows), the norms inside them, the attention kernel that rotates and
+    stores, steps filled up to a multiple of 8 and graphs, while requests are preempted and come back. Checked
+    without an assumption about bits: every generated token is, by the plain implementation run over the request's
+    whole sequence on weights rounded to bf16, the best token or within the engine's tolerance of it."""
+    import hf_cpu_amd.session as S
+    cfg = helpers.CONFIG_C
+    d = helpers.make_model_dir(str(tmp_path / "c"), cfg, seed=33)
+    rng = np.random.default_rng(12)
+    prompts = [[int(t) for t in rng.integers(0, cfg["vocab_size"], int(rng.integers(1, 101)))] for _ in range(28)]
+    news = [int(rng.integers(10, 41)) for _ in prompts]
+    s = S.Session(d, dtype="bfloat16", ctx_max=160, batch=64, page_size=16, max_seqs=28, kv_tokens=28 * 52)
+    from hf_cpu_amd.engine.scheduler import Request
+    from hf_cpu_amd.sampling import SamplerParams
+    sched = s.scheduler()
+    reqs = [Request(i, list(p), SamplerParams(0.0, 40, 0.95, 0.05), n, i) for i, (p, n) in enumerate(zip(prompts, news))]
+    for r in reqs:
+        sched.submit(r)
+    sched.run()
+    s.engine.manager.check()
+    assert not s.engine.manager.held
+    assert s.engine.graph_replays > 0 and any(16 < key[0] <= 32 for key in s.engine._graph_seen)
+    assert sum(r.preemptions for r in reqs) > 0, "the cache was meant to run out"
+    pcfg, w = plain.read_model(d)
+    w = {k: (helpers.bf16_round(v).astype(np.float64) if v.ndim == 2 else v) for k, v in w.items()}
+    worst = 0.0
+    for r, p, n in zip(reqs, prompts, news):
+        assert r.error is None and r.stop == "length" and len(r.generated) == n, (r.req_id, r.error, r.stop)
+        logits = plain.forward(pcfg, w, p + r.generated)
+        scale = float(np.max(np.abs(logits)))
+        for j, tok in enumerate(r.generated):
+            row = logits[len(p) - 1 + j]
+            gap = float(row.max() - row[tok]) / scale
+            worst = max(worst, gap)
+            assert gap <= 2e-2, f"request {r.req_id} token {j}: the plain implementation's best is {gap:.3e} of the largest logit above it"
+    print(f"serving on the decode path's kernels: a generated token is at most {worst:.2e} of the largest logit below the plain best")
+
+
 def test_real_layer_sizes_in_both_precisions(gpu, tmp_path):
     """One layer with the sizes of the 7B shape (hidden 3584, 28 query heads on 4 key/value heads of
     128, feed-forward 18944; the vocabulary cut to 4096 to keep the plain implementation quick):

@@ -38,16 +38,17 @@ int hfa_gemm(const void* a, int a_dtype, int lda, const void* w, int w_dtype, in
 int hfa_gemm_finish(const void* partial, int splits, const float* bias, void* out, int out_dtype, int ldo,
                     int accumulate, int epilogue, int M, int N, hipStream_t stream);
 
-// The product for up to 16 rows in which every block owns a range of outputs and finishes them itself (bf16
+// The product for up to 32 rows in which every block owns a range of outputs and finishes them itself (bf16
 // operands, K a multiple of 128; see gemm_rows.hip), with what follows a product in a decode step in its last lines:
 //   HFA_ROWS_OUT     out[m, n] = r[m] * sum + bias[n], fp32 or bf16 (out_dtype)
 //   HFA_ROWS_RESID   x[m, n] += sum + bias[n] (fp32, in place); ssq_out[b][m] = block b's share of sum_n x[m, n]^2
-//                    ([hfa_gemm_rows_parts()][16] floats); xg[m, n] = bf16(x[m, n] * g[n]) if xg is given
+//                    ([hfa_gemm_rows_parts()][16] floats, [..][32] from 17 rows up: give room for 32); xg[m, n] = bf16(x[m, n] * g[n]) if xg is given
 //   HFA_ROWS_SWIGLU  act[m, f] = bf16(silu(r[m] * sum_gate) * (r[m] * sum_up)), N features, w's 2 N rows in blocks of
 //                    32 gate rows, 32 up rows (src/model.c:537)
 // r[m] = rsqrt(sum over the parts_in shares ssq_in[.][m] * inv_width + eps), or 1 without ssq_in: the RMS norm of the
 // tensor whose product with the norm's weight is `a` (src/mathx.c:65-75), applied to the sums instead of the operand.
-// hfa_gemm_rows_supports says whether a shape is taken (1 to 16 rows, K a multiple of 128, strides multiples of 8).
+// hfa_gemm_rows_supports says whether a shape is taken (1 to 32 rows, K a multiple of 128, strides multiples of 8).
+// ssq_in has the layout that a HFA_ROWS_RESID product of the same number of rows left.
 #define HFA_ROWS_OUT 0
 #define HFA_ROWS_RESID 1
 #define HFA_ROWS_SWIGLU 2

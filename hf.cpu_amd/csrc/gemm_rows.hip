@@ -1,4 +1,4 @@
-// bf16 matrix product for up to 16 rows (decode) in which every block owns a range of outputs and finishes
+// bf16 matrix product for up to 32 rows (decode) in which every block owns a range of outputs and finishes
 // them itself: out[m, n] = sum_k a[m, k] * w[n, k] over the whole of K inside one block, so no partial sums
 // leave the kernel and what usually follows a product in a decode step happens in its last lines:
 //
@@ -18,7 +18,7 @@
 // memory into its own ring in LDS by direct loads (global_load_lds_dwordx4: 64 lanes x 16 bytes = 8 rows of 128
 // bytes a request, rows swizzled so that the fragment reads are conflict-free), R units ahead, with no barrier
 // and no traffic between the waves while they stream. The activations of a unit of K (16 rows x 128 columns,
-// rows past the last one repeated) go from L2 straight into registers, requested together with the first tile of
+// rows past the last one repeated; from 17 rows up two such tiles, MT = 2) go from L2 straight into registers, requested together with the first tile of
 // that unit of K, so the order of all requests of a wave is fixed by the sizes alone and every wait names a count
 // that is known when the kernel is compiled. v_mfma_f32_16x16x32_bf16: tokens are the rows of the product, the
 // weights' rows its columns. At the end the waves' sums meet in LDS (in the rings, free by then) and are added in

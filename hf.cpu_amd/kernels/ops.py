@@ -466,6 +466,7 @@ class Ops:
                 and pend.out.data_ptr() == qkv.data_ptr() and pend.out.shape == qkv.shape and qkv.shape[1] == row_width \
                 and qkv.dtype == torch.bfloat16 and slot_map is not None and n_kv_heads and v_head_dim == head_dim \
                 and qkv.is_contiguous() and getattr(cache, "k", None) is not None and cache.k.dtype == torch.bfloat16 \
+                and cache.k.numel() < 1 << 32 and cache.k.shape[0] < 1 << 24 \
                 and self.lib.hfa_decode_attention_supports(n_heads, n_kv_heads, head_dim, rot_dim, cache.page_tokens,
                                                            cache.k.shape[1], row_width, n_heads * head_dim):
             self._lazy_rope = LazyRope((qkv, positions, inv_freq, rot_dim, n_heads, n_kv_heads, head_dim, cache, slot_map,

@@ -201,9 +201,12 @@ class Ops:
 
     def call(self, entry_point, *args, what=None):
         """Launches an entry point of an extension library (``kernels.lib.load_extension``) on the step's
-        stream: ``args`` are its arguments but the last, the stream. A deferred product is added up first,
+        stream: ``args`` are its arguments but the last, the stream. What was deferred is done first,
         since the kernel may read any tensor. Raises EngineError unless it returns 0."""
         self.settle()
+        for sc in list(self._scaled.values()):               # and a norm's output that was left undivided is made whole
+            if not sc.source_changed:
+                self._whole(sc.out)
         rc = entry_point(*args, self._stream())
         if rc != 0:
             raise EngineError(EINVAL if rc == 1 else ENOTSUP,
@@ -510,6 +513,7 @@ class Ops:
         added, for position encodings that enter the scores; the plain kernel then runs, as it does when
         value heads have a size of their own (``v_head_dim``; ``out`` then has that many columns a head)."""
         v_head_dim = head_dim if v_head_dim is None else int(v_head_dim)
+        self._scaled.pop(out.data_ptr(), None)               # whatever `out` held, it is no norm's lazy output any more
         lr = self._lazy_rope
         if lr is not None and lr.qkv.data_ptr() == q.data_ptr() and lr.cache is cache and slopes is None \
                 and step.max_q_len == 1 and step.n_seqs == q.shape[0] and not self.force_plain_attention \
@@ -583,6 +587,7 @@ class Ops:
 
     def swiglu(self, gate_up, out):
         self.settle()
+        self._scaled.pop(out.data_ptr(), None)
         T, F2 = gate_up.shape
         if not gate_up.is_contiguous() or not out.is_contiguous() or tuple(out.shape) != (T, F2 // 2) \
                 or out.dtype != gate_up.dtype or F2 % 2:

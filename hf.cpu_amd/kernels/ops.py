@@ -148,6 +148,7 @@ class Ops:
         self._scaled = {}                    # data_ptr of a norm's output -> Scaled
         self.rows_parts = int(self.lib.hfa_gemm_rows_parts())
         self.fuse_rows = True                # tests switch it off to compare with the chain of separate kernels
+        self.rows_always = False             # tests: every shape that the kernel of gemm_rows.hip takes goes through it
         self._splits_out = ctypes.c_int(0)
         self._sections = None                # while timing: (name, start event, end event, enclosing section) of every section left
         self._section_stack = []
@@ -314,6 +315,11 @@ class Ops:
                 mode, M, N, K, _rows(a, "gemm a"), _rows(w, "gemm w")):
             return None
         if accumulate:
+            # Every block of that kernel reads all the activations, and a block of a narrow product owns few weight
+            # rows to set against them: from 17 rows up a long K (the down projection) is quicker through the kernels
+            # that cut K over the blocks, with the norm as a kernel of its own (7B shape, 32 rows: 58 against 50 us).
+            if M > 16 and M * K > 128 << 10 and not self.rows_always:
+                return None
             return mode if out.dtype == torch.float32 else None
         if swiglu:
             return mode if out.dtype == torch.bfloat16 and bias is None else None

@@ -991,11 +991,12 @@ int attn_mfma_launch(const AttnArgs& a) {
     // How many waves in all is a measured choice. Head size 128 (7B shape): 512; with 1,024 a step took 1.3 % longer
     // at 64 sequences and 4.5 % longer at 8 sequences of 16,384 tokens, with 256 more than that. Head size 64 (0.5B
     // shape), where a wave has half the work per key: 1,024; with 512 a step of 64 sequences took 4.5 % longer; but no
-    // chunk of fewer than 128 keys (with chunks of 64 keys a step of 8 sequences at 2,048 took 5 % longer, one of 16 2 %).
+    // chunk of fewer than 128 keys for either head size (with chunks of 64 keys a step of 8 sequences of the 0.5B shape at
+    // 2,048 took 5 % longer, one of 16 2 %; one of 2 sequences of the 7B shape 2 % longer).
     const int fill = a.head_dim > 64 ? 512 : 1024;
     if (waves < fill && span > 128 && a.workspace) {
         int want = (int)((fill + waves - 1) / waves);
-        const int most = a.head_dim > 64 ? (span + 63) / 64 : (span + 127) / 128;
+        const int most = (span + 127) / 128;
         if (want > most) want = most;
         chunk_keys = ((a.max_seq_len + want - 1) / want + KB - 1) / KB * KB;
         if (chunk_keys < 64) chunk_keys = 64;

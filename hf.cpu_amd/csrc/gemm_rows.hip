@@ -179,6 +179,15 @@ __global__ __launch_bounds__(RG_WAVES * WAVE) void gemm_rows_kernel(const RowGem
         const float* src = p.x + (size_t)(m < p.T ? m : 0) * p.ldx + (col < own1 ? col : own0 < own1 ? own1 - 1 : 0);
         asm volatile("global_load_dword %0, %1, off" : "=v"(early[0]) : "v"(src) : "memory");
     }
+    // ... and the bias and the norm's weight of this thread's first output column (MODE != SWIGLU: column
+    // own0 + 16 (tid / (16 MR)) + tid % 16, the one of element tid of the first group of tiles)
+    float early_b = 0.f, early_g = 0.f;
+    if (MODE != HFA_ROWS_SWIGLU) {
+        const int col = own0 + 16 * (tid / (16 * MR)) + (tid & 15);
+        const int at = col < own1 ? col : own0 < own1 ? own1 - 1 : 0;
+        if (p.bias) asm volatile("global_load_dword %0, %1, off" : "=v"(early_b) : "v"(p.bias + at) : "memory");
+        if (MODE == HFA_ROWS_RESID && p.xg) asm volatile("global_load_dword %0, %1, off" : "=v"(early_g) : "v"(p.g + at) : "memory");
+    }
     float ssq_run = 0.f;                                                    // RESID: thread m's sum over the groups of tiles
 
     for (int tg0 = 0; tg0 < nt_all; tg0 += NT) {
@@ -259,6 +268,7 @@ __global__ __launch_bounds__(RG_WAVES * WAVE) void gemm_rows_kernel(const RowGem
         if (tg0 == 0) {
 #pragma unroll
             for (int i = 0; i < EARLY; i++) asm volatile("" : "+v"(early[i]));     // what was asked for first has landed too
+            asm volatile("" : "+v"(early_b), "+v"(early_g));
         }
         // ---- the waves' sums meet in LDS, in the rings (free by now): records of [tile][m][n] ----
         // element r of a lane's accumulator: token 16 mt + 4 (lane / 16) + r, weight row lane % 16 of the tile.
@@ -321,7 +331,7 @@ __global__ __launch_bounds__(RG_WAVES * WAVE) void gemm_rows_kernel(const RowGem
             for (int i = tid; i < nt * 16 * MR; i += RG_WAVES * WAVE) {
                 const int tt = i / (16 * MR), m = (i >> 4) % MR, n = i & 15, col = own0 + 16 * (tg0 + tt) + n;
                 if (m < p.T && col < own1) {
-                    const float v = r_s[m] * total(tt, m, n) + (p.bias ? p.bias[col] : 0.f);
+                    const float v = r_s[m] * total(tt, m, n) + (!p.bias ? 0.f : (tg0 == 0 && i == tid) ? early_b : p.bias[col]);
                     if (p.out_bf16) reinterpret_cast<uint16_t*>(p.out)[(size_t)m * p.ldo + col] = rg_bf16(v);
                     else reinterpret_cast<float*>(p.out)[(size_t)m * p.ldo + col] = v;
                 }
@@ -341,9 +351,10 @@ __global__ __launch_bounds__(RG_WAVES * WAVE) void gemm_rows_kernel(const RowGem
                 float v = 0.f;
                 if (m < p.T && col < own1) {
                     const float was = (tg0 == 0 && i == tid) ? early[0] : p.x[(size_t)m * p.ldx + col];
-                    v = was + (total(tt, m, n) + (p.bias ? p.bias[col] : 0.f));
+                    const bool first = tg0 == 0 && i == tid;
+                    v = was + (total(tt, m, n) + (!p.bias ? 0.f : first ? early_b : p.bias[col]));
                     p.x[(size_t)m * p.ldx + col] = v;
-                    if (p.xg) p.xg[(size_t)m * p.ldxg + col] = rg_bf16(v * p.g[col]);
+                    if (p.xg) p.xg[(size_t)m * p.ldxg + col] = rg_bf16(v * (first ? early_g : p.g[col]));
                 }
                 behind[m * (NT * 16) + tt * 16 + n] = v;
             }

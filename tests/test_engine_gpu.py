@@ -476,3 +476,29 @@ def test_tokens_taken_from_the_device(gpu, tiny, dtype):
     with pytest.raises(EngineError):
         eng.step([("q0", [1], [0])], fed=(pool.long(), {0: 3}))
     eng.manager.check()
+
+
+@pytest.mark.parametrize("rows", [(1 << 24) - 32, (1 << 24) + 1024])    # (the storage keeps one page more than the pool hands out)
+def test_pages_at_the_far_end_of_a_cache_of_many_gigabytes(gpu, tmp_path, rows):
+    """A pool so large that a layer's keys are 2^32 elements: the matrix-core attention reaches the cache with 32-bit
+    element offsets and 24-bit row numbers, so just below that size it must still be right at the pool's last pages,
+    and from that size on the calls go to the plain kernels, which count in 64 bits. The pool's free stack is turned
+    over, so that the requests get the highest page ids; a mixed trace against the plain implementation."""
+    import torch
+    import hf_cpu_amd
+    cfg = dict(helpers.CONFIG_C, num_hidden_layers=1, num_key_value_heads=4, use_sliding_window=False)
+    d = helpers.make_model_dir(str(tmp_path / "m"), cfg, seed=5)
+    reqs = helpers.random_requests(cfg, [40, 70, 33], seed=8)
+    steps = helpers.trace_mixed(reqs, seed=2, max_live=3, decode_tail=6)
+    want = helpers.plain_logits(d, reqs, round_weights_bf16=True)
+    engine = hf_cpu_amd.load_engine(d, dtype="bfloat16", page_tokens=16, max_tokens=rows, max_seqs=3, max_context=128)
+    k = next(v for v in engine.storage.views if v is not None).k
+    assert k.shape[0] >= rows and (k.numel() >= 1 << 32) == (rows >= 1 << 24)
+    for pool in engine.manager.pools:
+        pool._free.reverse()                                # the highest page ids first
+    got = helpers.run_trace_in_engine(engine, steps)
+    worst = helpers.compare(got, want, 2e-2, f"a cache of {rows} rows")
+    print(f"a cache of {rows} rows of 256 keys, pages from the far end: worst relative difference {worst:.2e}")
+    engine.manager.check()
+    del engine, k
+    torch.cuda.empty_cache()

@@ -319,6 +319,29 @@ def _products_of_few_rows(ops16, M, K, E, N):
         ops16.fuse_rows = True
 
 
+def test_products_with_a_weight_matrix_beyond_four_gigabytes(ops16):
+    """300,000 rows of 8,192 bf16 weights are 4.9 GB: byte offsets from the matrix's start no longer fit 32 bits.
+    Every product kernel (1, 8, 24, 64, 128, 300 and 2,048 rows of activations) against the library's product on
+    slices of the columns, among them the last ones and those around the 2 GB and 4 GB marks."""
+    bf = torch.bfloat16
+    N, K = 300000, 8192
+    g = torch.Generator(device="cuda").manual_seed(1)
+    w = torch.empty((N, K), device="cuda", dtype=bf)
+    for i in range(0, N, 50000):
+        w[i:i + 50000] = (torch.randn((min(50000, N - i), K), device="cuda", generator=g) * 0.02).to(bf)
+    for M in (1, 8, 24, 64, 128, 300, 2048):
+        a = torch.randn((M, K), device="cuda", generator=g).to(bf)
+        out = torch.empty((M, N), device="cuda", dtype=torch.float32)
+        ops16.gemm(a, w, out)
+        ops16.settle()
+        for c0 in (0, 131072 - 64, 262144 - 100, N - 5000):
+            ref = a.float() @ w[c0:c0 + 5000].float().T
+            err = float((out[:, c0:c0 + 5000] - ref).abs().max() / ref.abs().max())
+            assert err < 2e-5, f"{M} rows, columns from {c0}: {err:.2e}"
+    del w, out
+    torch.cuda.empty_cache()
+
+
 def test_gemm_matches_library_product(ops32):
     """The kernel against the library's fp32 matrix product on the same operands."""
     torch.manual_seed(0)

@@ -502,3 +502,30 @@ def test_pages_at_the_far_end_of_a_cache_of_many_gigabytes(gpu, tmp_path, rows):
     engine.manager.check()
     del engine, k
     torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("dtype,tol", [("bfloat16", 2e-2), ("float32", 1e-5)])
+def test_a_step_of_seventy_thousand_tokens(gpu, tmp_path, dtype, tol):
+    """400 requests with prompts of 174 to 180 tokens in ONE step: more tokens and more requests than any grid
+    dimension of 65,535 holds, so every launcher's way of counting blocks is exercised (rows of a norm, tiles of a
+    product, tiles and requests of attention). Every 25th request and the last, first and last position, against
+    the plain implementation."""
+    import hf_cpu_amd
+    cfg = dict(helpers.CONFIG_C, num_hidden_layers=1)
+    d = helpers.make_model_dir(str(tmp_path / "m"), cfg, seed=9)
+    rng = np.random.default_rng(0)
+    reqs = {f"r{i}": [int(t) for t in rng.integers(0, cfg["vocab_size"], 180 - (i % 7))] for i in range(400)}
+    engine = hf_cpu_amd.load_engine(d, dtype=dtype, page_tokens=16, max_tokens=400 * 192, max_seqs=400, max_context=192)
+    logits = engine.step([(r, toks, [0, len(toks) - 1]) for r, toks in reqs.items()]).float().cpu().numpy()
+    assert sum(len(t) for t in reqs.values()) > 70000
+    pcfg, w = plain.read_model(d)
+    if dtype == "bfloat16":
+        w = {k: (helpers.bf16_round(v).astype(np.float64) if v.ndim == 2 else v) for k, v in w.items()}
+    for j, (r, toks) in enumerate(reqs.items()):
+        if j % 25 and j != len(reqs) - 1:
+            continue
+        want = plain.forward(pcfg, w, toks)
+        for jj, at in enumerate((0, len(toks) - 1)):
+            err = float(np.max(np.abs(logits[2 * j + jj] - want[at])) / np.max(np.abs(want)))
+            assert err < tol, f"request {r} position {at}: {err:.2e}"
+    engine.manager.check()

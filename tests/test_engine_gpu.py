@@ -3,6 +3,7 @@ import numpy as np
 import pytest
 
 import helpers
+import plain
 
 pytestmark = pytest.mark.gpu
 

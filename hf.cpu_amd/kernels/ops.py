@@ -15,6 +15,7 @@ computes with a library routine or on the CPU.
 """
 import contextlib
 import ctypes
+import sys
 from dataclasses import dataclass
 
 import torch
@@ -154,6 +155,7 @@ class Ops:
         self._section_stack = []
         self.force_plain_gemm = False        # tests set these to compare the matrix-core paths with the plain ones
         self.force_plain_attention = False
+        self._said_cache_too_large = False
 
     # ---- timing (the reference's hfc_prof_enable / hfc_prof_take, src/model.h:75-79) ----
     def section(self, name):
@@ -541,7 +543,13 @@ class Ops:
         _ints(step.positions, "positions", T)
         _ints(step.q_start, "q_start", step.n_seqs + 1)
         # the matrix-core kernels address the cache with 32-bit element offsets and 24-bit row numbers
-        plain = self.force_plain_attention or slopes is not None or cache.k.numel() >= 1 << 32 or cache.k.shape[0] >= 1 << 24
+        too_large = cache.k.numel() >= 1 << 32 or cache.k.shape[0] >= 1 << 24
+        plain = self.force_plain_attention or slopes is not None or too_large
+        if too_large and q.dtype == torch.bfloat16 and not self._said_cache_too_large:
+            self._said_cache_too_large = True        # right, but many times slower: say so once
+            print(f"[hf_cpu_amd] a layer's cache of {cache.k.shape[0]} rows x {cache.k.shape[1]} is beyond what the "
+                  "matrix-core attention addresses (2^24 rows, 2^32 elements): the plain attention kernels run; "
+                  "a smaller --kv-tokens brings the fast ones back", file=sys.stderr, flush=True)
 
         def call(first, n_tokens, q_start, n_seqs, max_q_len):
             self._check(self.lib.hfa_paged_attention(
